@@ -1,0 +1,242 @@
+"""Pins for each oracle kernel that do not come from the gradient fixture:
+library routines (torch CPU), closed forms, golden JSON, special values.
+A plausible mistake (dropped term, wrong sign/index, transposed operand)
+fails at least one of these."""
+import json
+import math
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import cpu
+from oracle import reference_step as rs
+
+RNG = np.random.default_rng(1234)
+
+
+def randn(*shape):
+    return RNG.standard_normal(shape).astype(np.float32)
+
+
+# ---- f16 storage ---------------------------------------------------------
+
+def test_f16_rounding_matches_ieee_rne():
+    x = np.concatenate([
+        randn(20000), randn(2000) * 1e-6, randn(2000) * 1e5,
+        np.array([0.0, -0.0, 1.0, -1.0, 65504.0, 65519.99, 65520.0, 1e9, -1e9, 6.1035156e-05,
+                  5.9604645e-08, 2.9802322e-08, 2.98023224e-08 * 1.0001, 1e-10, np.inf, -np.inf,
+                  1.0009765625, 1.00048828125, 1.00146484375], np.float32)])
+    bits = cpu.pack_f16(x)
+    with np.errstate(over="ignore"):
+        want = x.astype(np.float16).view(np.uint16)
+    np.testing.assert_array_equal(bits, want)
+    np.testing.assert_array_equal(cpu.unpack_f16(bits).view(np.uint32),
+                                  want.view(np.float16).astype(np.float32).view(np.uint32))
+    assert np.isnan(cpu.unpack_f16(cpu.pack_f16(np.array([np.nan], np.float32))))[0]
+
+
+def test_f16_every_bit_pattern_round_trips():
+    bits = np.arange(65536, dtype=np.uint16)
+    f = cpu.unpack_f16(bits)
+    want = bits.view(np.float16).astype(np.float32)
+    ok = ~np.isnan(want)
+    np.testing.assert_array_equal(f[ok].view(np.uint32), want[ok].view(np.uint32))
+    np.testing.assert_array_equal(cpu.pack_f16(f[ok]), bits[ok])
+
+
+def test_f16_packing_is_little_endian_low_half_first():
+    # tensor.rs:258-269: two values per 32-bit word, the first in the low half.
+    bits = cpu.pack_f16(np.array([1.0, -2.0], np.float32))
+    word = bits.view(np.uint32)[0]
+    assert word & 0xFFFF == 0x3C00 and word >> 16 == 0xC000
+
+
+# ---- matmul layouts ------------------------------------------------------
+
+@pytest.mark.parametrize("M,K,N", [(1, 1, 1), (5, 7, 3), (33, 17, 65), (64, 576, 40), (130, 64, 129)])
+def test_matmul_layouts_against_f64(M, K, N):
+    a, b = randn(M, K), randn(K, N)
+    want = a.astype(np.float64) @ b.astype(np.float64)
+    tol = dict(rtol=1e-4, atol=1e-3)  # gpu_kernels.rs:989-1084 uses 1e-3 + 1e-4*|want|
+    np.testing.assert_allclose(cpu.matmul(a, b), want, **tol)
+    np.testing.assert_allclose(cpu.matmul_bt(a, np.ascontiguousarray(b.T)), want, **tol)
+    np.testing.assert_allclose(cpu.matmul_at(np.ascontiguousarray(a.T), b), want, **tol)
+
+
+def test_phase0_linear_and_rmsnorm_json(golden_dir):
+    with open(os.path.join(golden_dir, "phase0_linear_rmsnorm.json")) as f:
+        j = json.load(f)
+    x = np.array(j["input"], np.float32)
+    w_hf = np.array(j["linear_weight_hf_layout"], np.float32)
+    want_lin = np.array(j["linear_output"], np.float32)
+    got = cpu.matmul(x.reshape(-1, x.shape[-1]), cpu.transpose(w_hf))
+    np.testing.assert_allclose(got.reshape(want_lin.shape), want_lin, rtol=1e-5, atol=1e-5)
+    w = np.array(j["rms_weight"], np.float32)
+    want_rms = np.array(j["rms_output"], np.float32)
+    got = cpu.rms_norm(x, w, j["meta"]["eps"])
+    np.testing.assert_allclose(got, want_rms, rtol=1e-5, atol=1e-5)
+
+
+# ---- RMSNorm -------------------------------------------------------------
+
+def test_rms_norm_backward_against_torch_autograd():
+    x, w, g = randn(37, 96), randn(96), randn(37, 96)
+    eps = 1e-5
+    xt = torch.tensor(x, dtype=torch.float64, requires_grad=True)
+    wt = torch.tensor(w, dtype=torch.float64, requires_grad=True)
+    y = xt * torch.rsqrt(xt.pow(2).mean(-1, keepdim=True) + eps) * wt
+    y.backward(torch.tensor(g, dtype=torch.float64))
+    np.testing.assert_allclose(cpu.rms_norm(x, w, eps), y.detach().numpy(), rtol=1e-5, atol=1e-5)
+    gx, gw = cpu.rms_norm_backward(x, w, g, eps)
+    np.testing.assert_allclose(gx, xt.grad.numpy(), rtol=1e-4, atol=1e-5)
+    np.testing.assert_allclose(gw, wt.grad.numpy(), rtol=1e-4, atol=1e-4)
+
+
+# ---- RoPE ----------------------------------------------------------------
+
+def test_rope_closed_form_and_inverse():
+    B, S, heads, D, theta, pos0 = 2, 9, 3, 8, 10000.0, 5
+    x = randn(B, S, heads * D)
+    got = cpu.rope(x, D, pos0, theta)
+    x4 = x.reshape(B, S, heads, D).astype(np.float64)
+    i = np.arange(D // 2)
+    ang = (pos0 + np.arange(S))[:, None] * theta ** (-2.0 * i / D)[None, :]
+    c, s = np.cos(ang)[None, :, None, :], np.sin(ang)[None, :, None, :]
+    x1, x2 = x4[..., :D // 2], x4[..., D // 2:]
+    want = np.concatenate([x1 * c - x2 * s, x1 * s + x2 * c], -1).reshape(B, S, heads * D)
+    np.testing.assert_allclose(got, want, rtol=1e-4, atol=1e-5)
+    back = cpu.rope(got, D, pos0, theta, inverse=True)
+    np.testing.assert_allclose(back, x, rtol=1e-5, atol=1e-5)
+    # position 0 is the identity (autograd/src/lib.rs:1899-1912)
+    one = randn(1, 1, D)
+    np.testing.assert_array_equal(cpu.rope(one, D, 0, theta), one)
+
+
+# ---- attention -----------------------------------------------------------
+
+def _sdpa(q, k, v, causal, offset=0):
+    B, Sq, H, D = q.shape
+    Hkv = k.shape[2]
+    qt = torch.tensor(q, dtype=torch.float64, requires_grad=True)
+    kt = torch.tensor(k, dtype=torch.float64, requires_grad=True)
+    vt = torch.tensor(v, dtype=torch.float64, requires_grad=True)
+    qh = qt.transpose(1, 2)
+    kh = kt.transpose(1, 2).repeat_interleave(H // Hkv, dim=1)
+    vh = vt.transpose(1, 2).repeat_interleave(H // Hkv, dim=1)
+    s = qh @ kh.transpose(-1, -2) / math.sqrt(D)
+    Sk = k.shape[1]
+    if causal:
+        vis = torch.arange(Sk)[None, :] <= (torch.arange(Sq)[:, None] + offset)
+        s = s.masked_fill(~vis, float("-inf"))
+    lse = torch.logsumexp(s, -1)
+    out = (s.softmax(-1) @ vh).transpose(1, 2)
+    return qt, kt, vt, out, lse
+
+
+@pytest.mark.parametrize("B,S,H,Hkv,D,causal", [(2, 13, 4, 2, 8, True), (1, 40, 6, 6, 16, True),
+                                               (2, 17, 3, 1, 64, False), (1, 1, 2, 1, 4, True)])
+def test_attention_forward_backward_against_torch(B, S, H, Hkv, D, causal):
+    q, k, v, do = randn(B, S, H, D), randn(B, S, Hkv, D), randn(B, S, Hkv, D), randn(B, S, H, D)
+    qt, kt, vt, out, lse = _sdpa(q, k, v, causal)
+    out.backward(torch.tensor(do, dtype=torch.float64))
+    got, got_lse = cpu.attention(q, k, v, causal=causal)
+    np.testing.assert_allclose(got, out.detach().numpy(), rtol=1e-4, atol=1e-5)
+    np.testing.assert_allclose(got_lse, lse.detach().numpy(), rtol=1e-5, atol=1e-5)
+    dq, dk, dv = cpu.attention_backward(q, k, v, got, do, causal=causal)
+    np.testing.assert_allclose(dq, qt.grad.numpy(), rtol=1e-3, atol=1e-5)
+    np.testing.assert_allclose(dk, kt.grad.numpy(), rtol=1e-3, atol=1e-5)
+    np.testing.assert_allclose(dv, vt.grad.numpy(), rtol=1e-3, atol=1e-5)
+
+
+def test_attention_is_causal_bit_exact():
+    # changing later tokens must not change earlier outputs at all
+    # (ferrotensor-graph/tests/model_correctness.rs:281-300)
+    q, k, v = randn(1, 12, 2, 8), randn(1, 12, 1, 8), randn(1, 12, 1, 8)
+    a, _ = cpu.attention(q, k, v)
+    k2, v2 = k.copy(), v.copy()
+    k2[:, 7:], v2[:, 7:] = randn(1, 5, 1, 8), randn(1, 5, 1, 8)
+    b, _ = cpu.attention(q, k2, v2)
+    np.testing.assert_array_equal(a[:, :7], b[:, :7])
+
+
+# ---- SiLU gate -----------------------------------------------------------
+
+def test_silu_gate_against_torch():
+    a, b, g = randn(1000) * 3, randn(1000), randn(1000)
+    at = torch.tensor(a, dtype=torch.float64, requires_grad=True)
+    bt = torch.tensor(b, dtype=torch.float64, requires_grad=True)
+    y = torch.nn.functional.silu(at) * bt
+    y.backward(torch.tensor(g, dtype=torch.float64))
+    np.testing.assert_allclose(cpu.silu_gate(a, b), y.detach().numpy(), rtol=1e-5, atol=1e-6)
+    ga, gb = cpu.silu_gate_backward(a, b, g)
+    np.testing.assert_allclose(ga, at.grad.numpy(), rtol=1e-4, atol=1e-6)
+    np.testing.assert_allclose(gb, bt.grad.numpy(), rtol=1e-4, atol=1e-6)
+
+
+# ---- masked CE -----------------------------------------------------------
+
+def test_masked_cross_entropy_against_torch():
+    rows, vocab = 12, 50
+    logits = randn(rows, vocab) * 4
+    targets = RNG.integers(0, vocab, rows).astype(np.uint32)
+    weights = RNG.random(rows).astype(np.float32)
+    targets[[2, 7]] = rs.MASKED_CE_SKIP
+    lt = torch.tensor(logits, dtype=torch.float64, requires_grad=True)
+    keep = targets != rs.MASKED_CE_SKIP
+    tt = torch.tensor(np.where(keep, targets, 0).astype(np.int64))
+    per = torch.nn.functional.cross_entropy(lt, tt, reduction="none")
+    wt = torch.tensor(np.where(keep, weights, 0.0), dtype=torch.float64)
+    (per * wt).sum().backward()
+    grad, row_loss = cpu.masked_cross_entropy(logits, targets, weights)
+    np.testing.assert_allclose(row_loss[keep], per.detach().numpy()[keep], rtol=1e-5, atol=1e-5)
+    assert (row_loss[~keep] == 0).all() and (grad[~keep] == 0).all()
+    np.testing.assert_allclose(grad, lt.grad.numpy(), rtol=1e-4, atol=1e-6)
+
+
+def test_targets_and_weights_are_exact():
+    # trainer/src/lib.rs:695-722: out-of-vocab or masked rows are skipped;
+    # weight = 1 / supervised tokens of the row's own sequence.
+    tg = np.array([[1, 2, 99, 4], [5, 6, 7, 8]], np.uint32)
+    mk = np.array([[0, 1, 1, 1], [1, 1, 1, 0]], np.uint8)
+    t, w, tokens = rs.build_targets_and_weights(tg, mk, 2, vocab=10)
+    np.testing.assert_array_equal(t, np.array([0xFFFFFFFF, 2, 0xFFFFFFFF, 4, 5, 6, 7, 0xFFFFFFFF], np.uint32))
+    np.testing.assert_array_equal(tokens, [2, 3])
+    np.testing.assert_array_equal(w, np.array([0, .5, 0, .5, np.float32(1) / np.float32(3),
+                                               np.float32(1) / np.float32(3), np.float32(1) / np.float32(3), 0],
+                                              np.float32))
+
+
+# ---- grad norm, AdamW ----------------------------------------------------
+
+def test_sum_squares_partial_chunks():
+    x = randn(4096 * 2 + 100)
+    out = np.zeros(8, np.float32)
+    n = cpu.sum_squares_partial(x, out, 3)
+    assert n == 3 and (out[:3] == 0).all() and (out[6:] == 0).all()
+    want = [np.sum(x[i * 4096:(i + 1) * 4096].astype(np.float64) ** 2) for i in range(3)]
+    np.testing.assert_allclose(out[3:6], want, rtol=1e-5)
+    assert abs(float(rs.global_grad_norm([x])) - np.linalg.norm(x.astype(np.float64))) < 1e-3
+
+
+@pytest.mark.parametrize("wd", [0.0, 0.01])
+def test_adamw_against_torch_optim(wd):
+    n = 257
+    w0, grads = randn(n), [randn(n) for _ in range(4)]
+    wt = torch.nn.Parameter(torch.tensor(w0, dtype=torch.float64))
+    opt = torch.optim.AdamW([wt], lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=wd)
+    w, m, v = w0.copy(), np.zeros(n, np.float32), np.zeros(n, np.float32)
+    for t, g in enumerate(grads, 1):
+        wt.grad = torch.tensor(g, dtype=torch.float64)
+        opt.step()
+        cpu.adamw_update(w, g, m, v, 1e-3, 0.9, 0.999, 1e-8, wd, float(t))
+        np.testing.assert_allclose(w, wt.detach().numpy(), rtol=1e-5, atol=1e-6)
+
+
+def test_embedding_out_of_range_row_is_zero():
+    table = randn(5, 3)
+    out = cpu.embedding(table, np.array([[0, 4, 5, 1000]], np.uint32))
+    np.testing.assert_array_equal(out[0, 0], table[0])
+    np.testing.assert_array_equal(out[0, 1], table[4])
+    assert (out[0, 2:] == 0).all()
