@@ -1,0 +1,53 @@
+// Internal helpers shared by the sources of libferrotensor_hip.so.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <map>
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+#include "ferrotensor_hip.h"
+
+// The device-buffer pool: exact-size free lists, like the reference's
+// BufferPool (ferrotensor-backend/src/pool.rs), without its 512 MiB cap:
+// 288 GB of HBM leaves room to keep every step buffer resident.
+struct ft_context {
+    int device = 0;
+    hipStream_t stream = nullptr;
+    bool owns_stream = false;
+    std::unordered_map<void*, size_t> live;                 // ptr -> bytes handed out
+    std::unordered_map<size_t, std::vector<void*>> idle;    // bytes -> free buffers
+    size_t live_bytes = 0, idle_bytes = 0;
+    int num_cus = 256;
+};
+
+int ft_set_error(int code, const char* fmt, ...);
+
+#define FT_CHECK_ARG(cond, ...)                                  \
+    do {                                                         \
+        if (!(cond)) return ft_set_error(FT_ERR_INVALID, __VA_ARGS__); \
+    } while (0)
+
+#define FT_HIP(expr)                                                                      \
+    do {                                                                                  \
+        hipError_t _e = (expr);                                                           \
+        if (_e != hipSuccess)                                                             \
+            return ft_set_error(FT_ERR_HIP, "%s failed: %s (%s:%d)", #expr,               \
+                                hipGetErrorString(_e), __FILE__, __LINE__);               \
+    } while (0)
+
+#define FT_TRY(expr)                   \
+    do {                               \
+        int _rc = (expr);              \
+        if (_rc != FT_OK) return _rc;  \
+    } while (0)
+
+// Reports a launch-configuration error of the kernel just enqueued.
+#define FT_LAUNCH_CHECK() FT_HIP(hipGetLastError())
+
+static inline unsigned ft_div_up(size_t a, size_t b) { return (unsigned)((a + b - 1) / b); }

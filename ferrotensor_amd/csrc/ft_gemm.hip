@@ -1,0 +1,490 @@
+// f32 matrix products on the gfx950 matrix cores (v_mfma_f32_32x32x2_f32).
+//
+// gemm_kernel: out[M,N] = op(a) @ op(b) (+ a2[M,K2] @ op(b2)) for the three
+// layouts of the reference's tile kernel (a@b, a@b^T, a^T@b), with b stored as
+// f32 or as packed f16 (converted to f32 while the tile is staged into LDS).
+// The optional second product is the rank-r LoRA term: it runs as extra
+// iterations of the same K loop, so the fused linear costs r/K more MFMAs and
+// no extra pass over the output.
+//
+// Tiling: 256 threads = 4 waves, each wave owns a WM x WN block of 32x32 MFMA
+// accumulators. Tiles of BK = 32 are double-buffered in LDS in a "k-quad
+// major" layout [BK/4][rows][4]: one ds_read_b128 gives a lane the four k
+// values it feeds to four consecutive MFMAs (lanes 0-31 take the even quads,
+// lanes 32-63 the odd ones; the sum over k does not care about the order).
+//
+// skinny_kernel: products with at most 32 output columns (the LoRA x@A, dT, dA
+// and dB products), operands read straight from global memory into MFMA
+// operand registers, the reduction dimension split across the 4 waves.
+#include "ft_common.h"
+
+namespace {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+
+constexpr int BK = 32;
+constexpr int KQ = BK / 4;
+constexpr int LDS_PAD = 8;  // floats: makes the k-quad row stride = 8 (mod 32) banks
+
+struct GemmArgs {
+    const float* a;
+    const void* b;
+    float* out;
+    const float* a2;
+    const float* b2;
+    int M, N, K, K2;
+    long lda, ldb, ldc, lda2, ldb2;
+    int tiles_n;
+};
+
+// ---- guarded 4-element loads along the contiguous dimension --------------
+
+__device__ __forceinline__ float4 load4(const float* p, int nvalid) {
+    if (nvalid >= 4 && (((uintptr_t)p) & 15) == 0) return *reinterpret_cast<const float4*>(p);
+    float4 r = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (nvalid > 0) r.x = p[0];
+    if (nvalid > 1) r.y = p[1];
+    if (nvalid > 2) r.z = p[2];
+    if (nvalid > 3) r.w = p[3];
+    return r;
+}
+
+__device__ __forceinline__ float4 load4(const _Float16* p, int nvalid) {
+    if (nvalid >= 4 && (((uintptr_t)p) & 7) == 0) {
+        const half4_t h = *reinterpret_cast<const half4_t*>(p);
+        return make_float4((float)h.x, (float)h.y, (float)h.z, (float)h.w);
+    }
+    float4 r = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (nvalid > 0) r.x = (float)p[0];
+    if (nvalid > 1) r.y = (float)p[1];
+    if (nvalid > 2) r.z = (float)p[2];
+    if (nvalid > 3) r.w = (float)p[3];
+    return r;
+}
+
+__device__ __forceinline__ int clamp04(int v) { return v < 0 ? 0 : (v > 4 ? 4 : v); }
+
+// A ROWS x BK tile on its way from global memory to LDS, held in registers.
+// KCONTIG: element (row, k) at base[row*ld + k]; otherwise at base[k*ld + row].
+template <int ROWS, bool KCONTIG>
+struct TileRegs {
+    static constexpr int STRIDE = ROWS * 4 + LDS_PAD;  // floats per k-quad row in LDS
+    static constexpr int SLOTS_K = ROWS * KQ / 256;    // one float4 (4 k of one row) each
+    static constexpr int GROUPS = (ROWS / 4) * KQ;      // 4 rows x 4 k each
+    static constexpr int SLOTS_M = (GROUPS + 255) / 256;
+    static constexpr int NREG = KCONTIG ? SLOTS_K : SLOTS_M * 4;
+    float4 r[NREG];
+
+    template <typename T>
+    __device__ __forceinline__ void load(const T* base, long ld, int row0, int row_limit, int k0, int k_limit) {
+        const int tid = threadIdx.x;
+        if constexpr (KCONTIG) {
+#pragma unroll
+            for (int i = 0; i < SLOTS_K; i++) {
+                const int s = tid + i * 256;
+                const int row = s / KQ, kq = s % KQ;
+                const int gr = row0 + row, gk = k0 + kq * 4;
+                const int nvalid = gr < row_limit ? clamp04(k_limit - gk) : 0;
+                r[i] = load4(base + (long)gr * ld + gk, nvalid);
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < SLOTS_M; i++) {
+                const int s = tid + i * 256;
+                float4 v[4];
+#pragma unroll
+                for (int j = 0; j < 4; j++) v[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (s < GROUPS) {
+                    const int rg = s % (ROWS / 4), kq = s / (ROWS / 4);
+                    const int gr = row0 + rg * 4;
+                    const int nvalid = clamp04(row_limit - gr);
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        const int gk = k0 + kq * 4 + j;
+                        if (gk < k_limit) v[j] = load4(base + (long)gk * ld + gr, nvalid);
+                    }
+                }
+                // 4x4 transpose: register q holds the 4 k values of row q.
+                r[i * 4 + 0] = make_float4(v[0].x, v[1].x, v[2].x, v[3].x);
+                r[i * 4 + 1] = make_float4(v[0].y, v[1].y, v[2].y, v[3].y);
+                r[i * 4 + 2] = make_float4(v[0].z, v[1].z, v[2].z, v[3].z);
+                r[i * 4 + 3] = make_float4(v[0].w, v[1].w, v[2].w, v[3].w);
+            }
+        }
+    }
+
+    __device__ __forceinline__ void store(float* lds) const {
+        const int tid = threadIdx.x;
+        if constexpr (KCONTIG) {
+#pragma unroll
+            for (int i = 0; i < SLOTS_K; i++) {
+                const int s = tid + i * 256;
+                const int row = s / KQ, kq = s % KQ;
+                *reinterpret_cast<float4*>(lds + kq * STRIDE + row * 4) = r[i];
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < SLOTS_M; i++) {
+                const int s = tid + i * 256;
+                if (s < GROUPS) {
+                    const int rg = s % (ROWS / 4), kq = s / (ROWS / 4);
+                    float* dst = lds + kq * STRIDE + rg * 16;
+#pragma unroll
+                    for (int q = 0; q < 4; q++) *reinterpret_cast<float4*>(dst + q * 4) = r[i * 4 + q];
+                }
+            }
+        }
+    }
+};
+
+// LAYOUT 0: a[M,K]   b[K,N]   (a k-contiguous, b n-contiguous)
+// LAYOUT 1: a[M,K]   b[N,K]   (both k-contiguous)
+// LAYOUT 2: a[K,M]   b[K,N]   (both m/n-contiguous)
+template <int BM, int BN, int WM, int WN, int LAYOUT, bool HALF_B>
+__global__ __launch_bounds__(256) void gemm_kernel(GemmArgs p) {
+    constexpr bool A_KC = LAYOUT != 2;
+    constexpr bool B_KC = LAYOUT == 1;
+    constexpr int FM = WM / 32, FN = WN / 32;
+    constexpr int WAVES_N = BN / WN;
+    static_assert((BM / WM) * (BN / WN) == 4, "4 waves per workgroup");
+    using ATile = TileRegs<BM, A_KC>;
+    using BTile = TileRegs<BN, B_KC>;
+    using BType = typename std::conditional<HALF_B, _Float16, float>::type;
+
+    __shared__ __attribute__((aligned(16))) float As[2][KQ * (BM * 4 + LDS_PAD)];
+    __shared__ __attribute__((aligned(16))) float Bs[2][KQ * (BN * 4 + LDS_PAD)];
+
+    const int tile = blockIdx.x;
+    const int m0 = (tile / p.tiles_n) * BM;
+    const int n0 = (tile % p.tiles_n) * BN;
+    const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
+    const int wm0 = (wave / WAVES_N) * WM, wn0 = (wave % WAVES_N) * WN;
+    const int l32 = lane % 32, half = lane / 32;
+
+    floatx16 acc[FM][FN];
+#pragma unroll
+    for (int i = 0; i < FM; i++)
+#pragma unroll
+        for (int j = 0; j < FN; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
+
+    const int nt1 = (p.K + BK - 1) / BK;
+    const int nt2 = (LAYOUT != 2 && p.a2) ? (p.K2 + BK - 1) / BK : 0;
+    const int nt = nt1 + nt2;
+    const BType* bmat = reinterpret_cast<const BType*>(p.b);
+
+    ATile ta;
+    BTile tb;
+
+    // Tiles past nt1 belong to the second product (always f32, a2 k-contiguous,
+    // b2 oriented like b); they reuse the same registers and LDS slots.
+    auto fetch = [&](int t) {
+        if (t < nt1) {
+            ta.load(p.a, p.lda, m0, p.M, t * BK, p.K);
+            tb.load(bmat, p.ldb, n0, p.N, t * BK, p.K);
+        } else if constexpr (LAYOUT != 2) {
+            ta.load(p.a2, p.lda2, m0, p.M, (t - nt1) * BK, p.K2);
+            tb.load(p.b2, p.ldb2, n0, p.N, (t - nt1) * BK, p.K2);
+        }
+    };
+    auto stash = [&](int buf) {
+        ta.store(As[buf]);
+        tb.store(Bs[buf]);
+    };
+
+    if (nt > 0) {
+        fetch(0);
+        stash(0);
+    }
+    __syncthreads();
+    for (int t = 0; t < nt; t++) {
+        const int buf = t & 1;
+        if (t + 1 < nt) fetch(t + 1);
+        const float* as = As[buf];
+        const float* bs = Bs[buf];
+#pragma unroll
+        for (int s = 0; s < KQ / 2; s++) {
+            const int kq = 2 * s + half;
+            float4 af[FM], bf[FN];
+#pragma unroll
+            for (int i = 0; i < FM; i++)
+                af[i] = *reinterpret_cast<const float4*>(as + kq * (BM * 4 + LDS_PAD) + (wm0 + i * 32 + l32) * 4);
+#pragma unroll
+            for (int j = 0; j < FN; j++)
+                bf[j] = *reinterpret_cast<const float4*>(bs + kq * (BN * 4 + LDS_PAD) + (wn0 + j * 32 + l32) * 4);
+#pragma unroll
+            for (int i = 0; i < FM; i++)
+#pragma unroll
+                for (int j = 0; j < FN; j++) {
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i].x, bf[j].x, acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i].y, bf[j].y, acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i].z, bf[j].z, acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i].w, bf[j].w, acc[i][j], 0, 0, 0);
+                }
+        }
+        if (t + 1 < nt) stash(buf ^ 1);
+        __syncthreads();
+    }
+
+    // Accumulator register r of a lane is row (r/4)*8 + (lane/32)*4 + r%4,
+    // column lane%32 of its 32x32 block.
+#pragma unroll
+    for (int i = 0; i < FM; i++)
+#pragma unroll
+        for (int j = 0; j < FN; j++) {
+            const int col = n0 + wn0 + j * 32 + l32;
+            if (col >= p.N) continue;
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int row = m0 + wm0 + i * 32 + (r / 4) * 8 + half * 4 + (r % 4);
+                if (row < p.M) p.out[(long)row * p.ldc + col] = acc[i][j][r];
+            }
+        }
+}
+
+// ---------------------------------------------------------------------------
+// out[R, C] (C <= 32) = scale * X[R, Kr] @ Y[Kr, C].
+//   XT:  X is stored [Kr, R] (element (row,k) at x[k*ldx + row])
+//   YT:  Y is stored [C, Kr] (element (k,col) at y[col*ldy + k])
+//   OT:  out is stored [C, R]
+// One workgroup per 32 rows; wave w reduces k in [w*span, (w+1)*span).
+// ---------------------------------------------------------------------------
+template <bool XT, bool YT, bool OT>
+__global__ __launch_bounds__(256) void skinny_kernel(const float* __restrict__ x, const float* __restrict__ y,
+                                                     float* __restrict__ out, int R, int Kr, int C, long ldx,
+                                                     long ldy, long ldo, float scale) {
+    __shared__ float red[4][32 * 33];
+    const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
+    const int l32 = lane % 32, half = lane / 32;
+    const int r0 = blockIdx.x * 32;
+    const int row = r0 + l32;
+    const bool row_ok = row < R;
+    const bool col_ok = l32 < C;
+    // k range of this wave, in steps of 8
+    const int steps = (Kr + 7) / 8;
+    const int per = (steps + 3) / 4;
+    const int s_begin = wave * per;
+    const int s_end = (s_begin + per < steps) ? s_begin + per : steps;
+
+    floatx16 acc;
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc[r] = 0.0f;
+
+    auto load_x = [&](int k) -> float4 {  // X[row][k..k+3]
+        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (!row_ok) return v;
+        if constexpr (!XT) {
+            v = load4(x + (long)row * ldx + k, clamp04(Kr - k));
+        } else {
+            if (k + 0 < Kr) v.x = x[(long)(k + 0) * ldx + row];
+            if (k + 1 < Kr) v.y = x[(long)(k + 1) * ldx + row];
+            if (k + 2 < Kr) v.z = x[(long)(k + 2) * ldx + row];
+            if (k + 3 < Kr) v.w = x[(long)(k + 3) * ldx + row];
+        }
+        return v;
+    };
+    auto load_y = [&](int k) -> float4 {  // Y[k..k+3][col]
+        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (!col_ok) return v;
+        if constexpr (YT) {
+            v = load4(y + (long)l32 * ldy + k, clamp04(Kr - k));
+        } else {
+            if (k + 0 < Kr) v.x = y[(long)(k + 0) * ldy + l32];
+            if (k + 1 < Kr) v.y = y[(long)(k + 1) * ldy + l32];
+            if (k + 2 < Kr) v.z = y[(long)(k + 2) * ldy + l32];
+            if (k + 3 < Kr) v.w = y[(long)(k + 3) * ldy + l32];
+        }
+        return v;
+    };
+
+    constexpr int U = 4;
+    int s = s_begin;
+    for (; s + U <= s_end; s += U) {
+        float4 xv[U], yv[U];
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const int k = (s + u) * 8 + half * 4;
+            xv[u] = load_x(k);
+            yv[u] = load_y(k);
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xv[u].x, yv[u].x, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xv[u].y, yv[u].y, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xv[u].z, yv[u].z, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xv[u].w, yv[u].w, acc, 0, 0, 0);
+        }
+    }
+    for (; s < s_end; s++) {
+        const int k = s * 8 + half * 4;
+        const float4 xv = load_x(k), yv = load_y(k);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xv.x, yv.x, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xv.y, yv.y, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xv.z, yv.z, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(xv.w, yv.w, acc, 0, 0, 0);
+    }
+
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+        const int i = (r / 4) * 8 + half * 4 + (r % 4);
+        red[wave][i * 33 + l32] = acc[r];
+    }
+    __syncthreads();
+    // 1024 outputs, 256 threads: fixed order w0 + w1 + w2 + w3.
+    for (int e = threadIdx.x; e < 32 * 32; e += 256) {
+        const int i = e / 32, j = e % 32;
+        if (r0 + i < R && j < C) {
+            const float v = ((red[0][i * 33 + j] + red[1][i * 33 + j]) + red[2][i * 33 + j]) + red[3][i * 33 + j];
+            if constexpr (OT)
+                out[(long)j * ldo + r0 + i] = v * scale;
+            else
+                out[(long)(r0 + i) * ldo + j] = v * scale;
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Host side
+// ---------------------------------------------------------------------------
+
+struct TileCfg {
+    int bm, bn;
+    float eff;  // relative per-tile efficiency used only to rank configurations
+};
+
+template <int BM, int BN, int WM, int WN>
+int launch_cfg(ft_context* ctx, GemmArgs p, int layout, bool half_b) {
+    const int tiles_m = (p.M + BM - 1) / BM;
+    p.tiles_n = (p.N + BN - 1) / BN;
+    const dim3 grid((unsigned)(tiles_m * p.tiles_n));
+#define FT_GEMM_LAUNCH(L, H) \
+    hipLaunchKernelGGL((gemm_kernel<BM, BN, WM, WN, L, H>), grid, dim3(256), 0, ctx->stream, p)
+    if (layout == 0) {
+        if (half_b) FT_GEMM_LAUNCH(0, true); else FT_GEMM_LAUNCH(0, false);
+    } else if (layout == 1) {
+        if (half_b) FT_GEMM_LAUNCH(1, true); else FT_GEMM_LAUNCH(1, false);
+    } else {
+        FT_GEMM_LAUNCH(2, false);
+    }
+#undef FT_GEMM_LAUNCH
+    FT_LAUNCH_CHECK();
+    return FT_OK;
+}
+
+int gemm_dispatch(ft_context* ctx, const char* who, int layout, bool half_b, const float* a, const void* b,
+                  float* out, size_t M, size_t K, size_t N, const float* a2, const float* b2, size_t K2) {
+    FT_CHECK_ARG(ctx, "%s: ctx is NULL", who);
+    FT_CHECK_ARG(M < (1u << 30) && N < (1u << 30) && K < (1u << 30) && K2 < (1u << 30), "%s: dimension too large", who);
+    if (M == 0 || N == 0) return FT_OK;
+    FT_CHECK_ARG(out && (K == 0 || (a && b)), "%s: NULL operand", who);
+    FT_CHECK_ARG((a2 == nullptr) == (b2 == nullptr), "%s: a2 and b2 must come together", who);
+    FT_CHECK_ARG(!(layout == 2 && (half_b || a2)), "%s: unsupported operand combination", who);
+    GemmArgs p{};
+    p.a = a;
+    p.b = b;
+    p.out = out;
+    p.a2 = K2 > 0 ? a2 : nullptr;
+    p.b2 = K2 > 0 ? b2 : nullptr;
+    p.M = (int)M;
+    p.N = (int)N;
+    p.K = (int)K;
+    p.K2 = (int)K2;
+    p.lda = layout == 2 ? (long)M : (long)K;
+    p.ldb = layout == 1 ? (long)K : (long)N;
+    p.ldc = (long)N;
+    p.lda2 = (long)K2;
+    p.ldb2 = layout == 1 ? (long)K2 : (long)N;
+    // Pick the tile that needs the fewest rounds over the CUs, weighted by how
+    // well each shape amortises its loads.
+    const TileCfg cfgs[3] = {{128, 128, 1.00f}, {128, 64, 0.95f}, {64, 64, 0.88f}};
+    int best = 0;
+    float best_cost = 0.0f;
+    for (int c = 0; c < 3; c++) {
+        const size_t tiles = ((M + cfgs[c].bm - 1) / cfgs[c].bm) * ((N + cfgs[c].bn - 1) / cfgs[c].bn);
+        const size_t rounds = (tiles + ctx->num_cus - 1) / ctx->num_cus;
+        const float cost = (float)rounds * (float)(cfgs[c].bm * cfgs[c].bn) / cfgs[c].eff;
+        if (c == 0 || cost < best_cost) {
+            best = c;
+            best_cost = cost;
+        }
+    }
+    if (best == 0) return launch_cfg<128, 128, 64, 64>(ctx, p, layout, half_b);
+    if (best == 1) return launch_cfg<128, 64, 64, 32>(ctx, p, layout, half_b);
+    return launch_cfg<64, 64, 32, 32>(ctx, p, layout, half_b);
+}
+
+template <bool XT, bool YT, bool OT>
+int skinny_launch(ft_context* ctx, const float* x, const float* y, float* out, size_t R, size_t Kr, size_t C,
+                  long ldx, long ldy, long ldo, float scale) {
+    if (R == 0 || C == 0) return FT_OK;
+    hipLaunchKernelGGL((skinny_kernel<XT, YT, OT>), dim3(ft_div_up(R, 32)), dim3(256), 0, ctx->stream, x, y, out,
+                       (int)R, (int)Kr, (int)C, ldx, ldy, ldo, scale);
+    FT_LAUNCH_CHECK();
+    return FT_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int ft_matmul(ft_context* ctx, const float* a, const float* b, float* out, size_t M, size_t K, size_t N) {
+    return gemm_dispatch(ctx, "ft_matmul", 0, false, a, b, out, M, K, N, nullptr, nullptr, 0);
+}
+int ft_matmul_bt(ft_context* ctx, const float* a, const float* b, float* out, size_t M, size_t K, size_t N) {
+    return gemm_dispatch(ctx, "ft_matmul_bt", 1, false, a, b, out, M, K, N, nullptr, nullptr, 0);
+}
+int ft_matmul_at(ft_context* ctx, const float* a, const float* b, float* out, size_t M, size_t K, size_t N) {
+    return gemm_dispatch(ctx, "ft_matmul_at", 2, false, a, b, out, M, K, N, nullptr, nullptr, 0);
+}
+int ft_matmul_f16b(ft_context* ctx, const float* a, const uint16_t* b, float* out, size_t M, size_t K, size_t N) {
+    return gemm_dispatch(ctx, "ft_matmul_f16b", 0, true, a, b, out, M, K, N, nullptr, nullptr, 0);
+}
+int ft_matmul_bt_f16b(ft_context* ctx, const float* a, const uint16_t* b, float* out, size_t M, size_t K, size_t N) {
+    return gemm_dispatch(ctx, "ft_matmul_bt_f16b", 1, true, a, b, out, M, K, N, nullptr, nullptr, 0);
+}
+
+int ft_lora_down(ft_context* ctx, const float* x, const float* a, float* t, size_t M, size_t K, size_t r,
+                 float scale) {
+    FT_CHECK_ARG(ctx && x && a && t, "ft_lora_down: NULL argument");
+    FT_CHECK_ARG(r >= 1 && r <= 32, "ft_lora_down: rank %zu is outside 1..32", r);
+    return skinny_launch<false, false, false>(ctx, x, a, t, M, K, r, (long)K, (long)r, (long)r, scale);
+}
+
+int ft_lora_linear(ft_context* ctx, const float* x, const void* w, int w_dtype, const float* t, const float* b,
+                   float* y, size_t M, size_t K, size_t N, size_t r) {
+    FT_CHECK_ARG(w_dtype == FT_DTYPE_F32 || w_dtype == FT_DTYPE_F16, "ft_lora_linear: dtype %d", w_dtype);
+    return gemm_dispatch(ctx, "ft_lora_linear", 0, w_dtype == FT_DTYPE_F16, x, w, y, M, K, N, t, b, r);
+}
+
+int ft_lora_grad_down(ft_context* ctx, const float* dy, const float* b, float* dt, size_t M, size_t N, size_t r,
+                      float scale) {
+    FT_CHECK_ARG(ctx && dy && b && dt, "ft_lora_grad_down: NULL argument");
+    FT_CHECK_ARG(r >= 1 && r <= 32, "ft_lora_grad_down: rank %zu is outside 1..32", r);
+    // dt[m][j] = sum_n dy[m][n] * b[j][n]
+    return skinny_launch<false, true, false>(ctx, dy, b, dt, M, N, r, (long)N, (long)N, (long)r, scale);
+}
+
+int ft_lora_linear_dx(ft_context* ctx, const float* dy, const void* w, int w_dtype, const float* dt,
+                      const float* a, float* dx, size_t M, size_t K, size_t N, size_t r) {
+    FT_CHECK_ARG(w_dtype == FT_DTYPE_F32 || w_dtype == FT_DTYPE_F16, "ft_lora_linear_dx: dtype %d", w_dtype);
+    // dx[M,K] = dy[M,N] @ w[K,N]^T + dt[M,r] @ a[K,r]^T: layout 1 with output width K, reduction N.
+    return gemm_dispatch(ctx, "ft_lora_linear_dx", 1, w_dtype == FT_DTYPE_F16, dy, w, dx, M, N, K, dt, a, r);
+}
+
+int ft_lora_grad_b(ft_context* ctx, const float* t, const float* dy, float* db, size_t M, size_t N, size_t r) {
+    FT_CHECK_ARG(ctx && t && dy && db, "ft_lora_grad_b: NULL argument");
+    FT_CHECK_ARG(r >= 1 && r <= 32, "ft_lora_grad_b: rank %zu is outside 1..32", r);
+    // db^T[n][j] = sum_m dy[m][n] * t[m][j]: rows = n (dy read transposed), output stored transposed.
+    return skinny_launch<true, false, true>(ctx, dy, t, db, N, M, r, (long)N, (long)r, (long)N, 1.0f);
+}
+
+int ft_lora_grad_a(ft_context* ctx, const float* x, const float* dt, float* da, size_t M, size_t K, size_t r) {
+    FT_CHECK_ARG(ctx && x && dt && da, "ft_lora_grad_a: NULL argument");
+    FT_CHECK_ARG(r >= 1 && r <= 32, "ft_lora_grad_a: rank %zu is outside 1..32", r);
+    // da[k][j] = sum_m x[m][k] * dt[m][j]: rows = k (x read transposed).
+    return skinny_launch<true, false, false>(ctx, x, dt, da, K, M, r, (long)K, (long)r, (long)r, 1.0f);
+}
+
+}  // extern "C"

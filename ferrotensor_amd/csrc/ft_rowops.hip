@@ -1,0 +1,794 @@
+// Bandwidth-bound kernels of the LoRA step for gfx950: RMSNorm forward and
+// backward, RoPE, SiLU-gate, adds and scales, masked softmax-cross-entropy,
+// gradient-norm partials, AdamW, embedding gather. Each is written to touch
+// every array once (float4 accesses, one row or chunk per workgroup, 64-lane
+// wave reductions), so HBM traffic equals the algorithmic byte count.
+#include "ft_common.h"
+
+namespace {
+
+constexpr int kWave = 64;
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = kWave / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int o = kWave / 2; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, kWave));
+    return v;
+}
+
+// Block-wide sum / max over NT threads (NT a multiple of 64, <= 1024). Every
+// thread gets the result. `red` holds NT/64 floats.
+template <int NT>
+__device__ __forceinline__ float block_sum(float v, float* red) {
+    v = wave_sum(v);
+    const int w = threadIdx.x / kWave, l = threadIdx.x % kWave;
+    __syncthreads();
+    if (l == 0) red[w] = v;
+    __syncthreads();
+    float t = (l < NT / kWave) ? red[l] : 0.0f;
+    return wave_sum(t);
+}
+template <int NT>
+__device__ __forceinline__ float block_max(float v, float* red) {
+    v = wave_max(v);
+    const int w = threadIdx.x / kWave, l = threadIdx.x % kWave;
+    __syncthreads();
+    if (l == 0) red[w] = v;
+    __syncthreads();
+    float t = (l < NT / kWave) ? red[l] : -3.4e38f;
+    return wave_max(t);
+}
+
+__host__ __device__ inline bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
+
+// ---------------------------------------------------------------------------
+// Elementwise
+// ---------------------------------------------------------------------------
+
+enum class Ew { Add, AddBackward, SiluGate, SiluGateBackward, Scale, Accumulate, Zero };
+
+struct EwArgs {
+    const float* a;
+    const float* b;
+    const float* c;
+    float* o0;
+    float* o1;
+    size_t n;
+    float s;
+};
+
+template <Ew OP>
+__device__ __forceinline__ void ew_apply(const EwArgs& p, size_t i) {
+    if constexpr (OP == Ew::Add) {
+        p.o0[i] = p.a[i] + p.b[i];
+    } else if constexpr (OP == Ew::AddBackward) {
+        const float g = p.a[i];
+        p.o0[i] = g;
+        p.o1[i] = g;
+    } else if constexpr (OP == Ew::SiluGate) {
+        const float x = p.a[i];
+        const float silu = x * (1.0f / (1.0f + __expf(-x)));
+        p.o0[i] = silu * p.b[i];
+    } else if constexpr (OP == Ew::SiluGateBackward) {
+        const float x = p.a[i], y = p.b[i], g = p.c[i];
+        const float s = 1.0f / (1.0f + __expf(-x));
+        p.o1[i] = g * (x * s);
+        p.o0[i] = g * y * (s * (1.0f + x * (1.0f - s)));
+    } else if constexpr (OP == Ew::Scale) {
+        p.o0[i] = p.o0[i] * p.s;
+    } else if constexpr (OP == Ew::Accumulate) {
+        p.o0[i] = p.o0[i] + p.a[i];
+    } else {
+        p.o0[i] = 0.0f;
+    }
+}
+
+template <Ew OP>
+__device__ __forceinline__ void ew_apply4(const EwArgs& p, size_t i4) {
+    const float4* a = reinterpret_cast<const float4*>(p.a);
+    const float4* b = reinterpret_cast<const float4*>(p.b);
+    const float4* c = reinterpret_cast<const float4*>(p.c);
+    float4* o0 = reinterpret_cast<float4*>(p.o0);
+    float4* o1 = reinterpret_cast<float4*>(p.o1);
+    if constexpr (OP == Ew::Add) {
+        const float4 x = a[i4], y = b[i4];
+        o0[i4] = make_float4(x.x + y.x, x.y + y.y, x.z + y.z, x.w + y.w);
+    } else if constexpr (OP == Ew::AddBackward) {
+        const float4 g = a[i4];
+        o0[i4] = g;
+        o1[i4] = g;
+    } else if constexpr (OP == Ew::SiluGate) {
+        const float4 x = a[i4], y = b[i4];
+        float4 r;
+        r.x = x.x * (1.0f / (1.0f + __expf(-x.x))) * y.x;
+        r.y = x.y * (1.0f / (1.0f + __expf(-x.y))) * y.y;
+        r.z = x.z * (1.0f / (1.0f + __expf(-x.z))) * y.z;
+        r.w = x.w * (1.0f / (1.0f + __expf(-x.w))) * y.w;
+        o0[i4] = r;
+    } else if constexpr (OP == Ew::SiluGateBackward) {
+        const float4 x = a[i4], y = b[i4], g = c[i4];
+        float4 ga, gb;
+#define FT_SGB(f)                                              \
+    {                                                          \
+        const float s = 1.0f / (1.0f + __expf(-x.f));          \
+        gb.f = g.f * (x.f * s);                                \
+        ga.f = g.f * y.f * (s * (1.0f + x.f * (1.0f - s)));    \
+    }
+        FT_SGB(x) FT_SGB(y) FT_SGB(z) FT_SGB(w)
+#undef FT_SGB
+        o0[i4] = ga;
+        o1[i4] = gb;
+    } else if constexpr (OP == Ew::Scale) {
+        float4 x = o0[i4];
+        x.x *= p.s; x.y *= p.s; x.z *= p.s; x.w *= p.s;
+        o0[i4] = x;
+    } else if constexpr (OP == Ew::Accumulate) {
+        float4 x = o0[i4];
+        const float4 y = a[i4];
+        x.x += y.x; x.y += y.y; x.z += y.z; x.w += y.w;
+        o0[i4] = x;
+    } else {
+        o0[i4] = make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+}
+
+template <Ew OP, bool VEC>
+__global__ __launch_bounds__(256) void ew_kernel(EwArgs p) {
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if constexpr (VEC) {
+        const size_t n4 = p.n / 4;
+        for (; i < n4; i += stride) ew_apply4<OP>(p, i);
+        // tail (n % 4 elements) by the first threads
+        const size_t t = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+        if (t < p.n - n4 * 4) ew_apply<OP>(p, n4 * 4 + t);
+    } else {
+        for (; i < p.n; i += stride) ew_apply<OP>(p, i);
+    }
+}
+
+template <Ew OP>
+int ew_launch(ft_context* ctx, EwArgs p) {
+    if (p.n == 0) return FT_OK;
+    const bool vec = aligned16(p.a) && aligned16(p.b) && aligned16(p.c) && aligned16(p.o0) && aligned16(p.o1);
+    const size_t work = vec ? (p.n + 3) / 4 : p.n;
+    size_t blocks = (work + 255) / 256;
+    const size_t cap = (size_t)ctx->num_cus * 16;
+    if (blocks > cap) blocks = cap;
+    if (vec)
+        hipLaunchKernelGGL((ew_kernel<OP, true>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, p);
+    else
+        hipLaunchKernelGGL((ew_kernel<OP, false>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, p);
+    FT_LAUNCH_CHECK();
+    return FT_OK;
+}
+
+// ---------------------------------------------------------------------------
+// Embedding gather: one wave per token row.
+// ---------------------------------------------------------------------------
+
+__global__ __launch_bounds__(256) void embedding_kernel(const float* __restrict__ table, size_t vocab,
+                                                        size_t hidden, const uint32_t* __restrict__ ids,
+                                                        size_t n, float* __restrict__ out) {
+    const size_t row = (size_t)blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
+    if (row >= n) return;
+    const int lane = threadIdx.x % kWave;
+    const uint32_t id = ids[row];
+    float* o = out + row * hidden;
+    if ((size_t)id < vocab) {
+        const float* src = table + (size_t)id * hidden;
+        if ((hidden & 3) == 0 && aligned16(table) && aligned16(out)) {
+            const float4* s4 = reinterpret_cast<const float4*>(src);
+            float4* o4 = reinterpret_cast<float4*>(o);
+            for (size_t i = lane; i < hidden / 4; i += kWave) o4[i] = s4[i];
+        } else {
+            for (size_t i = lane; i < hidden; i += kWave) o[i] = src[i];
+        }
+    } else {
+        for (size_t i = lane; i < hidden; i += kWave) o[i] = 0.0f;
+    }
+}
+
+// ---------------------------------------------------------------------------
+// RMSNorm. One 256-thread workgroup per row; the second sweep over the row
+// re-reads what the first sweep just pulled into cache.
+// ---------------------------------------------------------------------------
+
+__global__ __launch_bounds__(256) void rms_norm_kernel(const float* __restrict__ x, const float* __restrict__ w,
+                                                       float* __restrict__ out, size_t rows, size_t size,
+                                                       float eps, int vec) {
+    __shared__ float red[4];
+    const size_t row = blockIdx.x;
+    const float* xr = x + row * size;
+    float* orow = out + row * size;
+    float ss = 0.0f;
+    if (vec) {
+        const float4* x4 = reinterpret_cast<const float4*>(xr);
+        for (size_t i = threadIdx.x; i < size / 4; i += 256) {
+            const float4 v = x4[i];
+            ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+        }
+    } else {
+        for (size_t i = threadIdx.x; i < size; i += 256) ss += xr[i] * xr[i];
+    }
+    ss = block_sum<256>(ss, red);
+    const float inv = 1.0f / sqrtf(ss / (float)size + eps);
+    if (vec) {
+        const float4* x4 = reinterpret_cast<const float4*>(xr);
+        const float4* w4 = reinterpret_cast<const float4*>(w);
+        float4* o4 = reinterpret_cast<float4*>(orow);
+        for (size_t i = threadIdx.x; i < size / 4; i += 256) {
+            const float4 v = x4[i], g = w4[i];
+            o4[i] = make_float4(v.x * inv * g.x, v.y * inv * g.y, v.z * inv * g.z, v.w * inv * g.w);
+        }
+    } else {
+        for (size_t i = threadIdx.x; i < size; i += 256) orow[i] = xr[i] * inv * w[i];
+    }
+}
+
+// Backward for ROWS_PER_WG consecutive rows per workgroup. gx as in the
+// reference; when gw_partial != nullptr each workgroup also writes its rows'
+// contribution sum g*x*inv per feature to gw_partial[blockIdx.x * size + i].
+template <int ROWS_PER_WG>
+__global__ __launch_bounds__(256) void rms_norm_backward_kernel(
+    const float* __restrict__ x, const float* __restrict__ w, const float* __restrict__ g,
+    float* __restrict__ gx, float* __restrict__ gw_partial, size_t rows, size_t size, float eps) {
+    __shared__ float red[4];
+    const size_t row0 = (size_t)blockIdx.x * ROWS_PER_WG;
+    // Columns this thread owns: threadIdx.x + 256*j. Up to 8 partial sums stay
+    // in registers; wider rows fall back to read-modify-write on the partial row.
+    constexpr int MAXC = 8;
+    float gwacc[MAXC];
+#pragma unroll
+    for (int j = 0; j < MAXC; j++) gwacc[j] = 0.0f;
+    const bool wide = size > (size_t)256 * MAXC;
+    if (gw_partial && wide)
+        for (size_t i = threadIdx.x; i < size; i += 256) gw_partial[(size_t)blockIdx.x * size + i] = 0.0f;
+    for (int rr = 0; rr < ROWS_PER_WG; rr++) {
+        const size_t row = row0 + rr;
+        if (row >= rows) break;  // uniform
+        const float* xr = x + row * size;
+        const float* gr = g + row * size;
+        float ss = 0.0f, gwx = 0.0f;
+        for (size_t i = threadIdx.x; i < size; i += 256) {
+            const float xv = xr[i];
+            ss += xv * xv;
+            gwx += gr[i] * w[i] * xv;
+        }
+        ss = block_sum<256>(ss, red);
+        gwx = block_sum<256>(gwx, red);
+        const float inv = 1.0f / sqrtf(ss / (float)size + eps);
+        const float coef = gwx * inv * inv * inv / (float)size;
+        int j = 0;
+        for (size_t i = threadIdx.x; i < size; i += 256, j++) {
+            const float xv = xr[i], gv = gr[i];
+            gx[row * size + i] = gv * w[i] * inv - xv * coef;
+            if (gw_partial) {
+                if (!wide) {
+                    // j < MAXC by construction; the unrolled select keeps gwacc in registers.
+#pragma unroll
+                    for (int q = 0; q < MAXC; q++)
+                        if (q == j) gwacc[q] += gv * xv * inv;
+                } else {
+                    gw_partial[(size_t)blockIdx.x * size + i] += gv * xv * inv;
+                }
+            }
+        }
+    }
+    if (gw_partial && !wide) {
+        int j = 0;
+        for (size_t i = threadIdx.x; i < size; i += 256, j++) {
+            float v = 0.0f;
+#pragma unroll
+            for (int q = 0; q < MAXC; q++)
+                if (q == j) v = gwacc[q];
+            gw_partial[(size_t)blockIdx.x * size + i] = v;
+        }
+    }
+}
+
+// gw[i] = sum over partial rows, in ascending order (deterministic).
+__global__ __launch_bounds__(256) void column_sum_kernel(const float* __restrict__ partial, float* __restrict__ out,
+                                                         size_t parts, size_t size) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= size) return;
+    float acc = 0.0f;
+    for (size_t p = 0; p < parts; p++) acc += partial[p * size + i];
+    out[i] = acc;
+}
+
+// ---------------------------------------------------------------------------
+// RoPE (rotate-half). One thread per (token, head, i < head_dim/2) pair.
+// Angles in f32 exactly as pos * powf(theta, -2i/head_dim), precise sin/cos.
+// ---------------------------------------------------------------------------
+
+__global__ __launch_bounds__(256) void rope_kernel(const float* __restrict__ src, float* __restrict__ dst,
+                                                   size_t pairs, unsigned head_dim, unsigned seq,
+                                                   unsigned pos0, unsigned heads, float theta, float dir) {
+    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= pairs) return;
+    const unsigned half = head_dim / 2;
+    const size_t vec = idx / half;              // head-vector index
+    const unsigned i = (unsigned)(idx % half);
+    const float pos = (float)(pos0 + (unsigned)((vec / heads) % seq));
+    const float freq_exp = -2.0f * (float)i / (float)head_dim;
+    const float angle = dir * pos * powf(theta, freq_exp);
+    float s, c;
+    sincosf(angle, &s, &c);
+    const size_t i1 = vec * head_dim + i, i2 = i1 + half;
+    const float v1 = src[i1], v2 = src[i2];
+    dst[i1] = v1 * c - v2 * s;
+    dst[i2] = v1 * s + v2 * c;
+}
+
+// ---------------------------------------------------------------------------
+// Masked softmax-cross-entropy. One 1024-thread workgroup per row. A row of up
+// to 1024*4*CACHE floats is held in registers between the reduction and the
+// gradient write, so logits are read once and the gradient written once.
+// ---------------------------------------------------------------------------
+
+constexpr int kCeThreads = 1024;
+
+template <int CACHE>  // float4 per thread kept in registers (0 = stream from memory)
+__global__ __launch_bounds__(kCeThreads) void masked_ce_kernel(
+    const float* __restrict__ logits, const uint32_t* __restrict__ targets, const float* __restrict__ weights,
+    float* grad, float* __restrict__ row_loss, size_t rows, size_t vocab, float grad_scale) {
+    __shared__ float red[kCeThreads / kWave];
+    const size_t row = blockIdx.x;
+    const float* x = logits + row * vocab;
+    float* gr = grad + row * vocab;
+    const uint32_t tgt = targets[row];
+    const size_t n4 = vocab / 4;
+    if (tgt == FT_MASKED_CE_SKIP) {
+        float4* g4 = reinterpret_cast<float4*>(gr);
+        for (size_t i = threadIdx.x; i < n4; i += kCeThreads) g4[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+        for (size_t i = n4 * 4 + threadIdx.x; i < vocab; i += kCeThreads) gr[i] = 0.0f;
+        if (threadIdx.x == 0) row_loss[row] = 0.0f;
+        return;
+    }
+    const float4* x4 = reinterpret_cast<const float4*>(x);
+    float4 cache[CACHE > 0 ? CACHE : 1];
+    float m = -3.4e38f;
+    if constexpr (CACHE > 0) {
+#pragma unroll
+        for (int j = 0; j < CACHE; j++) {
+            const size_t i = threadIdx.x + (size_t)j * kCeThreads;
+            if (i < n4) {
+                cache[j] = x4[i];
+                m = fmaxf(m, fmaxf(fmaxf(cache[j].x, cache[j].y), fmaxf(cache[j].z, cache[j].w)));
+            }
+        }
+    } else {
+        for (size_t i = threadIdx.x; i < n4; i += kCeThreads) {
+            const float4 v = x4[i];
+            m = fmaxf(m, fmaxf(fmaxf(v.x, v.y), fmaxf(v.z, v.w)));
+        }
+    }
+    for (size_t i = n4 * 4 + threadIdx.x; i < vocab; i += kCeThreads) m = fmaxf(m, x[i]);
+    m = block_max<kCeThreads>(m, red);
+    float se = 0.0f;
+    if constexpr (CACHE > 0) {
+#pragma unroll
+        for (int j = 0; j < CACHE; j++) {
+            const size_t i = threadIdx.x + (size_t)j * kCeThreads;
+            if (i < n4) se += expf(cache[j].x - m) + expf(cache[j].y - m) + expf(cache[j].z - m) + expf(cache[j].w - m);
+        }
+    } else {
+        for (size_t i = threadIdx.x; i < n4; i += kCeThreads) {
+            const float4 v = x4[i];
+            se += expf(v.x - m) + expf(v.y - m) + expf(v.z - m) + expf(v.w - m);
+        }
+    }
+    for (size_t i = n4 * 4 + threadIdx.x; i < vocab; i += kCeThreads) se += expf(x[i] - m);
+    se = block_sum<kCeThreads>(se, red);
+    const float log_z = m + logf(se);
+    const float w = weights[row];
+    // The target logit is read before any thread overwrites it (grad may alias logits).
+    const float x_t = x[tgt];
+    __syncthreads();
+    float4* g4 = reinterpret_cast<float4*>(gr);
+    auto one = [&](float xv, size_t i) {
+        float gv = expf(xv - log_z) * w;
+        if (i == (size_t)tgt) gv -= w;
+        return gv * grad_scale;
+    };
+    if constexpr (CACHE > 0) {
+#pragma unroll
+        for (int j = 0; j < CACHE; j++) {
+            const size_t i = threadIdx.x + (size_t)j * kCeThreads;
+            if (i < n4) {
+                const float4 v = cache[j];
+                g4[i] = make_float4(one(v.x, 4 * i), one(v.y, 4 * i + 1), one(v.z, 4 * i + 2), one(v.w, 4 * i + 3));
+            }
+        }
+    } else {
+        for (size_t i = threadIdx.x; i < n4; i += kCeThreads) {
+            const float4 v = x4[i];
+            g4[i] = make_float4(one(v.x, 4 * i), one(v.y, 4 * i + 1), one(v.z, 4 * i + 2), one(v.w, 4 * i + 3));
+        }
+    }
+    for (size_t i = n4 * 4 + threadIdx.x; i < vocab; i += kCeThreads) gr[i] = one(x[i], i);
+    if (threadIdx.x == 0) row_loss[row] = log_z - x_t;
+}
+
+// Scalar variant for rows that are not 16-byte aligned (vocab % 4 != 0).
+__global__ __launch_bounds__(256) void masked_ce_scalar_kernel(
+    const float* __restrict__ logits, const uint32_t* __restrict__ targets, const float* __restrict__ weights,
+    float* grad, float* __restrict__ row_loss, size_t rows, size_t vocab, float grad_scale) {
+    __shared__ float red[4];
+    const size_t row = blockIdx.x;
+    const float* x = logits + row * vocab;
+    float* gr = grad + row * vocab;
+    const uint32_t tgt = targets[row];
+    if (tgt == FT_MASKED_CE_SKIP) {
+        for (size_t i = threadIdx.x; i < vocab; i += 256) gr[i] = 0.0f;
+        if (threadIdx.x == 0) row_loss[row] = 0.0f;
+        return;
+    }
+    float m = -3.4e38f;
+    for (size_t i = threadIdx.x; i < vocab; i += 256) m = fmaxf(m, x[i]);
+    m = block_max<256>(m, red);
+    float se = 0.0f;
+    for (size_t i = threadIdx.x; i < vocab; i += 256) se += expf(x[i] - m);
+    se = block_sum<256>(se, red);
+    const float log_z = m + logf(se);
+    const float w = weights[row];
+    const float x_t = x[tgt];
+    __syncthreads();
+    for (size_t i = threadIdx.x; i < vocab; i += 256) {
+        float gv = expf(x[i] - log_z) * w;
+        if (i == (size_t)tgt) gv -= w;
+        gr[i] = gv * grad_scale;
+    }
+    if (threadIdx.x == 0) row_loss[row] = log_z - x_t;
+}
+
+// ---------------------------------------------------------------------------
+// Sum of squares per 4096-element chunk; AdamW.
+// ---------------------------------------------------------------------------
+
+__global__ __launch_bounds__(256) void sum_squares_kernel(const float* __restrict__ x, size_t n,
+                                                          float* __restrict__ out, size_t offset) {
+    __shared__ float red[4];
+    const size_t start = (size_t)blockIdx.x * FT_SUM_SQUARES_CHUNK;
+    const size_t end = start + FT_SUM_SQUARES_CHUNK < n ? start + FT_SUM_SQUARES_CHUNK : n;
+    float acc = 0.0f;
+    for (size_t i = start + threadIdx.x; i < end; i += 256) {
+        const float v = x[i];
+        acc += v * v;
+    }
+    acc = block_sum<256>(acc, red);
+    if (threadIdx.x == 0) out[offset + blockIdx.x] = acc;
+}
+
+__device__ __forceinline__ void adamw_one(float& w, float g, float& m, float& v, const ft_adam_params& p,
+                                          float bc1, float bc2) {
+    m = m * p.beta1 + (1.0f - p.beta1) * g;
+    v = v * p.beta2 + (1.0f - p.beta2) * g * g;
+    const float m_hat = m / bc1;
+    const float v_hat = v / bc2;
+    w = w - p.lr * (m_hat / (sqrtf(v_hat) + p.eps) + p.weight_decay * w);
+}
+
+__global__ __launch_bounds__(256) void adamw_kernel(float* __restrict__ w, const float* __restrict__ g,
+                                                    float* __restrict__ m, float* __restrict__ v, size_t n,
+                                                    ft_adam_params p, float grad_scale) {
+    const float bc1 = 1.0f - powf(p.beta1, p.t);
+    const float bc2 = 1.0f - powf(p.beta2, p.t);
+    const size_t stride = (size_t)gridDim.x * 256;
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) {
+        float wi = w[i], mi = m[i], vi = v[i];
+        adamw_one(wi, g[i] * grad_scale, mi, vi, p, bc1, bc2);
+        w[i] = wi;
+        m[i] = mi;
+        v[i] = vi;
+    }
+}
+
+}  // namespace
+
+// A segment of the multi-tensor AdamW / gradient-norm launch: one
+// FT_SUM_SQUARES_CHUNK-sized piece of one tensor.
+struct ft_segment {
+    float* w;
+    float* g;
+    float* m;
+    float* v;
+    uint32_t n;  // elements in this piece (<= 4096)
+};
+
+namespace {
+
+// Step control block in device memory, written by the norm kernel and read by
+// the AdamW kernel so that no host round trip sits between them.
+struct StepControl {
+    float grad_norm;
+    float clip_scale;
+    int apply;       // 0 when the norm is not finite: the update is skipped
+};
+
+__global__ __launch_bounds__(256) void multi_sum_squares_kernel(const ft_segment* __restrict__ segs,
+                                                                float* __restrict__ partials) {
+    __shared__ float red[4];
+    const ft_segment s = segs[blockIdx.x];
+    float acc = 0.0f;
+    for (uint32_t i = threadIdx.x; i < s.n; i += 256) {
+        const float v = s.g[i];
+        acc += v * v;
+    }
+    acc = block_sum<256>(acc, red);
+    if (threadIdx.x == 0) partials[blockIdx.x] = acc;
+}
+
+// Adds the partials in f64 in index order (the reference adds them on the host
+// in f64, trainer/src/lib.rs:528-533), then derives the clip scale
+// max / (norm + 1e-6) when norm > max (trainer/src/lib.rs:336-343).
+__global__ __launch_bounds__(256) void grad_norm_finish_kernel(const float* __restrict__ partials, size_t count,
+                                                               float max_norm, float* out /* StepControl */) {
+    __shared__ double red[256];
+    // Fixed assignment of contiguous ranges to threads keeps the result
+    // independent of scheduling.
+    const size_t per = (count + 255) / 256;
+    const size_t b = threadIdx.x * per;
+    const size_t e = b + per < count ? b + per : count;
+    double acc = 0.0;
+    for (size_t i = b; i < e; i++) acc += (double)partials[i];
+    red[threadIdx.x] = acc;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        double t = 0.0;
+        for (int i = 0; i < 256; i++) t += red[i];
+        const float norm = (float)sqrt(t);
+        StepControl* c = reinterpret_cast<StepControl*>(out);
+        c->grad_norm = norm;
+        const bool finite = isfinite(norm);
+        c->apply = finite ? 1 : 0;
+        c->clip_scale = (finite && max_norm > 0.0f && norm > max_norm) ? max_norm / (norm + 1e-6f) : 1.0f;
+    }
+}
+
+__global__ __launch_bounds__(256) void multi_adamw_kernel(const ft_segment* __restrict__ segs, ft_adam_params p,
+                                                          float grad_scale, const float* control) {
+    float scale = grad_scale;
+    if (control) {
+        const StepControl* c = reinterpret_cast<const StepControl*>(control);
+        if (!c->apply) return;
+        scale *= c->clip_scale;
+    }
+    const ft_segment s = segs[blockIdx.x];
+    const float bc1 = 1.0f - powf(p.beta1, p.t);
+    const float bc2 = 1.0f - powf(p.beta2, p.t);
+    for (uint32_t i = threadIdx.x; i < s.n; i += 256) {
+        float wi = s.w[i], mi = s.m[i], vi = s.v[i];
+        // The clip scale of the reference's clip_grad_by_norm pass is applied on
+        // the fly; the stored gradient stays unclipped.
+        adamw_one(wi, s.g[i] * scale, mi, vi, p, bc1, bc2);
+        s.w[i] = wi;
+        s.m[i] = mi;
+        s.v[i] = vi;
+    }
+}
+
+}  // namespace
+
+// Internal entry points used by the step driver (ft_step.cpp).
+int ft_internal_multi_grad_norm(ft_context* ctx, const ft_segment* segs_dev, size_t nseg, float* partials_dev,
+                                float max_norm, float* control_dev) {
+    if (nseg == 0) return FT_OK;
+    hipLaunchKernelGGL(multi_sum_squares_kernel, dim3((unsigned)nseg), dim3(256), 0, ctx->stream, segs_dev,
+                       partials_dev);
+    FT_LAUNCH_CHECK();
+    hipLaunchKernelGGL(grad_norm_finish_kernel, dim3(1), dim3(256), 0, ctx->stream, partials_dev, nseg, max_norm,
+                       control_dev);
+    FT_LAUNCH_CHECK();
+    return FT_OK;
+}
+
+int ft_internal_multi_adamw(ft_context* ctx, const ft_segment* segs_dev, size_t nseg, const ft_adam_params* p,
+                            float grad_scale, const float* control_dev) {
+    if (nseg == 0) return FT_OK;
+    hipLaunchKernelGGL(multi_adamw_kernel, dim3((unsigned)nseg), dim3(256), 0, ctx->stream, segs_dev, *p,
+                       grad_scale, control_dev);
+    FT_LAUNCH_CHECK();
+    return FT_OK;
+}
+
+extern "C" {
+
+int ft_zero(ft_context* ctx, void* dev, size_t bytes) {
+    FT_CHECK_ARG(ctx && (bytes == 0 || dev), "ft_zero: NULL argument");
+    FT_CHECK_ARG(bytes % 4 == 0, "ft_zero: %zu bytes is not a whole number of words", bytes);
+    EwArgs p{nullptr, nullptr, nullptr, (float*)dev, nullptr, bytes / 4, 0.0f};
+    return ew_launch<Ew::Zero>(ctx, p);
+}
+
+int ft_add(ft_context* ctx, const float* a, const float* b, float* out, size_t n) {
+    FT_CHECK_ARG(ctx && (n == 0 || (a && b && out)), "ft_add: NULL argument");
+    EwArgs p{a, b, nullptr, out, nullptr, n, 0.0f};
+    return ew_launch<Ew::Add>(ctx, p);
+}
+
+int ft_add_backward(ft_context* ctx, const float* g, float* ga, float* gb, size_t n) {
+    FT_CHECK_ARG(ctx && (n == 0 || (g && ga && gb)), "ft_add_backward: NULL argument");
+    EwArgs p{g, nullptr, nullptr, ga, gb, n, 0.0f};
+    return ew_launch<Ew::AddBackward>(ctx, p);
+}
+
+int ft_silu_gate_fused(ft_context* ctx, const float* first, const float* second, float* out, size_t n) {
+    FT_CHECK_ARG(ctx && (n == 0 || (first && second && out)), "ft_silu_gate_fused: NULL argument");
+    EwArgs p{first, second, nullptr, out, nullptr, n, 0.0f};
+    return ew_launch<Ew::SiluGate>(ctx, p);
+}
+
+int ft_silu_gate_backward(ft_context* ctx, const float* first, const float* second, const float* g,
+                          float* g_first, float* g_second, size_t n) {
+    FT_CHECK_ARG(ctx && (n == 0 || (first && second && g && g_first && g_second)),
+                 "ft_silu_gate_backward: NULL argument");
+    EwArgs p{first, second, g, g_first, g_second, n, 0.0f};
+    return ew_launch<Ew::SiluGateBackward>(ctx, p);
+}
+
+int ft_gradient_scale(ft_context* ctx, float* x, size_t n, float scale) {
+    FT_CHECK_ARG(ctx && (n == 0 || x), "ft_gradient_scale: NULL argument");
+    EwArgs p{nullptr, nullptr, nullptr, x, nullptr, n, scale};
+    return ew_launch<Ew::Scale>(ctx, p);
+}
+
+int ft_clip_grad_by_norm(ft_context* ctx, float* x, size_t n, float scale) {
+    return ft_gradient_scale(ctx, x, n, scale);
+}
+
+int ft_gradient_accumulate(ft_context* ctx, float* acc, const float* g, size_t n) {
+    FT_CHECK_ARG(ctx && (n == 0 || (acc && g)), "ft_gradient_accumulate: NULL argument");
+    EwArgs p{g, nullptr, nullptr, acc, nullptr, n, 0.0f};
+    return ew_launch<Ew::Accumulate>(ctx, p);
+}
+
+int ft_embedding(ft_context* ctx, const float* table, size_t vocab, size_t hidden, const uint32_t* ids,
+                 size_t n, float* out) {
+    FT_CHECK_ARG(ctx && table && ids && out, "ft_embedding: NULL argument");
+    if (n == 0 || hidden == 0) return FT_OK;
+    hipLaunchKernelGGL(embedding_kernel, dim3(ft_div_up(n, 4)), dim3(256), 0, ctx->stream, table, vocab, hidden,
+                       ids, n, out);
+    FT_LAUNCH_CHECK();
+    return FT_OK;
+}
+
+int ft_rms_norm_eps(ft_context* ctx, const float* x, const float* w, float* out, size_t rows, size_t size,
+                    float eps) {
+    FT_CHECK_ARG(ctx && x && w && out, "ft_rms_norm_eps: NULL argument");
+    FT_CHECK_ARG(size > 0, "ft_rms_norm_eps: size is 0");
+    if (rows == 0) return FT_OK;
+    const int vec = (size % 4 == 0) && aligned16(x) && aligned16(w) && aligned16(out);
+    hipLaunchKernelGGL(rms_norm_kernel, dim3((unsigned)rows), dim3(256), 0, ctx->stream, x, w, out, rows, size,
+                       eps, vec);
+    FT_LAUNCH_CHECK();
+    return FT_OK;
+}
+
+int ft_rms_norm_backward(ft_context* ctx, const float* x, const float* w, const float* g, float* gx, float* gw,
+                         size_t rows, size_t size, float eps) {
+    FT_CHECK_ARG(ctx && x && w && g && gx, "ft_rms_norm_backward: NULL argument");
+    FT_CHECK_ARG(size > 0, "ft_rms_norm_backward: size is 0");
+    if (rows == 0) {
+        if (gw) return ft_zero(ctx, gw, size * 4);
+        return FT_OK;
+    }
+    constexpr int RPW = 8;
+    const size_t wgs = (rows + RPW - 1) / RPW;
+    float* partial = nullptr;
+    if (gw) FT_TRY(ft_alloc(ctx, wgs * size * sizeof(float), (void**)&partial));
+    hipLaunchKernelGGL((rms_norm_backward_kernel<RPW>), dim3((unsigned)wgs), dim3(256), 0, ctx->stream, x, w, g,
+                       gx, partial, rows, size, eps);
+    FT_LAUNCH_CHECK();
+    if (gw) {
+        hipLaunchKernelGGL(column_sum_kernel, dim3(ft_div_up(size, 256)), dim3(256), 0, ctx->stream, partial, gw,
+                           wgs, size);
+        FT_LAUNCH_CHECK();
+        FT_TRY(ft_free(ctx, partial));
+    }
+    return FT_OK;
+}
+
+static int rope_launch(ft_context* ctx, const float* src, float* dst, size_t batch, size_t seq, size_t hidden,
+                       size_t head_dim, size_t pos, float theta, int inverse, const char* who) {
+    FT_CHECK_ARG(ctx && src && dst, "%s: NULL argument", who);
+    FT_CHECK_ARG(head_dim >= 2 && head_dim % 2 == 0, "%s: head_dim %zu must be even", who, head_dim);
+    FT_CHECK_ARG(hidden % head_dim == 0, "%s: hidden %zu is not a multiple of head_dim %zu", who, hidden, head_dim);
+    const size_t pairs = batch * seq * hidden / 2;
+    if (pairs == 0) return FT_OK;
+    hipLaunchKernelGGL(rope_kernel, dim3(ft_div_up(pairs, 256)), dim3(256), 0, ctx->stream, src, dst, pairs,
+                       (unsigned)head_dim, (unsigned)seq, (unsigned)pos, (unsigned)(hidden / head_dim), theta,
+                       inverse ? -1.0f : 1.0f);
+    FT_LAUNCH_CHECK();
+    return FT_OK;
+}
+
+int ft_rope_theta(ft_context* ctx, float* t, size_t batch, size_t seq, size_t hidden, size_t head_dim, size_t pos,
+                  float theta) {
+    return rope_launch(ctx, t, t, batch, seq, hidden, head_dim, pos, theta, 0, "ft_rope_theta");
+}
+
+int ft_rope_theta_inverse(ft_context* ctx, float* t, size_t batch, size_t seq, size_t hidden, size_t head_dim,
+                          size_t pos, float theta) {
+    return rope_launch(ctx, t, t, batch, seq, hidden, head_dim, pos, theta, 1, "ft_rope_theta_inverse");
+}
+
+int ft_rope_theta_to(ft_context* ctx, const float* src, float* dst, size_t batch, size_t seq, size_t hidden,
+                     size_t head_dim, size_t pos, float theta, int inverse) {
+    return rope_launch(ctx, src, dst, batch, seq, hidden, head_dim, pos, theta, inverse, "ft_rope_theta_to");
+}
+
+int ft_sum_squares_partial(ft_context* ctx, const float* x, size_t n, float* out, size_t offset, size_t* chunks) {
+    FT_CHECK_ARG(ctx && out && (n == 0 || x), "ft_sum_squares_partial: NULL argument");
+    const size_t blocks = (n + FT_SUM_SQUARES_CHUNK - 1) / FT_SUM_SQUARES_CHUNK;
+    if (chunks) *chunks = blocks;
+    if (blocks == 0) return FT_OK;
+    hipLaunchKernelGGL(sum_squares_kernel, dim3((unsigned)blocks), dim3(256), 0, ctx->stream, x, n, out, offset);
+    FT_LAUNCH_CHECK();
+    return FT_OK;
+}
+
+int ft_masked_cross_entropy_weighted(ft_context* ctx, const float* logits, const uint32_t* targets,
+                                     const float* weights, float* grad, float* row_loss, size_t rows, size_t vocab,
+                                     float grad_scale) {
+    FT_CHECK_ARG(ctx && logits && targets && weights && grad && row_loss,
+                 "ft_masked_cross_entropy_weighted: NULL argument");
+    FT_CHECK_ARG(vocab > 0, "ft_masked_cross_entropy_weighted: vocab is 0");
+    if (rows == 0) return FT_OK;
+    const bool vec = (vocab % 4 == 0) && aligned16(logits) && aligned16(grad);
+    const dim3 grid((unsigned)rows);
+    if (!vec) {
+        hipLaunchKernelGGL(masked_ce_scalar_kernel, grid, dim3(256), 0, ctx->stream, logits, targets, weights, grad,
+                           row_loss, rows, vocab, grad_scale);
+    } else if (vocab <= (size_t)kCeThreads * 4 * 4) {
+        hipLaunchKernelGGL((masked_ce_kernel<4>), grid, dim3(kCeThreads), 0, ctx->stream, logits, targets, weights,
+                           grad, row_loss, rows, vocab, grad_scale);
+    } else if (vocab <= (size_t)kCeThreads * 4 * 12) {
+        hipLaunchKernelGGL((masked_ce_kernel<12>), grid, dim3(kCeThreads), 0, ctx->stream, logits, targets, weights,
+                           grad, row_loss, rows, vocab, grad_scale);
+    } else {
+        hipLaunchKernelGGL((masked_ce_kernel<0>), grid, dim3(kCeThreads), 0, ctx->stream, logits, targets, weights,
+                           grad, row_loss, rows, vocab, grad_scale);
+    }
+    FT_LAUNCH_CHECK();
+    return FT_OK;
+}
+
+int ft_adamw_update(ft_context* ctx, float* w, const float* g, float* m, float* v, size_t n,
+                    const ft_adam_params* p) {
+    FT_CHECK_ARG(ctx && p && (n == 0 || (w && g && m && v)), "ft_adamw_update: NULL argument");
+    if (n == 0) return FT_OK;
+    size_t blocks = (n + 255) / 256;
+    const size_t cap = (size_t)ctx->num_cus * 16;
+    if (blocks > cap) blocks = cap;
+    hipLaunchKernelGGL(adamw_kernel, dim3((unsigned)blocks), dim3(256), 0, ctx->stream, w, g, m, v, n, *p, 1.0f);
+    FT_LAUNCH_CHECK();
+    return FT_OK;
+}
+
+int ft_adamw_update_multi(ft_context* ctx, float* const* w, const float* const* g, float* const* m, float* const* v,
+                          const size_t* sizes, size_t count, const ft_adam_params* p, float grad_scale) {
+    FT_CHECK_ARG(ctx && p && (count == 0 || (w && g && m && v && sizes)), "ft_adamw_update_multi: NULL argument");
+    std::vector<ft_segment> segs;
+    for (size_t t = 0; t < count; t++) {
+        FT_CHECK_ARG(sizes[t] == 0 || (w[t] && g[t] && m[t] && v[t]), "ft_adamw_update_multi: tensor %zu is NULL", t);
+        for (size_t off = 0; off < sizes[t]; off += FT_SUM_SQUARES_CHUNK) {
+            const size_t n = sizes[t] - off < FT_SUM_SQUARES_CHUNK ? sizes[t] - off : FT_SUM_SQUARES_CHUNK;
+            segs.push_back(ft_segment{w[t] + off, const_cast<float*>(g[t]) + off, m[t] + off, v[t] + off, (uint32_t)n});
+        }
+    }
+    if (segs.empty()) return FT_OK;
+    ft_segment* dev = nullptr;
+    FT_TRY(ft_alloc(ctx, segs.size() * sizeof(ft_segment), (void**)&dev));
+    int rc = ft_upload(ctx, dev, segs.data(), segs.size() * sizeof(ft_segment));
+    if (rc == FT_OK) rc = ft_internal_multi_adamw(ctx, dev, segs.size(), p, grad_scale, nullptr);
+    const int rc2 = ft_free(ctx, dev);
+    return rc != FT_OK ? rc : rc2;
+}
+
+}  // extern "C"

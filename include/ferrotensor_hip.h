@@ -1,0 +1,319 @@
+/*
+ * ferrotensor_hip.h - C ABI of the MI355X (gfx950) kernel library behind
+ * Ferrotensor's LoRA training step.
+ *
+ * The reference has no FFI: its kernel boundary is the concrete Rust API
+ * `ferrotensor_backend::{ComputeEngine, UnifiedTensor, WgpuContext}`
+ * (ferrotensor-backend/src/lib.rs:38-46). Each entry point below is what a Rust
+ * shim implementing that API over HIP would bind; the comment above each one
+ * cites the `ComputeEngine` / `UnifiedTensor` / `WgpuContext` method it
+ * replaces.
+ *
+ * Conventions
+ *  - Every function returns FT_OK (0) or an FT_ERR_* code; `ft_last_error()`
+ *    returns the message of the calling thread's last failure. The reference
+ *    panics on shape/dtype violations (assert!); this library never aborts.
+ *  - Pointers named `*_dev`, and every tensor operand of an op, are device
+ *    pointers in the context's device. Shapes are plain sizes. f32 tensors are
+ *    row-major; "f16" operands are the packed little-endian binary16 storage of
+ *    `UnifiedTensor::from_f32_as_f16` (tensor.rs:258-269): element i at byte 2*i.
+ *  - Ops only enqueue work on the context's stream and return
+ *    (context.rs:291-317); order of execution = order of calls;
+ *    `ft_synchronize` waits (context.rs:380-391).
+ *  - Outputs are caller-allocated and written, never accumulated into, except
+ *    the in-place ops (rope, gradient_scale, clip_grad_by_norm,
+ *    gradient_accumulate, adamw_update), as in the reference.
+ *  - One thread per context at a time (the reference's autograd is
+ *    single-threaded, ferrotensor-autograd/src/lib.rs:11-14).
+ */
+#ifndef FERROTENSOR_HIP_H
+#define FERROTENSOR_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FT_OK 0
+#define FT_ERR_INVALID 1  /* bad argument / shape (the reference's assert! panics) */
+#define FT_ERR_HIP 2      /* a HIP runtime call failed */
+#define FT_ERR_OOM 3      /* device allocation failed */
+
+/* engine/training.rs:7 `MASKED_CE_SKIP`, training.rs `SUM_SQUARES_CHUNK`. */
+#define FT_MASKED_CE_SKIP 0xffffffffu
+#define FT_SUM_SQUARES_CHUNK 4096
+
+/* DType of tensor.rs:18-40 (Q4 is out of scope). */
+#define FT_DTYPE_F32 0
+#define FT_DTYPE_F16 1
+
+typedef struct ft_context ft_context;
+
+/* Message of this thread's last failing call ("" if none). */
+const char* ft_last_error(void);
+
+/* ---- context: WgpuContext (context.rs:96-156, 373-391) ------------------- */
+
+/* WgpuContext::try_new: binds HIP device `device`, creates one stream and the
+ * buffer pool. */
+int ft_context_create(int device, ft_context** out);
+/* Same, but enqueues on a stream the caller owns (hipStream_t as void*). */
+int ft_context_create_on_stream(int device, void* hip_stream, ft_context** out);
+int ft_context_destroy(ft_context* ctx);
+/* WgpuContext::synchronize (context.rs:380-391). */
+int ft_synchronize(ft_context* ctx);
+/* WgpuContext::flush (context.rs:373-378): a no-op here, launches are already submitted. */
+int ft_flush(ft_context* ctx);
+/* The hipStream_t the context enqueues on. */
+void* ft_context_stream(ft_context* ctx);
+
+/* ---- buffers: UnifiedTensor storage + BufferPool (tensor.rs, pool.rs) ---- */
+
+/* UnifiedTensor::empty (tensor.rs:184-210): uninitialised device buffer from
+ * the exact-size pool (pool.rs). */
+int ft_alloc(ft_context* ctx, size_t bytes, void** out_dev);
+/* Drop of the last Arc<TensorData> (tensor.rs:106-115): back to the pool. */
+int ft_free(ft_context* ctx, void* dev);
+/* Releases every pooled buffer to the driver. */
+int ft_pool_trim(ft_context* ctx);
+/* Bytes currently handed out / held idle by the pool. */
+int ft_pool_stats(ft_context* ctx, size_t* live_bytes, size_t* idle_bytes);
+/* UnifiedTensor::zeros (tensor.rs:213-217) on an existing buffer. */
+int ft_zero(ft_context* ctx, void* dev, size_t bytes);
+/* UnifiedTensor::write_data / new / from_bytes (tensor.rs:146-181, 220-255): host -> device. */
+int ft_upload(ft_context* ctx, void* dst_dev, const void* src_host, size_t bytes);
+/* UnifiedTensor::to_vec (tensor.rs:333-369): device -> host, waits for the copy. */
+int ft_download(ft_context* ctx, void* dst_host, const void* src_dev, size_t bytes);
+/* UnifiedTensor::from_f32_as_f16 (tensor.rs:258-269): rounds n f32 values to
+ * f16 (nearest even) and uploads them packed; dst holds 2*n bytes rounded up
+ * to a multiple of 4. */
+int ft_upload_f32_as_f16(ft_context* ctx, void* dst_dev, const float* src_host, size_t n);
+/* UnifiedTensor::from_f32_transposed (tensor.rs:385-406, 490-514): src is
+ * [rows, cols] row-major; dst receives [cols, rows] as FT_DTYPE_F32 or _F16. */
+int ft_upload_f32_transposed(ft_context* ctx, void* dst_dev, const float* src_host, size_t rows,
+                             size_t cols, int dtype);
+/* ComputeEngine::copy_tensor (engine/mod.rs:399-415): device -> device. */
+int ft_copy_tensor(ft_context* ctx, const void* src_dev, size_t bytes, void* dst_dev,
+                   size_t dst_byte_offset);
+
+/* ---- matrix products (engine/matmul.rs:94-156) --------------------------- */
+
+/* ComputeEngine::matmul: out[M,N] = a[M,K] @ b[K,N]. */
+int ft_matmul(ft_context* ctx, const float* a, const float* b, float* out, size_t M, size_t K, size_t N);
+/* ComputeEngine::matmul_bt: out[M,N] = a[M,K] @ b[N,K]^T. */
+int ft_matmul_bt(ft_context* ctx, const float* a, const float* b, float* out, size_t M, size_t K, size_t N);
+/* ComputeEngine::matmul_at: out[M,N] = a[K,M]^T @ b[K,N]. */
+int ft_matmul_at(ft_context* ctx, const float* a, const float* b, float* out, size_t M, size_t K, size_t N);
+/* ComputeEngine::matmul_f16b: matmul with b[K,N] stored as packed f16. */
+int ft_matmul_f16b(ft_context* ctx, const float* a, const uint16_t* b, float* out, size_t M, size_t K, size_t N);
+/* ComputeEngine::matmul_bt_f16b: matmul_bt with b[N,K] stored as packed f16. */
+int ft_matmul_bt_f16b(ft_context* ctx, const float* a, const uint16_t* b, float* out, size_t M, size_t K, size_t N);
+
+/* ---- LoRA linear, fused (replaces the 6 dispatches of Linear::project_2d,
+ *      ferrotensor-graph/src/lib.rs:112-126, and of its backward,
+ *      ferrotensor-autograd/src/lib.rs:262-290, 340-357) ---------------------- */
+
+/* t[M,r] = scale * (x[M,K] @ a[K,r]): the `x @ A` product with the alpha/rank
+ * scale applied where the reference applies it (graph/src/lib.rs:116-122).
+ * r <= 32. */
+int ft_lora_down(ft_context* ctx, const float* x, const float* a, float* t, size_t M, size_t K,
+                 size_t r, float scale);
+/* y[M,N] = x[M,K] @ w[K,N] + t[M,r] @ b[r,N]; w is f32 (w_dtype FT_DTYPE_F32)
+ * or packed f16. The rank-r product rides in the GEMM's K loop. */
+int ft_lora_linear(ft_context* ctx, const float* x, const void* w, int w_dtype, const float* t,
+                   const float* b, float* y, size_t M, size_t K, size_t N, size_t r);
+/* dt[M,r] = scale * (dy[M,N] @ b[r,N]^T): gradient of the scaled `x @ A`. */
+int ft_lora_grad_down(ft_context* ctx, const float* dy, const float* b, float* dt, size_t M,
+                      size_t N, size_t r, float scale);
+/* dx[M,K] = dy[M,N] @ w[K,N]^T + dt[M,r] @ a[K,r]^T (both MatMulNode input
+ * gradients and their AddNode sum in one GEMM). */
+int ft_lora_linear_dx(ft_context* ctx, const float* dy, const void* w, int w_dtype, const float* dt,
+                      const float* a, float* dx, size_t M, size_t K, size_t N, size_t r);
+/* db[r,N] = t[M,r]^T @ dy[M,N]  (matmul_at of the scaled x@A and dy). */
+int ft_lora_grad_b(ft_context* ctx, const float* t, const float* dy, float* db, size_t M, size_t N,
+                   size_t r);
+/* da[K,r] = x[M,K]^T @ dt[M,r]  (matmul_at of x and dt). */
+int ft_lora_grad_a(ft_context* ctx, const float* x, const float* dt, float* da, size_t M, size_t K,
+                   size_t r);
+
+/* ---- normalisation (engine/norm.rs:20-99) -------------------------------- */
+
+/* ComputeEngine::rms_norm_eps: out = x * rsqrt(mean(x^2) + eps) * w, rows x size. */
+int ft_rms_norm_eps(ft_context* ctx, const float* x, const float* w, float* out, size_t rows,
+                    size_t size, float eps);
+/* ComputeEngine::rms_norm_backward: gx (rows x size) and gw (size); gw may be
+ * NULL when the norm scale is frozen and nobody reads it. */
+int ft_rms_norm_backward(ft_context* ctx, const float* x, const float* w, const float* g, float* gx,
+                         float* gw, size_t rows, size_t size, float eps);
+
+/* ---- RoPE (engine/attention.rs:21-83) ------------------------------------ */
+
+/* ComputeEngine::rope_theta / rope_theta_inverse: in place on t[batch, seq,
+ * hidden]; token i of each row sits at position pos + i. */
+int ft_rope_theta(ft_context* ctx, float* t, size_t batch, size_t seq, size_t hidden, size_t head_dim,
+                  size_t pos, float theta);
+int ft_rope_theta_inverse(ft_context* ctx, float* t, size_t batch, size_t seq, size_t hidden,
+                          size_t head_dim, size_t pos, float theta);
+/* Out-of-place form (saves the copy RoPENode::backward and Tensor::rope_theta
+ * make first, autograd/src/lib.rs:509-533, 1122-1139). */
+int ft_rope_theta_to(ft_context* ctx, const float* src, float* dst, size_t batch, size_t seq,
+                     size_t hidden, size_t head_dim, size_t pos, float theta, int inverse);
+
+/* ---- attention (engine/attention.rs:165-177, 341-358, 581-594) ----------- */
+
+/* AttentionOptions. window and dropout are not supported (0 only): the model
+ * builder refuses windows (model_builder.rs:212-221) and every SmolLM2 config
+ * has attention_dropout 0. */
+typedef struct ft_attention_options {
+    int32_t causal;
+    uint32_t causal_offset;
+    uint32_t window;
+    float dropout_prob;
+    uint64_t seed;
+} ft_attention_options;
+
+/* ComputeEngine::flash_attention_v2_with_stats. q/out [B,Sq,H,D], k/v
+ * [B,Sk,Hkv,D], stats [B*H*Sq, 2] (slot 2*row+1 receives the row's
+ * log-sum-exp, row = (b*H+h)*Sq+i); stats may be NULL. D <= 128. */
+int ft_flash_attention_v2_with_stats(ft_context* ctx, const float* q, const float* k, const float* v,
+                                     float* out, float* stats, size_t B, size_t Sq, size_t Sk,
+                                     size_t H, size_t Hkv, size_t D, const ft_attention_options* opts);
+/* ComputeEngine::flash_attention_v2_backward_with_stats: reads the saved
+ * log-sum-exp, overwrites slot 2*row with Delta = dO.O, writes dq, dk, dv. */
+int ft_flash_attention_v2_backward_with_stats(ft_context* ctx, const float* q, const float* k,
+                                              const float* v, const float* out, const float* d_out,
+                                              float* dq, float* dk, float* dv, float* stats, size_t B,
+                                              size_t Sq, size_t Sk, size_t H, size_t Hkv, size_t D,
+                                              const ft_attention_options* opts);
+
+/* ---- elementwise (engine/elementwise.rs:8-17, 57-75, 183-216) ------------ */
+
+/* ComputeEngine::add: out = a + b. */
+int ft_add(ft_context* ctx, const float* a, const float* b, float* out, size_t n);
+/* ComputeEngine::add_backward: ga = gb = g. */
+int ft_add_backward(ft_context* ctx, const float* g, float* ga, float* gb, size_t n);
+/* ComputeEngine::silu_gate_fused(first, second, out): out = silu(first) * second. */
+int ft_silu_gate_fused(ft_context* ctx, const float* first, const float* second, float* out, size_t n);
+/* ComputeEngine::silu_gate_backward(first, second, g, g_first, g_second). */
+int ft_silu_gate_backward(ft_context* ctx, const float* first, const float* second, const float* g,
+                          float* g_first, float* g_second, size_t n);
+
+/* ---- training (engine/training.rs:54-76, 161-283) ------------------------ */
+
+/* ComputeEngine::gradient_scale / clip_grad_by_norm: x *= scale, in place. */
+int ft_gradient_scale(ft_context* ctx, float* x, size_t n, float scale);
+int ft_clip_grad_by_norm(ft_context* ctx, float* x, size_t n, float scale);
+/* ComputeEngine::gradient_accumulate: acc += g. */
+int ft_gradient_accumulate(ft_context* ctx, float* acc, const float* g, size_t n);
+/* ComputeEngine::sum_squares_partial: sum of x^2 per FT_SUM_SQUARES_CHUNK
+ * elements into out[offset + b]; *chunks receives the number written. */
+int ft_sum_squares_partial(ft_context* ctx, const float* x, size_t n, float* out, size_t offset,
+                           size_t* chunks);
+/* ComputeEngine::masked_cross_entropy_weighted: logits/grad [rows, vocab],
+ * targets u32 [rows] (FT_MASKED_CE_SKIP = outside the loss), weights f32
+ * [rows], row_loss [rows]. `grad_scale` multiplies the gradient (1.0 gives
+ * the reference kernel; 1/grad_accum_steps folds the copy + gradient_scale of
+ * MaskedCrossEntropyNode::backward, ferrotensor-trainer/src/lib.rs:553-572).
+ * grad may alias logits. */
+int ft_masked_cross_entropy_weighted(ft_context* ctx, const float* logits, const uint32_t* targets,
+                                     const float* weights, float* grad, float* row_loss, size_t rows,
+                                     size_t vocab, float grad_scale);
+
+/* AdamParams (engine/training.rs:13-32). */
+typedef struct ft_adam_params {
+    float lr, beta1, beta2, eps, weight_decay, t;
+} ft_adam_params;
+/* ComputeEngine::adamw_update on one tensor. */
+int ft_adamw_update(ft_context* ctx, float* w, const float* g, float* m, float* v, size_t n,
+                    const ft_adam_params* p);
+/* AdamW::apply_step over a list of tensors in one launch
+ * (ferrotensor-autograd/src/lib.rs:1522-1552 issues one dispatch per tensor).
+ * The four arrays hold `count` device pointers each (host memory), sizes the
+ * element counts. `grad_scale` multiplies every gradient first (the clip scale
+ * of Trainer::apply_gradients, trainer/src/lib.rs:336-343; 1.0 = none). */
+int ft_adamw_update_multi(ft_context* ctx, float* const* w, const float* const* g, float* const* m,
+                          float* const* v, const size_t* sizes, size_t count, const ft_adam_params* p,
+                          float grad_scale);
+
+/* ---- embedding gather (Tensor::embedding, autograd/src/lib.rs:1159-1179;
+ *      done on the host in the reference) ------------------------------------ */
+
+/* out[n, hidden] = table[ids[i]] or a zero row when ids[i] >= vocab. */
+int ft_embedding(ft_context* ctx, const float* table, size_t vocab, size_t hidden, const uint32_t* ids,
+                 size_t n, float* out);
+
+/* ---- the step driver: Lfm2Model + Trainer over the ops above ------------- */
+
+/* Lfm2Config fields the step uses (ferrotensor-loader/src/lib.rs:74-142). */
+typedef struct ft_model_config {
+    uint32_t vocab_size, hidden_size, intermediate_size, num_hidden_layers;
+    uint32_t num_attention_heads, num_key_value_heads;
+    float rms_norm_eps, rope_theta;
+    int32_t tie_word_embeddings;
+    int32_t f16_linears;   /* frozen linear weights stored as f16 (CLI default, main.rs:230-234) */
+} ft_model_config;
+
+typedef struct ft_model ft_model;
+typedef struct ft_trainer ft_trainer;
+
+/* Lfm2ModelBuilder::build (model_builder.rs:623-709): an empty model; weights
+ * arrive through ft_model_set_tensor. */
+int ft_model_create(ft_context* ctx, const ft_model_config* cfg, ft_model** out);
+int ft_model_destroy(ft_model* m);
+/* Uploads one Hugging Face tensor by name (`model.embed_tokens.weight`,
+ * `model.layers.N.self_attn.q_proj.weight` [out,in], `...input_layernorm.weight`,
+ * `model.norm.weight`, `lm_head.weight`), applying the builder's rules
+ * (model_builder.rs:400-424, 653-689): linears are transposed to [in,out] and
+ * rounded to f16 when cfg.f16_linears; a tied head is the transposed embedding. */
+int ft_model_set_tensor(ft_model* m, const char* hf_name, const float* data, const size_t* shape, int ndim);
+/* Attaches a LoRA adapter (LoRAAdapter, graph/src/lib.rs:28-98) to the linear
+ * named `prefix` (`model.layers.N.self_attn.q_proj`, `lm_head`, ...):
+ * a [in, rank], b [rank, out], both copied. */
+int ft_model_set_lora(ft_model* m, const char* prefix, const float* a, const float* b, size_t rank, float alpha);
+/* Number of trainable tensors and their fixture names / sizes, in the order
+ * gradients and parameters are reported (`<prefix>.lora_a`, `<prefix>.lora_b`). */
+int ft_model_param_count(ft_model* m, size_t* count);
+int ft_model_param_info(ft_model* m, size_t index, const char** name, size_t* numel);
+/* Copies parameter / gradient `index` to the host (numel f32 values). The
+ * gradient is the one the last step left (scaled by 1/grad_accum, unclipped). */
+int ft_model_read_param(ft_model* m, size_t index, float* out_host);
+int ft_model_read_grad(ft_model* m, size_t index, float* out_host);
+/* Lfm2Model::forward_batch (lfm.rs:590-623): logits [B*S, vocab] to the host. */
+int ft_model_forward_logits(ft_model* m, const uint32_t* rows, size_t B, size_t S, float* logits_host);
+
+/* Trainer::new + with_clip_grad_norm (trainer/src/lib.rs:113-205) with an
+ * AdamW (autograd/src/lib.rs:1502-1515). clip_grad_norm <= 0 disables
+ * clipping. */
+typedef struct ft_trainer_config {
+    float lr, beta1, beta2, eps, weight_decay;
+    float clip_grad_norm;
+    uint32_t grad_accum_steps;   /* 0 = the chunk's number of sequences */
+} ft_trainer_config;
+
+/* StepStats of a chunk (trainer/src/lib.rs:36-58). */
+typedef struct ft_step_stats {
+    float loss;            /* sum of the per-sequence mean losses */
+    float grad_norm;
+    float clip_scale;      /* 1.0 when not clipped */
+    uint32_t supervised_tokens;
+    int32_t optimizer_step;
+} ft_step_stats;
+
+int ft_trainer_create(ft_model* m, const ft_trainer_config* cfg, ft_trainer** out);
+int ft_trainer_destroy(ft_trainer* t);
+/* Trainer::train_chunk (trainer/src/lib.rs:426-502) for B equally long rows
+ * (already padded; see ft_pad_chunk): forward, masked cross-entropy, backward
+ * with seed 1/grad_accum_steps, gradient norm, clip, AdamW. rows/targets are
+ * [B,S] u32 and loss_mask [B,S] u8 in host memory; per_sequence_loss (B
+ * values) may be NULL. `apply` = 0 stops after backward (gradients readable,
+ * no optimizer step). */
+int ft_trainer_train_chunk(ft_trainer* t, const uint32_t* rows, const uint32_t* targets,
+                           const uint8_t* loss_mask, size_t B, size_t S, int apply,
+                           ft_step_stats* stats, float* per_sequence_loss);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FERROTENSOR_HIP_H */

@@ -1,0 +1,341 @@
+"""HIP kernels against the CPU oracle, through the C ABI.
+
+Follows ferrotensor-backend/tests/gpu_kernels.rs: every kernel on seeded
+inputs at the reference's shapes (MATMUL_SHAPES :234-246, SMOLLM2_PROJECTIONS
+:966-982, row kernels, masked CE, AdamW), compared with the oracle within
+|a-e| <= 1e-4 + 1e-3*|e| (f32) and bit-exactly for integer/index work.
+"""
+import numpy as np
+import pytest
+
+from oracle import cpu
+from oracle import reference_step as rs
+from tests.gpu_util import assert_close, make_ctx
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def g():
+    ctx, eng = make_ctx()
+    yield ctx, eng
+    ctx.close()
+
+
+def rnd(seed, *shape, scale=1.0):
+    return (np.random.default_rng(seed).standard_normal(shape) * scale).astype(np.float32)
+
+
+def up(ctx, x):
+    from ferrotensor_amd import UnifiedTensor
+    return UnifiedTensor.new(ctx, x, list(x.shape))
+
+
+def empty(ctx, *shape):
+    from ferrotensor_amd import UnifiedTensor
+    return UnifiedTensor.empty(ctx, list(shape))
+
+
+MATMUL_SHAPES = [(1, 1, 1), (1, 7, 1), (3, 5, 7), (16, 16, 16), (17, 33, 9), (64, 64, 64), (65, 1, 130),
+                 (127, 129, 65), (1, 512, 300), (300, 512, 1), (256, 384, 128), (130, 70, 200), (256, 96, 320)]
+
+# GEMM tolerance of the reference's f64 comparisons (gpu_kernels.rs:989-1084): 1e-3 + 1e-4*|want|
+# for N(0,1) operands; the oracle itself adds in f32, so compare against f64 here.
+
+
+def f64_mm(a, b):
+    return a.astype(np.float64) @ b.astype(np.float64)
+
+
+@pytest.mark.parametrize("M,K,N", MATMUL_SHAPES)
+def test_matmul_layouts_match_cpu(g, M, K, N):
+    ctx, eng = g
+    a, b = rnd(M * 7 + K, M, K), rnd(N * 3 + K, K, N)
+    want = f64_mm(a, b)
+    out = empty(ctx, M, N)
+    eng.matmul(ctx, up(ctx, a), up(ctx, b), out)
+    assert_close(f"matmul {M}x{K}x{N}", out.to_numpy(), want, atol=1e-3, rtol=1e-4)
+    out = empty(ctx, M, N)
+    eng.matmul_bt(ctx, up(ctx, a), up(ctx, np.ascontiguousarray(b.T)), out)
+    assert_close(f"matmul_bt {M}x{K}x{N}", out.to_numpy(), want, atol=1e-3, rtol=1e-4)
+    out = empty(ctx, M, N)
+    eng.matmul_at(ctx, up(ctx, np.ascontiguousarray(a.T)), up(ctx, b), out)
+    assert_close(f"matmul_at {M}x{K}x{N}", out.to_numpy(), want, atol=1e-3, rtol=1e-4)
+    # and against the oracle's own f32 product
+    assert_close(f"matmul vs oracle {M}x{K}x{N}", out.to_numpy(), cpu.matmul(a, b), atol=1e-3, rtol=1e-4)
+
+
+SMOLLM2_PROJECTIONS = [("135M q/o", 576, 576), ("135M k/v", 576, 192), ("135M gate/up", 576, 1536),
+                       ("135M down", 1536, 576), ("360M q/o", 960, 960), ("360M k/v", 960, 320),
+                       ("360M gate/up", 960, 2560), ("360M down", 2560, 960), ("1.7B q/k/v/o", 2048, 2048)]
+
+
+@pytest.mark.parametrize("name,K,N", SMOLLM2_PROJECTIONS)
+@pytest.mark.parametrize("M", [31, 256])
+def test_f16_weight_projections(g, name, K, N, M):
+    from ferrotensor_amd import UnifiedTensor
+    ctx, eng = g
+    a, w = rnd(K + N, M, K), rnd(K * 2 + N, K, N, scale=0.05)
+    w16 = UnifiedTensor.from_f32_as_f16(ctx, w, [K, N])
+    wr = cpu.round_f16(w)
+    out = empty(ctx, M, N)
+    eng.matmul_f16b(ctx, up(ctx, a), w16, out)
+    assert_close(f"{name} matmul_f16b", out.to_numpy(), f64_mm(a, wr), atol=1e-3, rtol=1e-4)
+    # input gradient: g[M,N] @ w[K,N]^T
+    gy = rnd(7, M, N)
+    dx = empty(ctx, M, K)
+    eng.matmul_bt_f16b(ctx, up(ctx, gy), w16, dx)
+    assert_close(f"{name} matmul_bt_f16b", dx.to_numpy(), f64_mm(gy, wr.T), atol=2e-3, rtol=1e-4)
+
+
+def test_f16_upload_is_bit_exact(g):
+    from ferrotensor_amd import DType, UnifiedTensor
+    ctx, _ = g
+    x = np.concatenate([rnd(1, 4097), rnd(2, 100) * 1e-6, rnd(3, 100) * 1e5,
+                        np.array([0.0, -0.0, 65504.0, 65520.0, 1e9, 5.9604645e-08, 2.9802322e-08], np.float32)])
+    t = UnifiedTensor.from_f32_as_f16(ctx, x, [x.size])
+    got = t.to_vec(ctx, np.uint16)
+    np.testing.assert_array_equal(got, cpu.pack_f16(x))
+    m = rnd(4, 37, 53)
+    tt = UnifiedTensor.from_f32_transposed(ctx, m, 37, 53, DType.FP16)
+    assert tt.shape == [53, 37]
+    np.testing.assert_array_equal(tt.to_vec(ctx, np.uint16), cpu.pack_f16(np.ascontiguousarray(m.T)).reshape(-1))
+    tf = UnifiedTensor.from_f32_transposed(ctx, m, 37, 53, DType.FP32)
+    np.testing.assert_array_equal(tf.to_numpy(), m.T)
+
+
+@pytest.mark.parametrize("M,K,N,r", [(64, 32, 48, 4), (256, 576, 1536, 8), (100, 960, 320, 8), (96, 64, 40, 16)])
+@pytest.mark.parametrize("f16", [False, True])
+def test_fused_lora_linear_forward_and_backward(g, M, K, N, r, f16):
+    """Linear::project_2d and its backward (graph/src/lib.rs:112-126; autograd MatMulNode/ScaleNode)."""
+    from ferrotensor_amd import UnifiedTensor
+    ctx, eng = g
+    x, w = rnd(1, M, K), rnd(2, K, N, scale=0.05)
+    A, B = rnd(3, K, r, scale=0.1), rnd(4, r, N, scale=0.1)
+    dy = rnd(5, M, N)
+    s = 2.0
+    wr = cpu.round_f16(w) if f16 else w
+    lin = rs.Linear(weight=wr, lora_a=A, lora_b=B, alpha=s * r, rank=r)
+    cache, grads = {}, {}
+    want_y = lin.forward(x, cache)
+    want_dx = lin.backward(dy, cache, True, False, grads, "l")
+
+    wt = UnifiedTensor.from_f32_as_f16(ctx, w, [K, N]) if f16 else up(ctx, w)
+    xt, At, Bt, dyt = up(ctx, x), up(ctx, A), up(ctx, B), up(ctx, dy)
+    t = empty(ctx, M, r)
+    eng.lora_down(ctx, xt, At, t, s)
+    assert_close("x@A*s", t.to_numpy(), cache["temp"], atol=1e-3, rtol=1e-4)
+    y = empty(ctx, M, N)
+    eng.lora_linear(ctx, xt, wt, t, Bt, y)
+    assert_close("lora_linear", y.to_numpy(), want_y, atol=1e-3, rtol=1e-4)
+    dt = empty(ctx, M, r)
+    eng.lora_grad_down(ctx, dyt, Bt, dt, s)
+    dx = empty(ctx, M, K)
+    eng.lora_linear_dx(ctx, dyt, wt, dt, At, dx)
+    assert_close("lora_linear_dx", dx.to_numpy(), want_dx, atol=2e-3, rtol=1e-4)
+    db, da = empty(ctx, r, N), empty(ctx, K, r)
+    eng.lora_grad_b(ctx, t, dyt, db)
+    eng.lora_grad_a(ctx, xt, dt, da)
+    assert_close("dB", db.to_numpy(), grads["l.lora_b"], atol=2e-3, rtol=1e-4)
+    assert_close("dA", da.to_numpy(), grads["l.lora_a"], atol=2e-3, rtol=1e-4)
+
+
+@pytest.mark.parametrize("rows,size", [(1, 1), (3, 7), (37, 96), (16, 576), (64, 960), (5, 2048), (3, 2100)])
+def test_rms_norm_forward_backward(g, rows, size):
+    ctx, eng = g
+    x, w, gy = rnd(1, rows, size), rnd(2, size), rnd(3, rows, size)
+    eps = 1e-5
+    out = empty(ctx, rows, size)
+    eng.rms_norm_eps(ctx, up(ctx, x), up(ctx, w), out, eps)
+    assert_close("rms_norm", out.to_numpy(), cpu.rms_norm(x, w, eps))
+    gx, gw = empty(ctx, rows, size), empty(ctx, size)
+    eng.rms_norm_backward(ctx, up(ctx, x), up(ctx, w), up(ctx, gy), gx, gw, eps)
+    want_gx, want_gw = cpu.rms_norm_backward(x, w, gy, eps)
+    assert_close("rms gx", gx.to_numpy(), want_gx)
+    assert_close("rms gw", gw.to_numpy(), want_gw, atol=2e-4)
+    gx2 = empty(ctx, rows, size)
+    eng.rms_norm_backward(ctx, up(ctx, x), up(ctx, w), up(ctx, gy), gx2, None, eps)
+    np.testing.assert_array_equal(gx2.to_numpy(), gx.to_numpy())
+
+
+@pytest.mark.parametrize("B,S,heads,D,pos,theta", [(1, 1, 1, 2, 0, 10000.0), (2, 9, 3, 8, 5, 10000.0),
+                                                  (2, 256, 9, 64, 0, 100000.0), (1, 64, 4, 64, 960, 500.0)])
+def test_rope_forward_and_inverse(g, B, S, heads, D, pos, theta):
+    ctx, eng = g
+    x = rnd(11, B, S, heads * D)
+    t = up(ctx, x)
+    eng.rope_theta(ctx, t, D, pos, theta)
+    want = cpu.rope(x, D, pos, theta)
+    assert_close("rope", t.to_numpy(), want)
+    eng.rope_theta_inverse(ctx, t, D, pos, theta)
+    assert_close("rope inverse", t.to_numpy(), x)
+
+
+@pytest.mark.parametrize("n", [1, 5, 64, 1000, 4096 * 3 + 1])
+def test_elementwise(g, n):
+    ctx, eng = g
+    a, b, gy = rnd(1, n, scale=3.0), rnd(2, n), rnd(3, n)
+    out = empty(ctx, n)
+    eng.add(ctx, up(ctx, a), up(ctx, b), out)
+    np.testing.assert_array_equal(out.to_numpy(), a + b)
+    ga, gb = empty(ctx, n), empty(ctx, n)
+    eng.add_backward(ctx, up(ctx, gy), ga, gb)
+    np.testing.assert_array_equal(ga.to_numpy(), gy)
+    np.testing.assert_array_equal(gb.to_numpy(), gy)
+    eng.silu_gate_fused(ctx, up(ctx, a), up(ctx, b), out)
+    assert_close("silu_gate", out.to_numpy(), cpu.silu_gate(a, b))
+    eng.silu_gate_backward(ctx, up(ctx, a), up(ctx, b), up(ctx, gy), ga, gb)
+    wa, wb = cpu.silu_gate_backward(a, b, gy)
+    assert_close("silu ga", ga.to_numpy(), wa)
+    assert_close("silu gb", gb.to_numpy(), wb)
+    t = up(ctx, a)
+    eng.gradient_scale(ctx, t, 0.37)
+    np.testing.assert_array_equal(t.to_numpy(), a * np.float32(0.37))
+    eng.gradient_accumulate(ctx, t, up(ctx, b))
+    np.testing.assert_array_equal(t.to_numpy(), a * np.float32(0.37) + b)
+
+
+def test_embedding_gather_bit_exact(g):
+    from ferrotensor_amd import UnifiedTensor
+    ctx, eng = g
+    table = rnd(5, 50, 24)
+    ids = np.array([0, 49, 7, 50, 4000000000, 3], np.uint32)
+    out = empty(ctx, ids.size, 24)
+    eng.embedding(ctx, up(ctx, table), UnifiedTensor.from_bytes(ctx, ids, [ids.size]), out)
+    np.testing.assert_array_equal(out.to_numpy(), cpu.embedding(table, ids))
+
+
+@pytest.mark.parametrize("rows,vocab", [(4, 7), (12, 50), (9, 4096), (5, 16384 + 4), (3, 49152), (2, 50000)])
+def test_masked_cross_entropy(g, rows, vocab):
+    from ferrotensor_amd import UnifiedTensor
+    ctx, eng = g
+    rng = np.random.default_rng(rows * vocab)
+    logits = rnd(3, rows, vocab, scale=4.0)
+    targets = rng.integers(0, vocab, rows).astype(np.uint32)
+    targets[rows // 2] = rs.MASKED_CE_SKIP
+    weights = rng.random(rows).astype(np.float32)
+    want_g, want_l = cpu.masked_cross_entropy(logits, targets, weights)
+    grad, row_loss = empty(ctx, rows, vocab), empty(ctx, rows)
+    tl = up(ctx, logits)
+    tt = UnifiedTensor.from_bytes(ctx, targets, [rows])
+    eng.masked_cross_entropy_weighted(ctx, tl, tt, up(ctx, weights), grad, row_loss)
+    assert_close("ce loss", row_loss.to_numpy(), want_l)
+    assert_close("ce grad", grad.to_numpy(), want_g, atol=1e-6)
+    skipped = targets == rs.MASKED_CE_SKIP
+    assert (grad.to_numpy()[skipped] == 0).all() and (row_loss.to_numpy()[skipped] == 0).all()
+    # in place, with the upstream scale folded in
+    eng.masked_cross_entropy_weighted(ctx, tl, tt, up(ctx, weights), tl, row_loss, grad_scale=0.125)
+    assert_close("ce grad in place", tl.to_numpy(), want_g * np.float32(0.125), atol=1e-6)
+
+
+def test_sum_squares_and_adamw(g):
+    ctx, eng = g
+    from ferrotensor_amd import AdamParams, UnifiedTensor
+    x = rnd(9, 4096 * 2 + 100)
+    out = UnifiedTensor.zeros(ctx, [8])
+    n = eng.sum_squares_partial(ctx, up(ctx, x), out, 3)
+    want = np.zeros(8, np.float32)
+    assert n == cpu.sum_squares_partial(x, want, 3) == 3
+    assert_close("sum squares", out.to_numpy(), want, atol=1e-3)
+
+    n = 4096 * 5 + 17
+    w0, gr = rnd(1, n), rnd(2, n)
+    m0, v0 = rnd(3, n, scale=0.1), np.abs(rnd(4, n, scale=0.1))
+    for wd, t in [(0.0, 1.0), (0.01, 7.0)]:
+        p = AdamParams(lr=1e-3, weight_decay=wd, t=t)
+        w, m, v = w0.copy(), m0.copy(), v0.copy()
+        cpu.adamw_update(w, gr, m, v, p.lr, p.beta1, p.beta2, p.eps, p.weight_decay, p.t)
+        tw, tm, tv = up(ctx, w0), up(ctx, m0), up(ctx, v0)
+        eng.adamw_update(ctx, tw, up(ctx, gr), tm, tv, p)
+        assert_close("adamw w", tw.to_numpy(), w, atol=1e-6, rtol=1e-5)
+        assert_close("adamw m", tm.to_numpy(), m, atol=1e-7, rtol=1e-5)
+        assert_close("adamw v", tv.to_numpy(), v, atol=1e-7, rtol=1e-5)
+        # multi-tensor launch over uneven pieces gives the same numbers
+        cuts = [0, 100, 4096 + 100, n]
+        parts = lambda a: [up(ctx, a[cuts[i]:cuts[i + 1]]) for i in range(3)]
+        ws, gs, ms, vs = parts(w0), parts(gr), parts(m0), parts(v0)
+        eng.adamw_update_multi(ctx, ws, gs, ms, vs, p)
+        got = np.concatenate([t_.to_numpy() for t_ in ws])
+        np.testing.assert_array_equal(got, tw.to_numpy())
+
+
+def test_errors_are_reported_not_fatal(g):
+    from ferrotensor_amd import FtError
+    ctx, eng = g
+    x = up(ctx, rnd(1, 4, 6))
+    with pytest.raises(FtError):
+        eng.rope_theta(ctx, x, 4, 0, 10000.0)  # hidden 6 is not a multiple of head_dim 4
+    with pytest.raises(FtError):
+        eng.lora_down(ctx, x, up(ctx, rnd(2, 6, 40)), empty(ctx, 4, 40), 1.0)  # rank > 32
+
+
+# ---- attention (gpu_kernels.rs cpu_attention :132-179, cpu_attention_backward :183-224) ----
+
+ATTN_CASES = [
+    # B, Sq, Sk, H, Hkv, D, causal, offset
+    (1, 1, 1, 1, 1, 8, True, 0),
+    (2, 16, 16, 4, 2, 8, True, 0),          # tiny config of the gradient fixture
+    (2, 13, 13, 4, 2, 8, True, 0),
+    (1, 40, 40, 6, 6, 16, True, 0),
+    (2, 17, 17, 3, 1, 64, False, 0),
+    (1, 100, 100, 2, 2, 64, True, 0),
+    (2, 256, 256, 9, 3, 64, True, 0),       # SmolLM2-135M heads at seq 256
+    (1, 70, 70, 2, 1, 128, True, 0),
+    (1, 33, 65, 2, 1, 32, True, 32),        # queries at positions 32.. against a longer key run
+    (1, 5, 37, 4, 4, 24, False, 0),
+]
+
+
+@pytest.mark.parametrize("B,Sq,Sk,H,Hkv,D,causal,offset", ATTN_CASES)
+def test_flash_attention_forward_backward(g, B, Sq, Sk, H, Hkv, D, causal, offset):
+    from ferrotensor_amd import AttentionOptions, UnifiedTensor
+    ctx, eng = g
+    q, k, v = rnd(1, B, Sq, H, D), rnd(2, B, Sk, Hkv, D), rnd(3, B, Sk, Hkv, D)
+    do = rnd(4, B, Sq, H, D)
+    want_o, want_lse = cpu.attention(q, k, v, causal=causal, causal_offset=offset)
+    want_dq, want_dk, want_dv = cpu.attention_backward(q, k, v, want_o, do, causal=causal, causal_offset=offset)
+    opts = AttentionOptions(causal=causal, causal_offset=offset)
+    tq, tk, tv, tdo = up(ctx, q), up(ctx, k), up(ctx, v), up(ctx, do)
+    out = empty(ctx, B, Sq, H, D)
+    stats = UnifiedTensor.zeros(ctx, [B, H, Sq, 2])
+    eng.flash_attention_v2_with_stats(ctx, tq, tk, tv, out, stats, opts)
+    assert_close("attention out", out.to_numpy(), want_o)
+    assert_close("attention lse", stats.to_numpy()[..., 1], want_lse)
+    dq, dk, dv = empty(ctx, B, Sq, H, D), empty(ctx, B, Sk, Hkv, D), empty(ctx, B, Sk, Hkv, D)
+    eng.flash_attention_v2_backward_with_stats(ctx, tq, tk, tv, out, tdo, dq, dk, dv, stats, opts)
+    delta = (do.astype(np.float64) * want_o.astype(np.float64)).sum(-1).transpose(0, 2, 1)
+    assert_close("attention delta", stats.to_numpy()[..., 0], delta, atol=1e-3)
+    assert_close("dq", dq.to_numpy(), want_dq, atol=2e-4)
+    assert_close("dk", dk.to_numpy(), want_dk, atol=2e-4)
+    assert_close("dv", dv.to_numpy(), want_dv, atol=2e-4)
+    # forward without stats gives the same output
+    out2 = empty(ctx, B, Sq, H, D)
+    eng.flash_attention_v2_with(ctx, tq, tk, tv, out2, opts)
+    np.testing.assert_array_equal(out2.to_numpy(), out.to_numpy())
+
+
+def test_attention_causality_is_bit_exact(g):
+    """Changing later tokens leaves earlier outputs untouched (model_correctness.rs:281-300)."""
+    from ferrotensor_amd import AttentionOptions
+    ctx, eng = g
+    q, k, v = rnd(1, 1, 96, 3, 64), rnd(2, 1, 96, 1, 64), rnd(3, 1, 96, 1, 64)
+    opts = AttentionOptions(causal=True)
+    a = empty(ctx, 1, 96, 3, 64)
+    eng.flash_attention_v2_with(ctx, up(ctx, q), up(ctx, k), up(ctx, v), a, opts)
+    k2, v2 = k.copy(), v.copy()
+    k2[:, 64:], v2[:, 64:] = rnd(5, 1, 32, 1, 64), rnd(6, 1, 32, 1, 64)
+    b = empty(ctx, 1, 96, 3, 64)
+    eng.flash_attention_v2_with(ctx, up(ctx, q), up(ctx, k2), up(ctx, v2), b, opts)
+    np.testing.assert_array_equal(a.to_numpy()[:, :64], b.to_numpy()[:, :64])
+
+
+def test_attention_rejects_unsupported_options(g):
+    from ferrotensor_amd import AttentionOptions, FtError
+    ctx, eng = g
+    q = up(ctx, rnd(1, 1, 4, 2, 8))
+    k = up(ctx, rnd(2, 1, 4, 1, 8))
+    out = empty(ctx, 1, 4, 2, 8)
+    with pytest.raises(FtError):
+        eng.flash_attention_v2_with(ctx, q, k, k, out, AttentionOptions(causal=True, window=2))
+    with pytest.raises(FtError):
+        eng.flash_attention_v2_with(ctx, q, k, k, out, AttentionOptions(causal=True, dropout_prob=0.1))
