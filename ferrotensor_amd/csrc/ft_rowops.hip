@@ -326,7 +326,9 @@ __global__ __launch_bounds__(256) void rope_kernel(const float* __restrict__ src
 }
 
 // ---------------------------------------------------------------------------
-// Masked softmax-cross-entropy. One 1024-thread workgroup per row. A row of up
+// Masked softmax-cross-entropy. One 1024-thread workgroup per row. grad may
+// alias logits (no __restrict__ on either), so the target logit is loaded
+// before the barrier that precedes the gradient stores. A row of up
 // to 1024*4*CACHE floats is held in registers between the reduction and the
 // gradient write, so logits are read once and the gradient written once.
 // ---------------------------------------------------------------------------
@@ -335,7 +337,7 @@ constexpr int kCeThreads = 1024;
 
 template <int CACHE>  // float4 per thread kept in registers (0 = stream from memory)
 __global__ __launch_bounds__(kCeThreads) void masked_ce_kernel(
-    const float* __restrict__ logits, const uint32_t* __restrict__ targets, const float* __restrict__ weights,
+    const float* logits, const uint32_t* __restrict__ targets, const float* __restrict__ weights,
     float* grad, float* __restrict__ row_loss, size_t rows, size_t vocab, float grad_scale) {
     __shared__ float red[kCeThreads / kWave];
     const size_t row = blockIdx.x;
@@ -417,7 +419,7 @@ __global__ __launch_bounds__(kCeThreads) void masked_ce_kernel(
 
 // Scalar variant for rows that are not 16-byte aligned (vocab % 4 != 0).
 __global__ __launch_bounds__(256) void masked_ce_scalar_kernel(
-    const float* __restrict__ logits, const uint32_t* __restrict__ targets, const float* __restrict__ weights,
+    const float* logits, const uint32_t* __restrict__ targets, const float* __restrict__ weights,
     float* grad, float* __restrict__ row_loss, size_t rows, size_t vocab, float grad_scale) {
     __shared__ float red[4];
     const size_t row = blockIdx.x;

@@ -1,15 +1,706 @@
+// Host driver of one LoRA training step over the kernels of this library: the
+// part of the reference that sits above ComputeEngine on the hot path.
+//
+//   model     Lfm2Model / Lfm2Block / Attention / MLP / Linear(+LoRAAdapter)
+//             ferrotensor-graph/src/lfm.rs:116-139, 597-623;
+//             ferrotensor-graph/src/lib.rs:112-142, 367-414, 504-510
+//   builder   transpose [out,in] -> [in,out], f16 storage, tied head
+//             ferrotensor-graph/src/model_builder.rs:400-424, 653-689
+//   loss      masked_cross_entropy_batch, ferrotensor-trainer/src/lib.rs:676-752
+//   backward  the node rules of ferrotensor-autograd/src/lib.rs (MatMulNode
+//             :262-290, AddNode, ScaleNode, RoPENode :509-533, RMSNormNode
+//             :575-595, SiLUGateNode, FlashAttentionNode :1328-1390)
+//   step      Trainer::train_chunk / apply_gradients / global_grad_norm,
+//             trainer/src/lib.rs:296-360, 426-534; AdamW::apply_step,
+//             autograd/src/lib.rs:1522-1552
+//
+// The reference records a tape and walks it; the step's graph is static, so
+// forward and backward are written out here and every buffer is allocated once
+// per (batch, sequence) shape and kept. Nothing in the step waits for the GPU
+// until the per-row losses and the gradient norm are read back at its end.
 #include "ft_common.h"
-extern "C" {
-int ft_model_create(ft_context*, const ft_model_config*, ft_model**) { return ft_set_error(FT_ERR_INVALID, "not implemented"); }
-int ft_model_destroy(ft_model*) { return FT_OK; }
-int ft_model_set_tensor(ft_model*, const char*, const float*, const size_t*, int) { return ft_set_error(FT_ERR_INVALID, "not implemented"); }
-int ft_model_set_lora(ft_model*, const char*, const float*, const float*, size_t, float) { return ft_set_error(FT_ERR_INVALID, "not implemented"); }
-int ft_model_param_count(ft_model*, size_t*) { return ft_set_error(FT_ERR_INVALID, "not implemented"); }
-int ft_model_param_info(ft_model*, size_t, const char**, size_t*) { return ft_set_error(FT_ERR_INVALID, "not implemented"); }
-int ft_model_read_param(ft_model*, size_t, float*) { return ft_set_error(FT_ERR_INVALID, "not implemented"); }
-int ft_model_read_grad(ft_model*, size_t, float*) { return ft_set_error(FT_ERR_INVALID, "not implemented"); }
-int ft_model_forward_logits(ft_model*, const uint32_t*, size_t, size_t, float*) { return ft_set_error(FT_ERR_INVALID, "not implemented"); }
-int ft_trainer_create(ft_model*, const ft_trainer_config*, ft_trainer**) { return ft_set_error(FT_ERR_INVALID, "not implemented"); }
-int ft_trainer_destroy(ft_trainer*) { return FT_OK; }
-int ft_trainer_train_chunk(ft_trainer*, const uint32_t*, const uint32_t*, const uint8_t*, size_t, size_t, int, ft_step_stats*, float*) { return ft_set_error(FT_ERR_INVALID, "not implemented"); }
+
+#include <cmath>
+#include <cstring>
+#include <memory>
+#include <string>
+
+// Defined in ft_rowops.hip.
+struct ft_segment {
+    float* w;
+    float* g;
+    float* m;
+    float* v;
+    uint32_t n;
+};
+int ft_internal_multi_grad_norm(ft_context* ctx, const ft_segment* segs_dev, size_t nseg, float* partials_dev,
+                                float max_norm, float* control_dev);
+int ft_internal_multi_adamw(ft_context* ctx, const ft_segment* segs_dev, size_t nseg, const ft_adam_params* p,
+                            float grad_scale, const float* control_dev);
+
+namespace {
+
+constexpr float kF32Epsilon = 1.1920929e-07f;
+
+struct LinearW {
+    std::string prefix;
+    size_t in = 0, out = 0;
+    void* w = nullptr;
+    int dtype = FT_DTYPE_F32;
+    size_t r = 0;
+    float alpha = 0.0f;
+    float* a = nullptr;   // [in, r]
+    float* b = nullptr;   // [r, out]
+    float* ga = nullptr;
+    float* gb = nullptr;
+    bool has_lora() const { return r > 0; }
+    // graph/src/lib.rs:119-122: the scale is alpha / rank, skipped when it is exactly 1.
+    float scale() const {
+        const float s = alpha / (float)r;
+        return std::fabs(s - 1.0f) > kF32Epsilon ? s : 1.0f;
+    }
+};
+
+struct Layer {
+    float* norm1 = nullptr;
+    float* norm2 = nullptr;
+    LinearW q, k, v, o, gate, up, down;
+    LinearW* all[7] = {&q, &k, &v, &o, &gate, &up, &down};
+};
+
+struct ParamRef {
+    std::string name;
+    float* w;
+    float* g;
+    size_t n;
+};
+
+// Activations of one layer kept for backward.
+struct LayerActs {
+    float *x, *h1, *q, *k, *v, *attn, *stats, *h, *h2, *gate, *up, *act;
+    float *tq, *tk, *tv, *to, *tgate, *tup, *tdown;
+};
+
+}  // namespace
+
+struct ft_model {
+    ft_context* ctx = nullptr;
+    ft_model_config cfg{};
+    float* embed = nullptr;
+    std::vector<Layer> layers;
+    float* norm_f = nullptr;
+    LinearW lm_head;
+    std::vector<ParamRef> params;
+    bool params_dirty = true;
+
+    // Step buffers, valid for (ws_B, ws_S).
+    size_t ws_B = 0, ws_S = 0;
+    std::vector<void*> ws_allocs;
+    std::vector<LayerActs> acts;
+    float *x_final = nullptr, *hf = nullptr, *thead = nullptr, *logits = nullptr;
+    uint32_t *ids_dev = nullptr, *targets_dev = nullptr;
+    float *weights_dev = nullptr, *row_loss = nullptr;
+    // backward scratch
+    float *g0 = nullptr, *g1 = nullptr, *gx = nullptr, *d_act = nullptr, *d_gate = nullptr, *d_up = nullptr,
+          *d_h2 = nullptr, *d_h2b = nullptr, *d_attn = nullptr, *dq = nullptr, *dk = nullptr, *dv = nullptr,
+          *d_h1 = nullptr, *d_h1b = nullptr, *dt = nullptr, *gtmp = nullptr;
+
+    size_t head_dim() const { return cfg.hidden_size / cfg.num_attention_heads; }
+};
+
+struct ft_trainer {
+    ft_model* model = nullptr;
+    ft_trainer_config cfg{};
+    float t = 0.0f;                 // AdamW step counter (f32, as in the reference)
+    size_t step_in_accum = 0;
+    std::vector<float*> m, v;       // per parameter
+    ft_segment* segs_dev = nullptr;
+    size_t nseg = 0;
+    float* partials = nullptr;
+    float* control = nullptr;       // {grad_norm, clip_scale, apply}
+};
+
+namespace {
+
+int alloc_f(ft_context* ctx, size_t n, float** out) { return ft_alloc(ctx, n * sizeof(float), (void**)out); }
+
+int ws_alloc(ft_model* m, size_t n, float** out) {
+    FT_TRY(alloc_f(m->ctx, n, out));
+    m->ws_allocs.push_back(*out);
+    return FT_OK;
 }
+
+void ws_free(ft_model* m) {
+    for (void* p : m->ws_allocs) (void)ft_free(m->ctx, p);
+    m->ws_allocs.clear();
+    m->acts.clear();
+    m->ws_B = m->ws_S = 0;
+}
+
+int ensure_workspace(ft_model* m, size_t B, size_t S) {
+    if (m->ws_B == B && m->ws_S == S) return FT_OK;
+    ws_free(m);
+    const ft_model_config& c = m->cfg;
+    const size_t T = B * S, H = c.hidden_size, F = c.intermediate_size, V = c.vocab_size;
+    const size_t D = m->head_dim(), QD = c.num_attention_heads * D, KD = c.num_key_value_heads * D;
+    size_t rmax = m->lm_head.r;
+    m->acts.resize(c.num_hidden_layers);
+    for (size_t l = 0; l < c.num_hidden_layers; l++) {
+        LayerActs& a = m->acts[l];
+        Layer& L = m->layers[l];
+        FT_TRY(ws_alloc(m, T * H, &a.x));
+        FT_TRY(ws_alloc(m, T * H, &a.h1));
+        FT_TRY(ws_alloc(m, T * QD, &a.q));
+        FT_TRY(ws_alloc(m, T * KD, &a.k));
+        FT_TRY(ws_alloc(m, T * KD, &a.v));
+        FT_TRY(ws_alloc(m, T * QD, &a.attn));
+        FT_TRY(ws_alloc(m, B * c.num_attention_heads * S * 2, &a.stats));
+        FT_TRY(ws_alloc(m, T * H, &a.h));
+        FT_TRY(ws_alloc(m, T * H, &a.h2));
+        FT_TRY(ws_alloc(m, T * F, &a.gate));
+        FT_TRY(ws_alloc(m, T * F, &a.up));
+        FT_TRY(ws_alloc(m, T * F, &a.act));
+        float** ts[7] = {&a.tq, &a.tk, &a.tv, &a.to, &a.tgate, &a.tup, &a.tdown};
+        for (int i = 0; i < 7; i++) {
+            *ts[i] = nullptr;
+            if (L.all[i]->has_lora()) {
+                FT_TRY(ws_alloc(m, T * L.all[i]->r, ts[i]));
+                if (L.all[i]->r > rmax) rmax = L.all[i]->r;
+            }
+        }
+    }
+    FT_TRY(ws_alloc(m, T * H, &m->x_final));
+    FT_TRY(ws_alloc(m, T * H, &m->hf));
+    m->thead = nullptr;
+    if (m->lm_head.has_lora()) FT_TRY(ws_alloc(m, T * m->lm_head.r, &m->thead));
+    FT_TRY(ws_alloc(m, T * V, &m->logits));
+    FT_TRY(ws_alloc(m, T, (float**)&m->ids_dev));
+    FT_TRY(ws_alloc(m, T, (float**)&m->targets_dev));
+    FT_TRY(ws_alloc(m, T, &m->weights_dev));
+    FT_TRY(ws_alloc(m, T, &m->row_loss));
+    FT_TRY(ws_alloc(m, T * H, &m->g0));
+    FT_TRY(ws_alloc(m, T * H, &m->g1));
+    FT_TRY(ws_alloc(m, T * H, &m->gx));
+    FT_TRY(ws_alloc(m, T * F, &m->d_act));
+    FT_TRY(ws_alloc(m, T * F, &m->d_gate));
+    FT_TRY(ws_alloc(m, T * F, &m->d_up));
+    FT_TRY(ws_alloc(m, T * H, &m->d_h2));
+    FT_TRY(ws_alloc(m, T * H, &m->d_h2b));
+    FT_TRY(ws_alloc(m, T * QD, &m->d_attn));
+    FT_TRY(ws_alloc(m, T * QD, &m->dq));
+    FT_TRY(ws_alloc(m, T * KD, &m->dk));
+    FT_TRY(ws_alloc(m, T * KD, &m->dv));
+    FT_TRY(ws_alloc(m, T * H, &m->d_h1));
+    FT_TRY(ws_alloc(m, T * H, &m->d_h1b));
+    FT_TRY(ws_alloc(m, T * (rmax ? rmax : 1), &m->dt));
+    size_t gmax = 1;
+    for (auto& p : m->params) gmax = p.n > gmax ? p.n : gmax;
+    FT_TRY(ws_alloc(m, gmax, &m->gtmp));
+    m->ws_B = B;
+    m->ws_S = S;
+    return FT_OK;
+}
+
+void rebuild_params(ft_model* m) {
+    m->params.clear();
+    auto add = [&](LinearW& l) {
+        if (!l.has_lora()) return;
+        m->params.push_back({l.prefix + ".lora_a", l.a, l.ga, l.in * l.r});
+        m->params.push_back({l.prefix + ".lora_b", l.b, l.gb, l.r * l.out});
+    };
+    for (auto& L : m->layers)
+        for (auto* l : L.all) add(*l);
+    add(m->lm_head);
+    m->params_dirty = false;
+}
+
+// y = x @ W (+ (scale * x @ A) @ B), keeping t = scale * x @ A for backward.
+int linear_forward(ft_context* ctx, const LinearW& l, const float* x, float* t, float* y, size_t T) {
+    FT_CHECK_ARG(l.w, "linear %s has no weight", l.prefix.c_str());
+    if (l.has_lora()) {
+        FT_TRY(ft_lora_down(ctx, x, l.a, t, T, l.in, l.r, l.scale()));
+        return ft_lora_linear(ctx, x, l.w, l.dtype, t, l.b, y, T, l.in, l.out, l.r);
+    }
+    return ft_lora_linear(ctx, x, l.w, l.dtype, nullptr, nullptr, y, T, l.in, l.out, 0);
+}
+
+// Gradients of one linear given dy: LoRA factor gradients (written, or added
+// when `accumulate`), and dx when wanted.
+int linear_backward(ft_model* m, LinearW& l, const float* x, const float* t, const float* dy, float* dx, size_t T,
+                    bool accumulate) {
+    ft_context* ctx = m->ctx;
+    if (l.has_lora()) {
+        FT_TRY(ft_lora_grad_down(ctx, dy, l.b, m->dt, T, l.out, l.r, l.scale()));
+        float* gb = accumulate ? m->gtmp : l.gb;
+        FT_TRY(ft_lora_grad_b(ctx, t, dy, gb, T, l.out, l.r));
+        if (accumulate) FT_TRY(ft_gradient_accumulate(ctx, l.gb, gb, l.r * l.out));
+        float* ga = accumulate ? m->gtmp : l.ga;
+        FT_TRY(ft_lora_grad_a(ctx, x, m->dt, ga, T, l.in, l.r));
+        if (accumulate) FT_TRY(ft_gradient_accumulate(ctx, l.ga, ga, l.in * l.r));
+        if (dx) FT_TRY(ft_lora_linear_dx(ctx, dy, l.w, l.dtype, m->dt, l.a, dx, T, l.in, l.out, l.r));
+    } else if (dx) {
+        FT_TRY(ft_lora_linear_dx(ctx, dy, l.w, l.dtype, nullptr, nullptr, dx, T, l.in, l.out, 0));
+    }
+    return FT_OK;
+}
+
+int model_forward(ft_model* m, const uint32_t* rows_host, size_t B, size_t S) {
+    ft_context* ctx = m->ctx;
+    const ft_model_config& c = m->cfg;
+    FT_CHECK_ARG(m->embed && m->norm_f && m->lm_head.w, "model is missing embed_tokens, norm or lm_head weights");
+    for (auto& L : m->layers) {
+        FT_CHECK_ARG(L.norm1 && L.norm2, "a layer is missing its norm weights");
+        for (auto* l : L.all) FT_CHECK_ARG(l->w, "linear %s has no weight", l->prefix.c_str());
+    }
+    if (m->params_dirty) {
+        rebuild_params(m);
+        ws_free(m);
+    }
+    FT_TRY(ensure_workspace(m, B, S));
+    const size_t T = B * S, H = c.hidden_size, F = c.intermediate_size;
+    const size_t D = m->head_dim(), nh = c.num_attention_heads, nkv = c.num_key_value_heads;
+    FT_TRY(ft_upload(ctx, m->ids_dev, rows_host, T * sizeof(uint32_t)));
+    FT_TRY(ft_embedding(ctx, m->embed, c.vocab_size, H, m->ids_dev, T, m->acts.empty() ? m->x_final : m->acts[0].x));
+    ft_attention_options opts{};
+    opts.causal = 1;
+    for (size_t l = 0; l < m->layers.size(); l++) {
+        Layer& L = m->layers[l];
+        LayerActs& a = m->acts[l];
+        float* x_next = l + 1 < m->layers.size() ? m->acts[l + 1].x : m->x_final;
+        FT_TRY(ft_rms_norm_eps(ctx, a.x, L.norm1, a.h1, T, H, c.rms_norm_eps));
+        FT_TRY(linear_forward(ctx, L.q, a.h1, a.tq, a.q, T));
+        FT_TRY(linear_forward(ctx, L.k, a.h1, a.tk, a.k, T));
+        FT_TRY(linear_forward(ctx, L.v, a.h1, a.tv, a.v, T));
+        FT_TRY(ft_rope_theta(ctx, a.q, B, S, nh * D, D, 0, c.rope_theta));
+        FT_TRY(ft_rope_theta(ctx, a.k, B, S, nkv * D, D, 0, c.rope_theta));
+        FT_TRY(ft_flash_attention_v2_with_stats(ctx, a.q, a.k, a.v, a.attn, a.stats, B, S, S, nh, nkv, D, &opts));
+        // o_proj output lands in gx (scratch), then h = x + o
+        FT_TRY(linear_forward(ctx, L.o, a.attn, a.to, m->gx, T));
+        FT_TRY(ft_add(ctx, a.x, m->gx, a.h, T * H));
+        FT_TRY(ft_rms_norm_eps(ctx, a.h, L.norm2, a.h2, T, H, c.rms_norm_eps));
+        FT_TRY(linear_forward(ctx, L.up, a.h2, a.tup, a.up, T));
+        FT_TRY(linear_forward(ctx, L.gate, a.h2, a.tgate, a.gate, T));
+        FT_TRY(ft_silu_gate_fused(ctx, a.gate, a.up, a.act, T * F));
+        FT_TRY(linear_forward(ctx, L.down, a.act, a.tdown, m->gx, T));
+        FT_TRY(ft_add(ctx, a.h, m->gx, x_next, T * H));
+    }
+    FT_TRY(ft_rms_norm_eps(ctx, m->x_final, m->norm_f, m->hf, T, H, c.rms_norm_eps));
+    FT_TRY(linear_forward(ctx, m->lm_head, m->hf, m->thead, m->logits, T));
+    return FT_OK;
+}
+
+// Backward from d_logits (in m->logits) to every LoRA gradient.
+int model_backward(ft_model* m, size_t B, size_t S, bool accumulate) {
+    ft_context* ctx = m->ctx;
+    const ft_model_config& c = m->cfg;
+    const size_t T = B * S, H = c.hidden_size, F = c.intermediate_size;
+    const size_t D = m->head_dim(), nh = c.num_attention_heads, nkv = c.num_key_value_heads;
+    ft_attention_options opts{};
+    opts.causal = 1;
+    // lm_head and final norm
+    FT_TRY(linear_backward(m, m->lm_head, m->hf, m->thead, m->logits, m->d_h2, T, accumulate));
+    float* g = m->g0;
+    float* g_other = m->g1;
+    FT_TRY(ft_rms_norm_backward(ctx, m->x_final, m->norm_f, m->d_h2, g, nullptr, T, H, c.rms_norm_eps));
+    for (size_t li = m->layers.size(); li-- > 0;) {
+        Layer& L = m->layers[li];
+        LayerActs& a = m->acts[li];
+        // x_next = h + down(silu(gate) * up)
+        FT_TRY(linear_backward(m, L.down, a.act, a.tdown, g, m->d_act, T, accumulate));
+        FT_TRY(ft_silu_gate_backward(ctx, a.gate, a.up, m->d_act, m->d_gate, m->d_up, T * F));
+        FT_TRY(linear_backward(m, L.up, a.h2, a.tup, m->d_up, m->d_h2, T, accumulate));
+        FT_TRY(linear_backward(m, L.gate, a.h2, a.tgate, m->d_gate, m->d_h2b, T, accumulate));
+        FT_TRY(ft_gradient_accumulate(ctx, m->d_h2, m->d_h2b, T * H));
+        FT_TRY(ft_rms_norm_backward(ctx, a.h, L.norm2, m->d_h2, m->gx, nullptr, T, H, c.rms_norm_eps));
+        // g_h = g + gx (into g_other)
+        FT_TRY(ft_add(ctx, g, m->gx, g_other, T * H));
+        // h = x + o_proj(attn)
+        FT_TRY(linear_backward(m, L.o, a.attn, a.to, g_other, m->d_attn, T, accumulate));
+        FT_TRY(ft_flash_attention_v2_backward_with_stats(ctx, a.q, a.k, a.v, a.attn, m->d_attn, m->dq, m->dk, m->dv,
+                                                         a.stats, B, S, S, nh, nkv, D, &opts));
+        FT_TRY(ft_rope_theta_inverse(ctx, m->dq, B, S, nh * D, D, 0, c.rope_theta));
+        FT_TRY(ft_rope_theta_inverse(ctx, m->dk, B, S, nkv * D, D, 0, c.rope_theta));
+        // The first block's input is the frozen embedding: its norm output needs
+        // no gradient, so the three input-gradient GEMMs are skipped
+        // (MatMulNode::backward, autograd/src/lib.rs:268-287).
+        const bool need_dx = li > 0;
+        FT_TRY(linear_backward(m, L.q, a.h1, a.tq, m->dq, need_dx ? m->d_h1 : nullptr, T, accumulate));
+        FT_TRY(linear_backward(m, L.k, a.h1, a.tk, m->dk, need_dx ? m->d_h1b : nullptr, T, accumulate));
+        if (need_dx) FT_TRY(ft_gradient_accumulate(ctx, m->d_h1, m->d_h1b, T * H));
+        FT_TRY(linear_backward(m, L.v, a.h1, a.tv, m->dv, need_dx ? m->d_h1b : nullptr, T, accumulate));
+        if (!need_dx) break;
+        FT_TRY(ft_gradient_accumulate(ctx, m->d_h1, m->d_h1b, T * H));
+        FT_TRY(ft_rms_norm_backward(ctx, a.x, L.norm1, m->d_h1, m->gx, nullptr, T, H, c.rms_norm_eps));
+        FT_TRY(ft_add(ctx, g_other, m->gx, g, T * H));
+    }
+    return FT_OK;
+}
+
+LinearW* find_linear(ft_model* m, const std::string& prefix) {
+    if (prefix == "lm_head") return &m->lm_head;
+    for (auto& L : m->layers)
+        for (auto* l : L.all)
+            if (l->prefix == prefix) return l;
+    return nullptr;
+}
+
+int set_linear_weight(ft_model* m, LinearW& l, const float* hf_out_in, size_t out, size_t in) {
+    FT_CHECK_ARG(out == l.out && in == l.in, "%s.weight is [%zu, %zu], expected [%zu, %zu]", l.prefix.c_str(), out, in,
+                 l.out, l.in);
+    const int dtype = m->cfg.f16_linears ? FT_DTYPE_F16 : FT_DTYPE_F32;
+    if (!l.w) {
+        size_t bytes = in * out * (dtype == FT_DTYPE_F16 ? 2 : 4);
+        bytes = (bytes + 3) / 4 * 4;
+        FT_TRY(ft_alloc(m->ctx, bytes, &l.w));
+    }
+    l.dtype = dtype;
+    // builder rule: HF [out, in] -> [in, out] (model_builder.rs:415-424)
+    return ft_upload_f32_transposed(m->ctx, l.w, hf_out_in, out, in, dtype);
+}
+
+int set_vector(ft_model* m, float** slot, const float* data, size_t n, size_t want, const char* name) {
+    FT_CHECK_ARG(n == want, "%s has %zu values, expected %zu", name, n, want);
+    if (!*slot) FT_TRY(alloc_f(m->ctx, n, slot));
+    return ft_upload(m->ctx, *slot, data, n * sizeof(float));
+}
+
+template <typename Fn>
+int guarded(Fn&& fn) {
+    try {
+        return fn();
+    } catch (const std::exception& e) {
+        return ft_set_error(FT_ERR_INVALID, "exception: %s", e.what());
+    } catch (...) {
+        return ft_set_error(FT_ERR_INVALID, "unknown exception");
+    }
+}
+
+}  // namespace
+
+extern "C" {
+
+int ft_model_create(ft_context* ctx, const ft_model_config* cfg, ft_model** out) {
+    return guarded([&]() -> int {
+        FT_CHECK_ARG(ctx && cfg && out, "ft_model_create: NULL argument");
+        FT_CHECK_ARG(cfg->num_attention_heads > 0 && cfg->hidden_size % cfg->num_attention_heads == 0,
+                     "ft_model_create: hidden_size %u is not a multiple of %u heads", cfg->hidden_size,
+                     cfg->num_attention_heads);
+        FT_CHECK_ARG(cfg->num_key_value_heads > 0 && cfg->num_attention_heads % cfg->num_key_value_heads == 0,
+                     "ft_model_create: %u heads is not a multiple of %u kv heads", cfg->num_attention_heads,
+                     cfg->num_key_value_heads);
+        const size_t D = cfg->hidden_size / cfg->num_attention_heads;
+        FT_CHECK_ARG(D <= 128 && D % 2 == 0, "ft_model_create: head_dim %zu must be even and <= 128", D);
+        auto m = std::make_unique<ft_model>();
+        m->ctx = ctx;
+        m->cfg = *cfg;
+        const size_t H = cfg->hidden_size, F = cfg->intermediate_size;
+        const size_t QD = cfg->num_attention_heads * D, KD = cfg->num_key_value_heads * D;
+        m->layers.resize(cfg->num_hidden_layers);
+        for (size_t l = 0; l < m->layers.size(); l++) {
+            Layer& L = m->layers[l];
+            const std::string p = "model.layers." + std::to_string(l);
+            auto init = [&](LinearW& w, const char* name, size_t in, size_t o) {
+                w.prefix = p + name;
+                w.in = in;
+                w.out = o;
+            };
+            init(L.q, ".self_attn.q_proj", H, QD);
+            init(L.k, ".self_attn.k_proj", H, KD);
+            init(L.v, ".self_attn.v_proj", H, KD);
+            init(L.o, ".self_attn.o_proj", QD, H);
+            init(L.gate, ".mlp.gate_proj", H, F);
+            init(L.up, ".mlp.up_proj", H, F);
+            init(L.down, ".mlp.down_proj", F, H);
+        }
+        m->lm_head.prefix = "lm_head";
+        m->lm_head.in = H;
+        m->lm_head.out = cfg->vocab_size;
+        *out = m.release();
+        return FT_OK;
+    });
+}
+
+int ft_model_destroy(ft_model* m) {
+    if (!m) return FT_OK;
+    ws_free(m);
+    ft_context* ctx = m->ctx;
+    auto rel = [&](void* p) {
+        if (p) (void)ft_free(ctx, p);
+    };
+    auto rel_lin = [&](LinearW& l) {
+        rel(l.w);
+        rel(l.a);
+        rel(l.b);
+        rel(l.ga);
+        rel(l.gb);
+    };
+    rel(m->embed);
+    rel(m->norm_f);
+    for (auto& L : m->layers) {
+        rel(L.norm1);
+        rel(L.norm2);
+        for (auto* l : L.all) rel_lin(*l);
+    }
+    rel_lin(m->lm_head);
+    delete m;
+    return FT_OK;
+}
+
+int ft_model_set_tensor(ft_model* m, const char* hf_name, const float* data, const size_t* shape, int ndim) {
+    return guarded([&]() -> int {
+        FT_CHECK_ARG(m && hf_name && data && shape, "ft_model_set_tensor: NULL argument");
+        const std::string name(hf_name);
+        const ft_model_config& c = m->cfg;
+        const size_t H = c.hidden_size, V = c.vocab_size;
+        size_t n = 1;
+        for (int i = 0; i < ndim; i++) n *= shape[i];
+        if (name == "model.embed_tokens.weight") {
+            FT_CHECK_ARG(ndim == 2 && shape[0] == V && shape[1] == H, "embed_tokens must be [%zu, %zu]", V, H);
+            FT_TRY(set_vector(m, &m->embed, data, n, V * H, hf_name));
+            // Tied head = embedding transposed (model_builder.rs:653-689).
+            if (c.tie_word_embeddings) FT_TRY(set_linear_weight(m, m->lm_head, data, V, H));
+            return FT_OK;
+        }
+        if (name == "model.norm.weight") return set_vector(m, &m->norm_f, data, n, H, hf_name);
+        if (name == "lm_head.weight") {
+            FT_CHECK_ARG(ndim == 2, "lm_head.weight must be 2-D");
+            if (c.tie_word_embeddings) return FT_OK;  // the tied head ignores a separate tensor
+            return set_linear_weight(m, m->lm_head, data, shape[0], shape[1]);
+        }
+        const std::string pre = "model.layers.";
+        FT_CHECK_ARG(name.compare(0, pre.size(), pre) == 0, "unknown tensor %s", hf_name);
+        const size_t dot = name.find('.', pre.size());
+        FT_CHECK_ARG(dot != std::string::npos, "unknown tensor %s", hf_name);
+        const size_t li = (size_t)std::stoul(name.substr(pre.size(), dot - pre.size()));
+        FT_CHECK_ARG(li < m->layers.size(), "%s: layer %zu of %zu", hf_name, li, m->layers.size());
+        Layer& L = m->layers[li];
+        const std::string rest = name.substr(dot);
+        if (rest == ".input_layernorm.weight") return set_vector(m, &L.norm1, data, n, H, hf_name);
+        if (rest == ".post_attention_layernorm.weight") return set_vector(m, &L.norm2, data, n, H, hf_name);
+        const std::string suffix = ".weight";
+        FT_CHECK_ARG(rest.size() > suffix.size() && rest.compare(rest.size() - suffix.size(), suffix.size(), suffix) == 0,
+                     "unknown tensor %s", hf_name);
+        LinearW* l = find_linear(m, name.substr(0, name.size() - suffix.size()));
+        FT_CHECK_ARG(l, "unknown tensor %s", hf_name);
+        FT_CHECK_ARG(ndim == 2, "%s must be 2-D", hf_name);
+        return set_linear_weight(m, *l, data, shape[0], shape[1]);
+    });
+}
+
+int ft_model_set_lora(ft_model* m, const char* prefix, const float* a, const float* b, size_t rank, float alpha) {
+    return guarded([&]() -> int {
+        FT_CHECK_ARG(m && prefix && a && b, "ft_model_set_lora: NULL argument");
+        FT_CHECK_ARG(rank >= 1 && rank <= 32, "ft_model_set_lora: rank %zu is outside 1..32", rank);
+        LinearW* l = find_linear(m, prefix);
+        FT_CHECK_ARG(l, "ft_model_set_lora: no linear named %s", prefix);
+        if (l->r != rank) {
+            for (float** p : {&l->a, &l->b, &l->ga, &l->gb}) {
+                if (*p) FT_TRY(ft_free(m->ctx, *p));
+                *p = nullptr;
+            }
+            FT_TRY(alloc_f(m->ctx, l->in * rank, &l->a));
+            FT_TRY(alloc_f(m->ctx, rank * l->out, &l->b));
+            FT_TRY(alloc_f(m->ctx, l->in * rank, &l->ga));
+            FT_TRY(alloc_f(m->ctx, rank * l->out, &l->gb));
+            FT_TRY(ft_zero(m->ctx, l->ga, l->in * rank * 4));
+            FT_TRY(ft_zero(m->ctx, l->gb, rank * l->out * 4));
+            l->r = rank;
+            m->params_dirty = true;
+        }
+        l->alpha = alpha;
+        FT_TRY(ft_upload(m->ctx, l->a, a, l->in * rank * sizeof(float)));
+        FT_TRY(ft_upload(m->ctx, l->b, b, rank * l->out * sizeof(float)));
+        return FT_OK;
+    });
+}
+
+int ft_model_param_count(ft_model* m, size_t* count) {
+    return guarded([&]() -> int {
+        FT_CHECK_ARG(m && count, "ft_model_param_count: NULL argument");
+        if (m->params_dirty) {
+            rebuild_params(m);
+            ws_free(m);
+        }
+        *count = m->params.size();
+        return FT_OK;
+    });
+}
+
+int ft_model_param_info(ft_model* m, size_t index, const char** name, size_t* numel) {
+    return guarded([&]() -> int {
+        FT_CHECK_ARG(m, "ft_model_param_info: NULL argument");
+        if (m->params_dirty) {
+            rebuild_params(m);
+            ws_free(m);
+        }
+        FT_CHECK_ARG(index < m->params.size(), "ft_model_param_info: index %zu of %zu", index, m->params.size());
+        if (name) *name = m->params[index].name.c_str();
+        if (numel) *numel = m->params[index].n;
+        return FT_OK;
+    });
+}
+
+int ft_model_read_param(ft_model* m, size_t index, float* out_host) {
+    FT_CHECK_ARG(m && out_host && !m->params_dirty && index < m->params.size(), "ft_model_read_param: bad argument");
+    return ft_download(m->ctx, out_host, m->params[index].w, m->params[index].n * sizeof(float));
+}
+
+int ft_model_read_grad(ft_model* m, size_t index, float* out_host) {
+    FT_CHECK_ARG(m && out_host && !m->params_dirty && index < m->params.size(), "ft_model_read_grad: bad argument");
+    return ft_download(m->ctx, out_host, m->params[index].g, m->params[index].n * sizeof(float));
+}
+
+int ft_model_forward_logits(ft_model* m, const uint32_t* rows, size_t B, size_t S, float* logits_host) {
+    return guarded([&]() -> int {
+        FT_CHECK_ARG(m && rows && logits_host && B > 0 && S > 0, "ft_model_forward_logits: bad argument");
+        FT_TRY(model_forward(m, rows, B, S));
+        return ft_download(m->ctx, logits_host, m->logits, B * S * m->cfg.vocab_size * sizeof(float));
+    });
+}
+
+int ft_trainer_create(ft_model* m, const ft_trainer_config* cfg, ft_trainer** out) {
+    return guarded([&]() -> int {
+        FT_CHECK_ARG(m && cfg && out, "ft_trainer_create: NULL argument");
+        if (m->params_dirty) {
+            rebuild_params(m);
+            ws_free(m);
+        }
+        FT_CHECK_ARG(!m->params.empty(), "ft_trainer_create: the model has no LoRA adapter to train");
+        auto t = std::make_unique<ft_trainer>();
+        t->model = m;
+        t->cfg = *cfg;
+        ft_context* ctx = m->ctx;
+        std::vector<ft_segment> segs;
+        for (auto& p : m->params) {
+            float *pm = nullptr, *pv = nullptr;
+            FT_TRY(alloc_f(ctx, p.n, &pm));
+            FT_TRY(alloc_f(ctx, p.n, &pv));
+            FT_TRY(ft_zero(ctx, pm, p.n * 4));   // moments start at zero (AdamW::apply_step)
+            FT_TRY(ft_zero(ctx, pv, p.n * 4));
+            t->m.push_back(pm);
+            t->v.push_back(pv);
+            for (size_t off = 0; off < p.n; off += FT_SUM_SQUARES_CHUNK) {
+                const size_t n = p.n - off < FT_SUM_SQUARES_CHUNK ? p.n - off : FT_SUM_SQUARES_CHUNK;
+                segs.push_back(ft_segment{p.w + off, p.g + off, pm + off, pv + off, (uint32_t)n});
+            }
+        }
+        t->nseg = segs.size();
+        FT_TRY(ft_alloc(ctx, segs.size() * sizeof(ft_segment), (void**)&t->segs_dev));
+        FT_TRY(ft_upload(ctx, t->segs_dev, segs.data(), segs.size() * sizeof(ft_segment)));
+        FT_TRY(alloc_f(ctx, segs.size(), &t->partials));
+        FT_TRY(alloc_f(ctx, 4, &t->control));
+        *out = t.release();
+        return FT_OK;
+    });
+}
+
+int ft_trainer_destroy(ft_trainer* t) {
+    if (!t) return FT_OK;
+    ft_context* ctx = t->model->ctx;
+    for (float* p : t->m) (void)ft_free(ctx, p);
+    for (float* p : t->v) (void)ft_free(ctx, p);
+    if (t->segs_dev) (void)ft_free(ctx, t->segs_dev);
+    if (t->partials) (void)ft_free(ctx, t->partials);
+    if (t->control) (void)ft_free(ctx, t->control);
+    delete t;
+    return FT_OK;
+}
+
+int ft_trainer_train_chunk(ft_trainer* t, const uint32_t* rows, const uint32_t* targets, const uint8_t* loss_mask,
+                           size_t B, size_t S, int apply, ft_step_stats* stats, float* per_sequence_loss) {
+    return guarded([&]() -> int {
+        FT_CHECK_ARG(t && rows && targets && loss_mask && stats, "ft_trainer_train_chunk: NULL argument");
+        FT_CHECK_ARG(B > 0 && S > 0, "ft_trainer_train_chunk: empty chunk");
+        ft_model* m = t->model;
+        ft_context* ctx = m->ctx;
+        const size_t T = B * S, V = m->cfg.vocab_size;
+        const size_t accum = t->cfg.grad_accum_steps ? t->cfg.grad_accum_steps : B;
+        std::memset(stats, 0, sizeof(*stats));
+        stats->clip_scale = 1.0f;
+
+        // Host half of masked_cross_entropy_batch (trainer/src/lib.rs:689-722):
+        // per-row target or MASKED_CE_SKIP, weight 1 / supervised tokens of the row's sequence.
+        std::vector<uint32_t> tg(T);
+        std::vector<float> wt(T);
+        std::vector<size_t> tokens(B, 0);
+        auto supervised = [&](size_t r) { return loss_mask[r] != 0 && (size_t)targets[r] < V; };
+        size_t total_tokens = 0;
+        for (size_t s = 0; s < B; s++) {
+            for (size_t i = 0; i < S; i++) tokens[s] += supervised(s * S + i) ? 1 : 0;
+            total_tokens += tokens[s];
+        }
+        stats->supervised_tokens = (uint32_t)total_tokens;
+        if (total_tokens == 0) {
+            // masked_cross_entropy_batch returns None: no forward result is used, no backward.
+            t->step_in_accum += B;
+            if (per_sequence_loss)
+                for (size_t s = 0; s < B; s++) per_sequence_loss[s] = 0.0f;
+        } else {
+            for (size_t r = 0; r < T; r++) {
+                if (supervised(r)) {
+                    tg[r] = targets[r];
+                    wt[r] = 1.0f / (float)tokens[r / S];
+                } else {
+                    tg[r] = FT_MASKED_CE_SKIP;
+                    wt[r] = 0.0f;
+                }
+            }
+            FT_TRY(model_forward(m, rows, B, S));
+            FT_TRY(ft_upload(ctx, m->targets_dev, tg.data(), T * sizeof(uint32_t)));
+            FT_TRY(ft_upload(ctx, m->weights_dev, wt.data(), T * sizeof(float)));
+            // Loss + d loss / d logits in place, with the backward seed
+            // 1 / grad_accum_steps folded in (trainer/src/lib.rs:474-480, 553-572).
+            const float seed = 1.0f / (float)accum;
+            const float gscale = std::fabs(seed - 1.0f) > kF32Epsilon ? seed : 1.0f;
+            FT_TRY(ft_masked_cross_entropy_weighted(ctx, m->logits, m->targets_dev, m->weights_dev, m->logits,
+                                                    m->row_loss, T, V, gscale));
+            FT_TRY(model_backward(m, B, S, t->step_in_accum > 0));
+            t->step_in_accum += B;
+        }
+
+        const bool window_full = t->step_in_accum >= accum;
+        bool launched_update = false;
+        ft_adam_params ap{t->cfg.lr, t->cfg.beta1, t->cfg.beta2, t->cfg.eps, t->cfg.weight_decay, t->t + 1.0f};
+        if (window_full) {
+            t->step_in_accum = 0;
+            if (total_tokens > 0 || true) {
+                FT_TRY(ft_internal_multi_grad_norm(ctx, t->segs_dev, t->nseg, t->partials, t->cfg.clip_grad_norm,
+                                                   t->control));
+                if (apply) {
+                    FT_TRY(ft_internal_multi_adamw(ctx, t->segs_dev, t->nseg, &ap, 1.0f, t->control));
+                    launched_update = true;
+                }
+            }
+        }
+
+        // The step's only wait: row losses and the control block.
+        if (total_tokens > 0) {
+            std::vector<float> losses(T);
+            FT_TRY(ft_download(ctx, losses.data(), m->row_loss, T * sizeof(float)));
+            float total = 0.0f;
+            for (size_t s = 0; s < B; s++) {
+                double sum = 0.0;
+                for (size_t i = 0; i < S; i++) sum += (double)losses[s * S + i];
+                const float mean = (float)(sum / (double)(tokens[s] ? tokens[s] : 1));
+                if (per_sequence_loss) per_sequence_loss[s] = mean;
+                total += mean;
+            }
+            stats->loss = total;
+        }
+        if (window_full) {
+            float control[3];
+            FT_TRY(ft_download(ctx, control, t->control, sizeof(control)));
+            int applied;
+            std::memcpy(&applied, &control[2], 4);
+            stats->grad_norm = control[0];
+            stats->clip_scale = control[1];
+            if (launched_update && applied) {
+                t->t += 1.0f;
+                stats->optimizer_step = 1;
+            }
+        }
+        return FT_OK;
+    });
+}
+
+}  // extern "C"

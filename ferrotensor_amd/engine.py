@@ -9,6 +9,7 @@ here, FtError for errors the library reports). All compute happens in the HIP
 library; numpy only carries host data in and out.
 """
 import ctypes as C
+import weakref
 from dataclasses import dataclass
 from typing import Optional, Sequence
 
@@ -42,6 +43,12 @@ class HipContext:
         else:
             check(self._lib.ft_context_create_on_stream(device, C.c_void_p(stream), C.byref(h)))
         self.handle = h
+        # Objects that hold device memory of this context (models, trainers):
+        # closed first, so no handle outlives the context it allocates from.
+        self._children = weakref.WeakSet()
+
+    def _adopt(self, child):
+        self._children.add(child)
 
     def synchronize(self):
         check(self._lib.ft_synchronize(self.handle))
@@ -60,6 +67,8 @@ class HipContext:
 
     def close(self):
         if self.handle is not None and self.handle.value:
+            for child in list(self._children):
+                child.close()
             self._lib.ft_context_destroy(self.handle)
             self.handle = None
 

@@ -1,0 +1,223 @@
+"""Python mirror of the reference's model and trainer over the library's step driver.
+
+`Lfm2Model` follows `ferrotensor_graph::lfm::Lfm2Model` + `Lfm2ModelBuilder`
+(ferrotensor-graph/src/lfm.rs:590-623, model_builder.rs:623-709) and `Trainer`
+follows `ferrotensor_trainer::Trainer` (ferrotensor-trainer/src/lib.rs:74-135,
+371-502). The work happens in libferrotensor_hip.so (`ft_model_*`,
+`ft_trainer_*`); this file only marshals host arrays.
+"""
+import ctypes as C
+import weakref
+from dataclasses import dataclass
+from typing import Dict, List, Optional, Sequence, Tuple
+
+import numpy as np
+
+from . import _lib
+from ._lib import check
+from .engine import HipContext
+
+
+@dataclass
+class ModelConfig:
+    """The `Lfm2Config` fields the step uses (ferrotensor-loader/src/lib.rs:74-142)."""
+    vocab_size: int
+    hidden_size: int
+    intermediate_size: int
+    num_hidden_layers: int
+    num_attention_heads: int
+    num_key_value_heads: int
+    rms_norm_eps: float = 1e-5
+    rope_theta: float = 10000.0
+    tie_word_embeddings: bool = False
+    f16_linears: bool = False
+
+    def c(self):
+        return _lib.ModelConfigC(self.vocab_size, self.hidden_size, self.intermediate_size, self.num_hidden_layers,
+                                 self.num_attention_heads, self.num_key_value_heads, self.rms_norm_eps,
+                                 self.rope_theta, 1 if self.tie_word_embeddings else 0, 1 if self.f16_linears else 0)
+
+
+@dataclass
+class LoRaConfig:
+    """model_builder.rs `LoRaConfig`: rank, alpha, target module names."""
+    rank: int = 8
+    alpha: float = 16.0
+    target_modules: Tuple[str, ...] = ("q_proj", "k_proj", "v_proj", "o_proj")
+
+
+@dataclass
+class StepStats:
+    """trainer/src/lib.rs:36-58 for one chunk."""
+    loss: float
+    tokens: int
+    optimizer_step: bool
+    grad_norm: Optional[float]
+    clip_scale: float
+    per_sequence: List[float]
+
+
+class Lfm2Model:
+    def __init__(self, ctx: HipContext, config: ModelConfig):
+        self.ctx = ctx
+        self.config = config
+        self._lib = ctx._lib
+        h = C.c_void_p()
+        cfg = config.c()
+        check(self._lib.ft_model_create(ctx.handle, C.byref(cfg), C.byref(h)))
+        self.handle = h
+        self._trainers = []
+        ctx._adopt(self)
+
+    def set_tensor(self, hf_name: str, data):
+        """One Hugging Face tensor ([out, in] for linears); the library applies the builder's layout rules."""
+        data = np.ascontiguousarray(data, np.float32)
+        shape = (C.c_size_t * data.ndim)(*data.shape)
+        check(self._lib.ft_model_set_tensor(self.handle, hf_name.encode(), data.ctypes.data_as(C.c_void_p), shape,
+                                            data.ndim))
+
+    def load_tensors(self, tensors: Dict[str, np.ndarray]):
+        for name, value in tensors.items():
+            self.set_tensor(name, value)
+
+    def set_lora(self, prefix: str, a, b, alpha: float):
+        a = np.ascontiguousarray(a, np.float32)
+        b = np.ascontiguousarray(b, np.float32)
+        assert a.ndim == 2 and b.ndim == 2 and a.shape[1] == b.shape[0]
+        check(self._lib.ft_model_set_lora(self.handle, prefix.encode(), a.ctypes.data_as(C.c_void_p),
+                                          b.ctypes.data_as(C.c_void_p), a.shape[1], alpha))
+
+    def linear_prefixes(self, targets: Sequence[str]) -> List[str]:
+        out = []
+        for l in range(self.config.num_hidden_layers):
+            for n in ("q_proj", "k_proj", "v_proj", "o_proj"):
+                if n in targets:
+                    out.append(f"model.layers.{l}.self_attn.{n}")
+            for n in ("gate_proj", "up_proj", "down_proj"):
+                if n in targets:
+                    out.append(f"model.layers.{l}.mlp.{n}")
+        if "lm_head" in targets:
+            out.append("lm_head")
+        return out
+
+    def linear_dims(self, prefix: str) -> Tuple[int, int]:
+        c = self.config
+        d = c.hidden_size // c.num_attention_heads
+        table = {"q_proj": (c.hidden_size, c.num_attention_heads * d),
+                 "k_proj": (c.hidden_size, c.num_key_value_heads * d),
+                 "v_proj": (c.hidden_size, c.num_key_value_heads * d),
+                 "o_proj": (c.num_attention_heads * d, c.hidden_size),
+                 "gate_proj": (c.hidden_size, c.intermediate_size),
+                 "up_proj": (c.hidden_size, c.intermediate_size),
+                 "down_proj": (c.intermediate_size, c.hidden_size),
+                 "lm_head": (c.hidden_size, c.vocab_size)}
+        return table[prefix.split(".")[-1]]
+
+    def named_params(self) -> List[Tuple[str, int]]:
+        n = C.c_size_t()
+        check(self._lib.ft_model_param_count(self.handle, C.byref(n)))
+        out = []
+        for i in range(n.value):
+            name, numel = C.c_char_p(), C.c_size_t()
+            check(self._lib.ft_model_param_info(self.handle, i, C.byref(name), C.byref(numel)))
+            out.append((name.value.decode(), numel.value))
+        return out
+
+    def _read(self, fn, index, numel):
+        out = np.empty(numel, np.float32)
+        check(fn(self.handle, index, out.ctypes.data_as(C.c_void_p)))
+        return out
+
+    def params(self) -> Dict[str, np.ndarray]:
+        return {n: self._read(self._lib.ft_model_read_param, i, k) for i, (n, k) in enumerate(self.named_params())}
+
+    def grads(self) -> Dict[str, np.ndarray]:
+        return {n: self._read(self._lib.ft_model_read_grad, i, k) for i, (n, k) in enumerate(self.named_params())}
+
+    def forward_batch(self, rows) -> np.ndarray:
+        """`Lfm2Model::forward_batch`: logits [B, S, vocab] on the host."""
+        rows = np.ascontiguousarray(rows, np.uint32)
+        assert rows.ndim == 2, "forward_batch: rows must have the same length"
+        B, S = rows.shape
+        out = np.empty((B, S, self.config.vocab_size), np.float32)
+        check(self._lib.ft_model_forward_logits(self.handle, rows.ctypes.data_as(C.c_void_p), B, S,
+                                                out.ctypes.data_as(C.c_void_p)))
+        return out
+
+    def close(self):
+        if self.handle is not None and self.handle.value:
+            for ref in self._trainers:
+                t = ref()
+                if t is not None:
+                    t.close()
+            self._lib.ft_model_destroy(self.handle)
+            self.handle = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+def pad_chunk(seqs, length_bucket=32):
+    """`Trainer::train_chunk` padding (trainer/src/lib.rs:431-450): right-pad to a
+    multiple of `length_bucket` with each row's last token, loss mask 0."""
+    longest = max(min(len(i), len(t)) for i, t, _ in seqs)
+    padded = -(-longest // length_bucket) * length_bucket
+    rows, targets, masks = [], [], []
+    for ids, tg, mk in seqs:
+        n = min(len(ids), len(tg))
+        pad = ids[n - 1] if n else 0
+        rows.append(list(ids[:n]) + [pad] * (padded - n))
+        targets.append(list(tg[:n]) + [pad] * (padded - n))
+        masks.append([mk[i] if i < len(mk) else 0 for i in range(n)] + [0] * (padded - n))
+    return np.array(rows, np.uint32), np.array(targets, np.uint32), np.array(masks, np.uint8)
+
+
+class Trainer:
+    """`Trainer::new(..).with_grad_accum_steps(..).with_clip_grad_norm(..)` with an AdamW optimizer."""
+
+    def __init__(self, model: Lfm2Model, lr: float, beta1=0.9, beta2=0.999, eps=1e-8, weight_decay=0.01,
+                 clip_grad_norm: Optional[float] = None, grad_accum_steps: int = 0, length_bucket: int = 32):
+        self.model = model
+        self.length_bucket = length_bucket
+        self._lib = model._lib
+        cfg = _lib.TrainerConfigC(lr, beta1, beta2, eps, weight_decay,
+                                  clip_grad_norm if clip_grad_norm else 0.0, grad_accum_steps)
+        h = C.c_void_p()
+        check(self._lib.ft_trainer_create(model.handle, C.byref(cfg), C.byref(h)))
+        self.handle = h
+        model._trainers.append(weakref.ref(self))
+
+    def train_chunk(self, rows, targets, masks, apply: bool = True) -> StepStats:
+        rows = np.ascontiguousarray(rows, np.uint32)
+        targets = np.ascontiguousarray(targets, np.uint32)
+        masks = np.ascontiguousarray(masks, np.uint8)
+        assert rows.ndim == 2 and rows.shape == targets.shape == masks.shape
+        B, S = rows.shape
+        st = _lib.StepStatsC()
+        per = np.zeros(B, np.float32)
+        check(self._lib.ft_trainer_train_chunk(self.handle, rows.ctypes.data_as(C.c_void_p),
+                                               targets.ctypes.data_as(C.c_void_p), masks.ctypes.data_as(C.c_void_p),
+                                               B, S, 1 if apply else 0, C.byref(st), per.ctypes.data_as(C.c_void_p)))
+        return StepStats(loss=st.loss, tokens=st.supervised_tokens, optimizer_step=bool(st.optimizer_step),
+                         grad_norm=st.grad_norm, clip_scale=st.clip_scale, per_sequence=per.tolist())
+
+    def train_batch(self, seqs, apply: bool = True) -> StepStats:
+        """Ragged sequences [(input_ids, target_ids, loss_mask)]: dropped when
+        unsupervised or shorter than 2 tokens (trainer/src/lib.rs:385-398), padded, trained."""
+        kept = [(i, t, m) for i, t, m in seqs if len(i) >= 2 and len(t) > 0 and any(m)]
+        rows, targets, masks = pad_chunk(kept, self.length_bucket)
+        return self.train_chunk(rows, targets, masks, apply)
+
+    def close(self):
+        if self.handle is not None and self.handle.value:
+            self._lib.ft_trainer_destroy(self.handle)
+            self.handle = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass

@@ -205,7 +205,7 @@ def test_embedding_gather_bit_exact(g):
     np.testing.assert_array_equal(out.to_numpy(), cpu.embedding(table, ids))
 
 
-@pytest.mark.parametrize("rows,vocab", [(4, 7), (12, 50), (9, 4096), (5, 16384 + 4), (3, 49152), (2, 50000)])
+@pytest.mark.parametrize("rows,vocab", [(4, 7), (8, 32), (12, 50), (9, 4096), (5, 16384 + 4), (3, 49152), (2, 50000)])
 def test_masked_cross_entropy(g, rows, vocab):
     from ferrotensor_amd import UnifiedTensor
     ctx, eng = g
@@ -226,6 +226,7 @@ def test_masked_cross_entropy(g, rows, vocab):
     # in place, with the upstream scale folded in
     eng.masked_cross_entropy_weighted(ctx, tl, tt, up(ctx, weights), tl, row_loss, grad_scale=0.125)
     assert_close("ce grad in place", tl.to_numpy(), want_g * np.float32(0.125), atol=1e-6)
+    assert_close("ce loss in place", row_loss.to_numpy(), want_l)
 
 
 def test_sum_squares_and_adamw(g):
