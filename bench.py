@@ -1,0 +1,255 @@
+#!/usr/bin/env python3
+"""LoRA train step benchmark on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload 360m|135m|1.7b|tiny]
+
+A step is one full optimizer step (forward, masked cross-entropy, backward,
+gradient norm, clip, AdamW) of the SmolLM2-360M-shaped model on 8 sequences x
+256 tokens of synthetic, seeded input (BASELINE.json configs[3]); frozen f16
+base weights, f32 LoRA rank 8 alpha 16 on q/k/v/o, AdamW lr 2e-4. Weights and
+inputs are resident in HBM when the timed region starts, except the 2048 token
+ids / targets / weights the step uploads itself (24 KiB).
+
+Prints ONE JSON line: tokens/s (positions = B*S / step time), plus
+  roofline     the dominant GEMM kernel: algorithmic 2*M*N*K flops per launch
+               over its HIP-event duration (events on the library's stream,
+               taken over K further steps identical to the timed ones), against
+               the 157.3 TFLOP/s dense FP32 matrix peak;
+  cpu_baseline the CPU oracle (oracle/) on this host's cores, on a bounded
+               sample of the same workload (stated in `sample`).
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+FP32_MFMA_PEAK_TFLOPS = 157.3
+HBM_PEAK_GBS = 8000.0
+
+WORKLOADS = {
+    # name: (layers, hidden, heads, kv_heads, ffn, vocab, batch, seq, rank, alpha, targets, prompt range)
+    "360m": dict(layers=32, hidden=960, heads=15, kv=5, ffn=2560, vocab=49152, B=8, S=256, rank=8, alpha=16.0,
+                 targets=("q_proj", "k_proj", "v_proj", "o_proj"), prompt=(32, 128),
+                 label="SmolLM2-360M-shaped LoRA step, 8x256 (BASELINE.json configs[3])"),
+    "135m": dict(layers=30, hidden=576, heads=9, kv=3, ffn=1536, vocab=49152, B=8, S=256, rank=8, alpha=16.0,
+                 targets=("q_proj", "k_proj", "v_proj", "o_proj"), prompt=(32, 128),
+                 label="SmolLM2-135M-shaped LoRA step, 8x256 (BASELINE.json configs[2])"),
+    "1.7b": dict(layers=24, hidden=2048, heads=32, kv=32, ffn=8192, vocab=49152, B=8, S=1024, rank=16, alpha=32.0,
+                 targets=("q_proj", "k_proj", "v_proj", "o_proj", "gate_proj", "up_proj", "down_proj"),
+                 prompt=(64, 512), label="SmolLM2-1.7B-shaped LoRA step, 8x1024 (BASELINE.json configs[4])"),
+    "tiny": dict(layers=2, hidden=64, heads=4, kv=2, ffn=128, vocab=256, B=2, S=32, rank=4, alpha=8.0,
+                 targets=("q_proj", "k_proj", "v_proj", "o_proj"), prompt=(4, 8), label="tiny Llama (plumbing check)"),
+}
+
+
+def synthetic_tensors(w, seed=0):
+    """Random-init N(0, 0.02) weights in Hugging Face layout ([out, in]); norm scales 1."""
+    rng = np.random.default_rng(seed)
+    H, F, V = w["hidden"], w["ffn"], w["vocab"]
+    D = H // w["heads"]
+
+    def n(*shape):
+        return rng.standard_normal(shape, dtype=np.float32) * np.float32(0.02)
+
+    yield "model.embed_tokens.weight", n(V, H)
+    yield "model.norm.weight", np.ones(H, np.float32)
+    for l in range(w["layers"]):
+        p = f"model.layers.{l}"
+        yield f"{p}.input_layernorm.weight", np.ones(H, np.float32)
+        yield f"{p}.post_attention_layernorm.weight", np.ones(H, np.float32)
+        yield f"{p}.self_attn.q_proj.weight", n(w["heads"] * D, H)
+        yield f"{p}.self_attn.k_proj.weight", n(w["kv"] * D, H)
+        yield f"{p}.self_attn.v_proj.weight", n(w["kv"] * D, H)
+        yield f"{p}.self_attn.o_proj.weight", n(H, w["heads"] * D)
+        yield f"{p}.mlp.gate_proj.weight", n(F, H)
+        yield f"{p}.mlp.up_proj.weight", n(F, H)
+        yield f"{p}.mlp.down_proj.weight", n(H, F)
+
+
+def synthetic_batch(w, seed=1, B=None):
+    """Token ids uniform over the vocabulary; targets = next token; the loss mask
+    zeroes a prompt prefix whose length is uniform in the workload's range."""
+    rng = np.random.default_rng(seed)
+    B = B or w["B"]
+    S, V = w["S"], w["vocab"]
+    rows = rng.integers(0, V, (B, S)).astype(np.uint32)
+    targets = np.concatenate([rows[:, 1:], rng.integers(0, V, (B, 1)).astype(np.uint32)], axis=1)
+    masks = np.ones((B, S), np.uint8)
+    lo, hi = w["prompt"]
+    for b in range(B):
+        masks[b, :int(rng.integers(lo, hi + 1))] = 0
+    return rows, targets, masks
+
+
+def lora_factors(model, w, seed=2):
+    rng = np.random.default_rng(seed)
+    for name in model.linear_prefixes(w["targets"]):
+        i, o = model.linear_dims(name)
+        a = rng.standard_normal((i, w["rank"]), dtype=np.float32) * np.float32(0.02)
+        b = rng.standard_normal((w["rank"], o), dtype=np.float32) * np.float32(0.02)
+        yield name, a, b
+
+
+def step_flops(w):
+    """Algorithmic flops of one step (SURVEY convention): fwd + dX GEMMs on the
+    frozen base incl. the head, LoRA products, attention fwd + 2.5x bwd."""
+    T = w["B"] * w["S"]
+    H, F, V, L = w["hidden"], w["ffn"], w["vocab"], w["layers"]
+    D = H // w["heads"]
+    p_layer = H * w["heads"] * D * 2 + H * w["kv"] * D * 2 + 3 * H * F
+    p_lin = L * p_layer + H * V
+    attn = 2.0 * w["B"] * w["heads"] * w["S"] ** 2 * D * 3.5 * L
+    return 2 * (2.0 * T * p_lin) + attn
+
+
+def read_profile(ctx):
+    lib = ctx._lib
+    n = C.c_size_t()
+    from ferrotensor_amd._lib import check
+    check(lib.ft_profile_end(ctx.handle, C.byref(n)))
+    out = []
+    for i in range(n.value):
+        name, launches = C.c_char_p(), C.c_uint64()
+        ms, fl, by = C.c_double(), C.c_double(), C.c_double()
+        check(lib.ft_profile_kernel(ctx.handle, i, C.byref(name), C.byref(launches), C.byref(ms), C.byref(fl),
+                                    C.byref(by)))
+        if launches.value:
+            out.append(dict(name=name.value.decode(), launches=launches.value, ms=ms.value, flops=fl.value,
+                            bytes=by.value))
+    return sorted(out, key=lambda r: -r["ms"])
+
+
+def cpu_baseline(w, seconds_budget=30.0):
+    """The CPU oracle on this host, on ONE of the B sequences (full depth, full
+    vocabulary): a bounded sample of the same workload, scaled to tokens/s."""
+    from oracle import cpu
+    from oracle import reference_step as rs
+    cfg = rs.ModelConfig(w["vocab"], w["hidden"], w["ffn"], w["layers"], w["heads"], w["kv"], 1e-5, 100000.0, True)
+    tensors = dict(synthetic_tensors(w))
+    model = rs.Model.from_hf_tensors(cfg, tensors, f16_linears=True)
+    del tensors
+    rng = np.random.default_rng(2)
+    for name, lin in model.named_linears():
+        if name.split(".")[-1] in w["targets"]:
+            i, o = lin.weight.shape
+            model.set_lora(name, rng.standard_normal((i, w["rank"]), dtype=np.float32) * np.float32(0.02),
+                           rng.standard_normal((w["rank"], o), dtype=np.float32) * np.float32(0.02), w["alpha"])
+    rows, targets, masks = synthetic_batch(w, B=1)
+    opt = rs.AdamW(lr=2e-4, weight_decay=0.0)
+    times = []
+    t_all = time.perf_counter()
+    for _ in range(3):
+        t0 = time.perf_counter()
+        rs.train_chunk(model, opt, rows, targets, masks, grad_accum_steps=w["B"], clip_grad_norm=1.0)
+        times.append(time.perf_counter() - t0)
+        if time.perf_counter() - t_all > seconds_budget:
+            break
+    t = float(np.median(times))
+    return {"value": w["S"] / t, "unit": "tokens/s", "cores": cpu.num_threads(), "kind": "port",
+            "sample": "1 of the %d sequences (%d tokens), all %d layers + head, fwd+bwd+AdamW, median of %d steps, "
+                      "%.2f s/step, %d OpenMP threads" % (w["B"], w["S"], w["layers"], len(times), t,
+                                                          cpu.num_threads())}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="360m", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--breakdown", action="store_true", help="print the per-kernel event-time table to stderr")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on ONE GPU (one process, one HIP stream); --gpus %d is not supported. "
+                 "The step would shard by data parallelism over sequences with one all-reduce of the LoRA "
+                 "gradients, which is not built." % args.gpus)
+    w = WORKLOADS[args.workload]
+
+    from ferrotensor_amd import HipContext
+    from ferrotensor_amd.trainer import Lfm2Model, ModelConfig, Trainer
+
+    ctx = HipContext(0)
+    cfg = ModelConfig(vocab_size=w["vocab"], hidden_size=w["hidden"], intermediate_size=w["ffn"],
+                      num_hidden_layers=w["layers"], num_attention_heads=w["heads"], num_key_value_heads=w["kv"],
+                      rms_norm_eps=1e-5, rope_theta=100000.0, tie_word_embeddings=True, f16_linears=True)
+    model = Lfm2Model(ctx, cfg)
+    for name, value in synthetic_tensors(w):
+        model.set_tensor(name, value)
+    for name, a, b in lora_factors(model, w):
+        model.set_lora(name, a, b, w["alpha"])
+    # CLI defaults of `ferrotensor train`: lr 2e-4, weight decay 0, clip 1.0, accumulation = batch.
+    trainer = Trainer(model, lr=2e-4, weight_decay=0.0, clip_grad_norm=1.0)
+    rows, targets, masks = synthetic_batch(w)
+
+    for _ in range(args.warmup):
+        st = trainer.train_chunk(rows, targets, masks)
+    ctx.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        st = trainer.train_chunk(rows, targets, masks)
+    ctx.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed / args.steps * 1e3
+    tokens = w["B"] * w["S"]
+    value = tokens / (elapsed / args.steps)
+    if not (np.isfinite(st.loss) and st.optimizer_step):
+        sys.exit("bench.py: the step did not produce a finite loss / optimizer step: %r" % (st,))
+
+    # Per-kernel HIP-event timing over the same number of identical steps.
+    from ferrotensor_amd._lib import check
+    check(ctx._lib.ft_profile_begin(ctx.handle))
+    for _ in range(args.steps):
+        trainer.train_chunk(rows, targets, masks)
+    prof = read_profile(ctx)
+    gemms = [r for r in prof if r["name"].startswith("gemm_kernel")]
+    dom = gemms[0]
+    achieved = dom["flops"] / (dom["ms"] * 1e-3) / 1e12
+    all_gemm_ms = sum(r["ms"] for r in gemms)
+    all_gemm_tf = sum(r["flops"] for r in gemms) / (all_gemm_ms * 1e-3) / 1e12
+    kernel_ms = sum(r["ms"] for r in prof) / args.steps
+    if args.breakdown:
+        print("%-44s %8s %10s %9s %9s" % ("kernel", "launches", "ms/step", "TFLOP/s", "GB/s"), file=sys.stderr)
+        for r in prof:
+            print("%-44s %8d %10.3f %9.1f %9.0f" % (r["name"], r["launches"] // args.steps, r["ms"] / args.steps,
+                                                    r["flops"] / (r["ms"] * 1e-3) / 1e12 if r["ms"] else 0,
+                                                    r["bytes"] / (r["ms"] * 1e-3) / 1e9 if r["ms"] else 0),
+                  file=sys.stderr)
+        print("sum of kernel event time: %.3f ms/step; wall %.3f ms/step" % (kernel_ms, ms_per_step), file=sys.stderr)
+
+    out = {
+        "metric": "LoRA train tokens/s at SmolLM2-360M shape, seq256x8; % FP32 MFMA peak",
+        "value": value, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": w["label"], "global_batch": w["B"], "seq_len": w["S"],
+                   "lora": "rank %d alpha %g on %s" % (w["rank"], w["alpha"], "/".join(w["targets"])),
+                   "base_weights": "f16 storage, f32 arithmetic", "optimizer": "AdamW lr 2e-4 wd 0 clip 1.0",
+                   "supervised_tokens": int(st.tokens), "loss": float(st.loss)},
+        "step_tflops": step_flops(w) / (elapsed / args.steps) / 1e12,
+        "step_mfma_frac": step_flops(w) / (elapsed / args.steps) / 1e12 / FP32_MFMA_PEAK_TFLOPS,
+        "roofline": {"bound": "mfma", "kernel": dom["name"], "achieved": achieved, "peak": FP32_MFMA_PEAK_TFLOPS,
+                     "unit": "TFLOP/s", "frac": achieved / FP32_MFMA_PEAK_TFLOPS, "traffic": None,
+                     "launches_per_step": dom["launches"] // args.steps,
+                     "avg_launch_us": dom["ms"] * 1e3 / dom["launches"],
+                     "all_gemm_kernels_tflops": all_gemm_tf,
+                     "all_gemm_kernels_frac": all_gemm_tf / FP32_MFMA_PEAK_TFLOPS,
+                     "gemm_ms_per_step": all_gemm_ms / args.steps, "kernel_ms_per_step": kernel_ms},
+    }
+    if not args.no_cpu_baseline:
+        trainer.close()
+        model.close()
+        ctx.close()
+        out["cpu_baseline"] = cpu_baseline(w)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

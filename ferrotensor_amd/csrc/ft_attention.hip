@@ -442,6 +442,10 @@ template <int DP>
 int launch_fwd(ft_context* ctx, const AttnArgs& a) {
     constexpr int NW = 2;
     const dim3 grid(ft_div_up(a.Sq, 32 * NW), (unsigned)(a.B * a.H));
+    // flop convention of the reference's benchmarks: causal forward 2*B*H*Sq*Sk*D, full 4*...
+    const double fl = (a.causal ? 2.0 : 4.0) * a.B * a.H * (double)a.Sq * a.Sk * a.D;
+    const double by = 4.0 * a.B * ((double)a.Sq * a.H * a.D * 2 + (double)a.Sk * a.Hkv * a.D * 2);
+    ft_prof_scope prof(ctx, "attn_fwd_kernel", fl, by);
     hipLaunchKernelGGL((attn_fwd_kernel<DP, NW>), grid, dim3(NW * 64), 0, ctx->stream, a);
     FT_LAUNCH_CHECK();
     return FT_OK;
@@ -451,7 +455,14 @@ template <int DP>
 int launch_bwd(ft_context* ctx, const AttnArgs& a) {
     constexpr int NW = 2;
     const dim3 grid(ft_div_up(a.Sq, 32 * NW), (unsigned)(a.B * a.H));
-    hipLaunchKernelGGL((attn_bwd_dq_kernel<DP, NW>), grid, dim3(NW * 64), 0, ctx->stream, a);
+    // backward = 2.5x forward by the reference's convention: 1.5x (3 products) in dQ, 2x (4 products)
+    // in dK/dV, minus the shared recomputation -> charged 1.0x and 1.5x.
+    const double fl = (a.causal ? 2.0 : 4.0) * a.B * a.H * (double)a.Sq * a.Sk * a.D;
+    const double by = 4.0 * a.B * ((double)a.Sq * a.H * a.D * 4 + (double)a.Sk * a.Hkv * a.D * 4);
+    {
+        ft_prof_scope prof(ctx, "attn_bwd_dq_kernel", 1.0 * fl, by * 0.5);
+        hipLaunchKernelGGL((attn_bwd_dq_kernel<DP, NW>), grid, dim3(NW * 64), 0, ctx->stream, a);
+    }
     FT_LAUNCH_CHECK();
     constexpr size_t smem = (size_t)4 * 2 * 32 * (DP + 4) * sizeof(float);
     static bool attr_set = false;
@@ -461,7 +472,10 @@ int launch_bwd(ft_context* ctx, const AttnArgs& a) {
         attr_set = true;
     }
     const dim3 grid2(ft_div_up(a.Sk, 32), (unsigned)(a.B * a.Hkv));
-    hipLaunchKernelGGL((attn_bwd_dkdv_kernel<DP>), grid2, dim3(256), smem, ctx->stream, a);
+    {
+        ft_prof_scope prof(ctx, "attn_bwd_dkdv_kernel", 1.5 * fl, by * 0.5);
+        hipLaunchKernelGGL((attn_bwd_dkdv_kernel<DP>), grid2, dim3(256), smem, ctx->stream, a);
+    }
     FT_LAUNCH_CHECK();
     return FT_OK;
 }

@@ -24,6 +24,32 @@ struct ft_context {
     std::unordered_map<size_t, std::vector<void*>> idle;    // bytes -> free buffers
     size_t live_bytes = 0, idle_bytes = 0;
     int num_cus = 256;
+
+    // Per-kernel timing with HIP events on the context's stream (off by default).
+    struct ProfRecord {
+        int key;
+        hipEvent_t e0, e1;
+        double flops, bytes;
+    };
+    bool prof_on = false;
+    std::vector<std::string> prof_names;
+    std::map<std::string, int> prof_keys;
+    std::vector<ProfRecord> prof_records;
+    std::vector<hipEvent_t> prof_event_pool;
+    struct ProfTotal {
+        uint64_t launches = 0;
+        double ms = 0, flops = 0, bytes = 0;
+    };
+    std::vector<ProfTotal> prof_totals;
+};
+
+// Brackets the launches made during its lifetime with two events when the
+// context is profiling; otherwise does nothing.
+struct ft_prof_scope {
+    ft_context* ctx;
+    int index;
+    ft_prof_scope(ft_context* c, const char* name, double flops, double bytes);
+    ~ft_prof_scope();
 };
 
 int ft_set_error(int code, const char* fmt, ...);

@@ -359,6 +359,13 @@ int launch_cfg(ft_context* ctx, GemmArgs p, int layout, bool half_b) {
     const int tiles_m = (p.M + BM - 1) / BM;
     p.tiles_n = (p.N + BN - 1) / BN;
     const dim3 grid((unsigned)(tiles_m * p.tiles_n));
+    char name[96];
+    snprintf(name, sizeof(name), "gemm_kernel<%d, %d, %d, %d, %d, %s>", BM, BN, WM, WN, layout,
+             half_b ? "true" : "false");
+    const double kk = (double)p.K + (p.a2 ? (double)p.K2 : 0.0);
+    ft_prof_scope prof(ctx, name, 2.0 * p.M * (double)p.N * kk,
+                       4.0 * p.M * kk + (half_b ? 2.0 : 4.0) * p.N * (double)p.K + 4.0 * p.N * (p.a2 ? p.K2 : 0) +
+                           4.0 * p.M * (double)p.N);
 #define FT_GEMM_LAUNCH(L, H) \
     hipLaunchKernelGGL((gemm_kernel<BM, BN, WM, WN, L, H>), grid, dim3(256), 0, ctx->stream, p)
     if (layout == 0) {
@@ -419,6 +426,10 @@ template <bool XT, bool YT, bool OT>
 int skinny_launch(ft_context* ctx, const float* x, const float* y, float* out, size_t R, size_t Kr, size_t C,
                   long ldx, long ldy, long ldo, float scale) {
     if (R == 0 || C == 0) return FT_OK;
+    char name[64];
+    snprintf(name, sizeof(name), "skinny_kernel<%s, %s, %s>", XT ? "true" : "false", YT ? "true" : "false",
+             OT ? "true" : "false");
+    ft_prof_scope prof(ctx, name, 2.0 * R * (double)Kr * C, 4.0 * ((double)R * Kr + (double)Kr * C + (double)R * C));
     hipLaunchKernelGGL((skinny_kernel<XT, YT, OT>), dim3(ft_div_up(R, 32)), dim3(256), 0, ctx->stream, x, y, out,
                        (int)R, (int)Kr, (int)C, ldx, ldy, ldo, scale);
     FT_LAUNCH_CHECK();

@@ -159,6 +159,11 @@ int ew_launch(ft_context* ctx, EwArgs p) {
     size_t blocks = (work + 255) / 256;
     const size_t cap = (size_t)ctx->num_cus * 16;
     if (blocks > cap) blocks = cap;
+    static const char* const names[] = {"ew_kernel<Add>", "ew_kernel<AddBackward>", "ew_kernel<SiluGate>",
+                                        "ew_kernel<SiluGateBackward>", "ew_kernel<Scale>", "ew_kernel<Accumulate>",
+                                        "ew_kernel<Zero>"};
+    static const double arrays[] = {3, 3, 3, 5, 2, 3, 1};
+    ft_prof_scope prof(ctx, names[(int)OP], 0.0, 4.0 * arrays[(int)OP] * (double)p.n);
     if (vec)
         hipLaunchKernelGGL((ew_kernel<OP, true>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, p);
     else
@@ -581,6 +586,7 @@ __global__ __launch_bounds__(256) void multi_adamw_kernel(const ft_segment* __re
 int ft_internal_multi_grad_norm(ft_context* ctx, const ft_segment* segs_dev, size_t nseg, float* partials_dev,
                                 float max_norm, float* control_dev) {
     if (nseg == 0) return FT_OK;
+    ft_prof_scope prof(ctx, "multi_sum_squares+finish", 0.0, 4.0 * (double)nseg * FT_SUM_SQUARES_CHUNK);
     hipLaunchKernelGGL(multi_sum_squares_kernel, dim3((unsigned)nseg), dim3(256), 0, ctx->stream, segs_dev,
                        partials_dev);
     FT_LAUNCH_CHECK();
@@ -593,6 +599,7 @@ int ft_internal_multi_grad_norm(ft_context* ctx, const ft_segment* segs_dev, siz
 int ft_internal_multi_adamw(ft_context* ctx, const ft_segment* segs_dev, size_t nseg, const ft_adam_params* p,
                             float grad_scale, const float* control_dev) {
     if (nseg == 0) return FT_OK;
+    ft_prof_scope prof(ctx, "multi_adamw_kernel", 0.0, 28.0 * (double)nseg * FT_SUM_SQUARES_CHUNK);
     hipLaunchKernelGGL(multi_adamw_kernel, dim3((unsigned)nseg), dim3(256), 0, ctx->stream, segs_dev, *p,
                        grad_scale, control_dev);
     FT_LAUNCH_CHECK();
@@ -654,6 +661,7 @@ int ft_embedding(ft_context* ctx, const float* table, size_t vocab, size_t hidde
                  size_t n, float* out) {
     FT_CHECK_ARG(ctx && table && ids && out, "ft_embedding: NULL argument");
     if (n == 0 || hidden == 0) return FT_OK;
+    ft_prof_scope prof(ctx, "embedding_kernel", 0.0, 8.0 * (double)n * hidden);
     hipLaunchKernelGGL(embedding_kernel, dim3(ft_div_up(n, 4)), dim3(256), 0, ctx->stream, table, vocab, hidden,
                        ids, n, out);
     FT_LAUNCH_CHECK();
@@ -666,6 +674,7 @@ int ft_rms_norm_eps(ft_context* ctx, const float* x, const float* w, float* out,
     FT_CHECK_ARG(size > 0, "ft_rms_norm_eps: size is 0");
     if (rows == 0) return FT_OK;
     const int vec = (size % 4 == 0) && aligned16(x) && aligned16(w) && aligned16(out);
+    ft_prof_scope prof(ctx, "rms_norm_kernel", 0.0, 8.0 * (double)rows * size);
     hipLaunchKernelGGL(rms_norm_kernel, dim3((unsigned)rows), dim3(256), 0, ctx->stream, x, w, out, rows, size,
                        eps, vec);
     FT_LAUNCH_CHECK();
@@ -684,6 +693,7 @@ int ft_rms_norm_backward(ft_context* ctx, const float* x, const float* w, const 
     const size_t wgs = (rows + RPW - 1) / RPW;
     float* partial = nullptr;
     if (gw) FT_TRY(ft_alloc(ctx, wgs * size * sizeof(float), (void**)&partial));
+    ft_prof_scope prof(ctx, "rms_norm_backward_kernel", 0.0, 12.0 * (double)rows * size);
     hipLaunchKernelGGL((rms_norm_backward_kernel<RPW>), dim3((unsigned)wgs), dim3(256), 0, ctx->stream, x, w, g,
                        gx, partial, rows, size, eps);
     FT_LAUNCH_CHECK();
@@ -703,6 +713,7 @@ static int rope_launch(ft_context* ctx, const float* src, float* dst, size_t bat
     FT_CHECK_ARG(hidden % head_dim == 0, "%s: hidden %zu is not a multiple of head_dim %zu", who, hidden, head_dim);
     const size_t pairs = batch * seq * hidden / 2;
     if (pairs == 0) return FT_OK;
+    ft_prof_scope prof(ctx, "rope_kernel", 0.0, 8.0 * (double)pairs * 2);
     hipLaunchKernelGGL(rope_kernel, dim3(ft_div_up(pairs, 256)), dim3(256), 0, ctx->stream, src, dst, pairs,
                        (unsigned)head_dim, (unsigned)seq, (unsigned)pos, (unsigned)(hidden / head_dim), theta,
                        inverse ? -1.0f : 1.0f);
@@ -744,6 +755,7 @@ int ft_masked_cross_entropy_weighted(ft_context* ctx, const float* logits, const
     if (rows == 0) return FT_OK;
     const bool vec = (vocab % 4 == 0) && aligned16(logits) && aligned16(grad);
     const dim3 grid((unsigned)rows);
+    ft_prof_scope prof(ctx, "masked_ce_kernel", 0.0, 8.0 * (double)rows * vocab);
     if (!vec) {
         hipLaunchKernelGGL(masked_ce_scalar_kernel, grid, dim3(256), 0, ctx->stream, logits, targets, weights, grad,
                            row_loss, rows, vocab, grad_scale);

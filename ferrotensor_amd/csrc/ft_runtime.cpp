@@ -17,9 +17,87 @@ int ft_set_error(int code, const char* fmt, ...) {
     return code;
 }
 
+ft_prof_scope::ft_prof_scope(ft_context* c, const char* name, double flops, double bytes) : ctx(c), index(-1) {
+    if (!c || !c->prof_on) return;
+    auto it = c->prof_keys.find(name);
+    int key;
+    if (it == c->prof_keys.end()) {
+        key = (int)c->prof_names.size();
+        c->prof_names.push_back(name);
+        c->prof_keys[name] = key;
+        c->prof_totals.emplace_back();
+    } else {
+        key = it->second;
+    }
+    ft_context::ProfRecord r{key, nullptr, nullptr, flops, bytes};
+    for (hipEvent_t* e : {&r.e0, &r.e1}) {
+        if (!c->prof_event_pool.empty()) {
+            *e = c->prof_event_pool.back();
+            c->prof_event_pool.pop_back();
+        } else if (hipEventCreate(e) != hipSuccess) {
+            return;
+        }
+    }
+    if (hipEventRecord(r.e0, c->stream) != hipSuccess) return;
+    index = (int)c->prof_records.size();
+    c->prof_records.push_back(r);
+}
+
+ft_prof_scope::~ft_prof_scope() {
+    if (index >= 0) (void)hipEventRecord(ctx->prof_records[index].e1, ctx->stream);
+}
+
+// Waits for the stream and folds the finished records into the totals.
+static int prof_collect(ft_context* ctx) {
+    FT_HIP(hipStreamSynchronize(ctx->stream));
+    for (auto& r : ctx->prof_records) {
+        float ms = 0.0f;
+        if (hipEventElapsedTime(&ms, r.e0, r.e1) == hipSuccess) {
+            auto& t = ctx->prof_totals[r.key];
+            t.launches += 1;
+            t.ms += ms;
+            t.flops += r.flops;
+            t.bytes += r.bytes;
+        }
+        ctx->prof_event_pool.push_back(r.e0);
+        ctx->prof_event_pool.push_back(r.e1);
+    }
+    ctx->prof_records.clear();
+    return FT_OK;
+}
+
 extern "C" {
 
 const char* ft_last_error(void) { return g_last_error.c_str(); }
+
+int ft_profile_begin(ft_context* ctx) {
+    FT_CHECK_ARG(ctx, "ft_profile_begin: ctx is NULL");
+    FT_TRY(prof_collect(ctx));
+    for (auto& t : ctx->prof_totals) t = ft_context::ProfTotal();
+    ctx->prof_on = true;
+    return FT_OK;
+}
+
+int ft_profile_end(ft_context* ctx, size_t* kernels) {
+    FT_CHECK_ARG(ctx, "ft_profile_end: ctx is NULL");
+    ctx->prof_on = false;
+    FT_TRY(prof_collect(ctx));
+    if (kernels) *kernels = ctx->prof_names.size();
+    return FT_OK;
+}
+
+int ft_profile_kernel(ft_context* ctx, size_t index, const char** name, uint64_t* launches, double* total_ms,
+                      double* flops, double* bytes) {
+    FT_CHECK_ARG(ctx && index < ctx->prof_names.size(), "ft_profile_kernel: bad index");
+    FT_TRY(prof_collect(ctx));
+    const auto& t = ctx->prof_totals[index];
+    if (name) *name = ctx->prof_names[index].c_str();
+    if (launches) *launches = t.launches;
+    if (total_ms) *total_ms = t.ms;
+    if (flops) *flops = t.flops;
+    if (bytes) *bytes = t.bytes;
+    return FT_OK;
+}
 
 static int context_create(int device, void* stream, bool own, ft_context** out) {
     FT_CHECK_ARG(out != nullptr, "ft_context_create: out is NULL");
@@ -73,6 +151,11 @@ int ft_context_destroy(ft_context* ctx) {
     for (auto& kv : ctx->idle)
         for (void* p : kv.second) (void)hipFree(p);
     for (auto& kv : ctx->live) (void)hipFree(kv.first);
+    for (auto& r : ctx->prof_records) {
+        (void)hipEventDestroy(r.e0);
+        (void)hipEventDestroy(r.e1);
+    }
+    for (hipEvent_t e : ctx->prof_event_pool) (void)hipEventDestroy(e);
     if (ctx->owns_stream) (void)hipStreamDestroy(ctx->stream);
     delete ctx;
     return FT_OK;

@@ -69,6 +69,22 @@ int ft_flush(ft_context* ctx);
 /* The hipStream_t the context enqueues on. */
 void* ft_context_stream(ft_context* ctx);
 
+/* ---- per-kernel timing (stands in for the reference's timestamp-query
+ *      kernel timing, ferrotensor-backend/src/kernel_timing.rs:31-71) -------- */
+
+/* Starts bracketing every kernel launch of this context with HIP events on its
+ * stream and clears earlier totals. Costs two event records per launch: keep
+ * it off in timed regions that report end-to-end throughput. */
+int ft_profile_begin(ft_context* ctx);
+/* Stops bracketing, waits for the stream, and reports how many distinct kernel
+ * names have totals. */
+int ft_profile_end(ft_context* ctx, size_t* kernels);
+/* Totals of kernel `index`: launches, summed event time (ms), and the
+ * algorithmic flops / bytes the launches were charged with (2MNK for GEMMs,
+ * each array once for row kernels; KernelTimes labels, engine/matmul.rs:429-444). */
+int ft_profile_kernel(ft_context* ctx, size_t index, const char** name, uint64_t* launches,
+                      double* total_ms, double* flops, double* bytes);
+
 /* ---- buffers: UnifiedTensor storage + BufferPool (tensor.rs, pool.rs) ---- */
 
 /* UnifiedTensor::empty (tensor.rs:184-210): uninitialised device buffer from

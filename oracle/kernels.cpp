@@ -138,9 +138,11 @@ void orc_transpose(const float* src, float* out, size_t rows, size_t cols) {
 
 static void gemm_nn(const float* a, const float* b, float* out, size_t M, size_t K, size_t N) {
     constexpr size_t RB = 4, CB = 32;
-#pragma omp parallel for schedule(dynamic, 4) collapse(2)
-    for (long i0 = 0; i0 < (long)M; i0 += RB) {
-        for (long j0 = 0; j0 < (long)N; j0 += CB) {
+    // Column panel outermost: the K x 32 panel of b stays in cache while the
+    // rows of a stream past it.
+#pragma omp parallel for schedule(dynamic, 16) collapse(2)
+    for (long j0 = 0; j0 < (long)N; j0 += CB) {
+        for (long i0 = 0; i0 < (long)M; i0 += RB) {
             const size_t rb = std::min(RB, M - (size_t)i0);
             const size_t cb = std::min(CB, N - (size_t)j0);
             float acc[RB][CB];
