@@ -209,7 +209,7 @@ def main():
     for _ in range(args.steps):
         trainer.train_chunk(rows, targets, masks)
     prof = read_profile(ctx)
-    gemms = [r for r in prof if r["name"].startswith("gemm_kernel")]
+    gemms = [r for r in prof if r["name"].startswith("gemm_")]
     dom = gemms[0]
     achieved = dom["flops"] / (dom["ms"] * 1e-3) / 1e12
     all_gemm_ms = sum(r["ms"] for r in gemms)

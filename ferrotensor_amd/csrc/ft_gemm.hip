@@ -245,6 +245,223 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs p) {
 }
 
 // ---------------------------------------------------------------------------
+// Fast path: the same product for operands that are 16-byte aligned with
+// leading dimensions and K, K2 multiples of 4 (and, for operands whose rows run
+// along the contiguous dimension, a row count that is a multiple of 4). Edge
+// tiles are handled without branches: out-of-range rows read a clamped (valid)
+// address and produce values that are never stored, out-of-range k is zeroed
+// by a select. The loop body is straight-line code.
+//
+// LDS layouts: a k-contiguous operand is staged "k-quad major" as above
+// ([BK/4][rows][4], one ds_read_b128 per 4 MFMAs); an operand whose rows are
+// contiguous in memory is staged k-major ([BK][rows]) exactly as loaded, so no
+// register transpose is needed and both the b128 stores and the b32 operand
+// reads are free of bank conflicts.
+// ---------------------------------------------------------------------------
+
+// 16 bytes of zeros that out-of-range k loads are redirected to, so that no
+// select has to wait for the load.
+__device__ __attribute__((aligned(16))) float g_zero16[4] = {0.f, 0.f, 0.f, 0.f};
+
+typedef float float2_t __attribute__((ext_vector_type(2)));
+
+template <int ROWS, bool KCONTIG>
+struct FastTile {
+    static constexpr int PAD = 4;
+    static constexpr int KQ_STRIDE = ROWS * 4 + PAD;   // k-quad major: floats per quad row (== 4 mod 32)
+    static constexpr int K_STRIDE = ROWS + PAD;        // k-major: floats per k row
+    static constexpr int LDS_FLOATS = KCONTIG ? KQ * KQ_STRIDE : BK * K_STRIDE;
+    static constexpr int SLOTS = KCONTIG ? ROWS * KQ / 256 : BK * (ROWS / 4) / 256;
+    static_assert(SLOTS >= 1, "tile too small for 256 threads");
+    // Raw loaded bits: 4 floats, or 4 halfs in .x/.y. Converted when stored to
+    // LDS, so nothing between the load and the MFMA block depends on it.
+    float4 r[SLOTS];
+
+    __device__ __forceinline__ static void slot_coords(int i, int& row, int& k) {
+        const int s = threadIdx.x + i * 256;
+        if constexpr (KCONTIG) {
+            row = s / KQ;
+            k = (s % KQ) * 4;
+        } else {
+            row = (s % (ROWS / 4)) * 4;
+            k = s / (ROWS / 4);
+        }
+    }
+
+    template <typename T>
+    __device__ __forceinline__ void load(const T* base, long ld, int row0, int row_limit, int k0, int k_limit) {
+#pragma unroll
+        for (int i = 0; i < SLOTS; i++) {
+            int row, k;
+            slot_coords(i, row, k);
+            int gr = row0 + row;
+            const int gk = k0 + k;
+            long off;
+            if constexpr (KCONTIG) {
+                gr = gr < row_limit ? gr : row_limit - 1;
+                off = (long)gr * ld + gk;
+            } else {
+                gr = gr + 4 <= row_limit ? gr : row_limit - 4;
+                off = (long)gk * ld + gr;
+            }
+            const T* src = gk < k_limit ? base + off : reinterpret_cast<const T*>(g_zero16);
+            if constexpr (sizeof(T) == 2) {
+                const float2_t raw = *reinterpret_cast<const float2_t*>(src);
+                r[i].x = raw.x;
+                r[i].y = raw.y;
+            } else {
+                r[i] = *reinterpret_cast<const float4*>(src);
+            }
+        }
+    }
+
+    template <typename T>
+    __device__ __forceinline__ void store(float* lds) const {
+#pragma unroll
+        for (int i = 0; i < SLOTS; i++) {
+            int row, k;
+            slot_coords(i, row, k);
+            float4 v;
+            if constexpr (sizeof(T) == 2) {
+                float2_t raw;
+                raw.x = r[i].x;
+                raw.y = r[i].y;
+                const half4_t h = __builtin_bit_cast(half4_t, raw);
+                v = make_float4((float)h.x, (float)h.y, (float)h.z, (float)h.w);
+            } else {
+                v = r[i];
+            }
+            if constexpr (KCONTIG)
+                *reinterpret_cast<float4*>(lds + (k / 4) * KQ_STRIDE + row * 4) = v;
+            else
+                *reinterpret_cast<float4*>(lds + k * K_STRIDE + row) = v;
+        }
+    }
+
+    // The 4 k values lane (row, half) feeds to MFMAs 4*step .. 4*step+3.
+    __device__ __forceinline__ static float4 frag(const float* lds, int step, int half, int row) {
+        if constexpr (KCONTIG) {
+            return *reinterpret_cast<const float4*>(lds + (2 * step + half) * KQ_STRIDE + row * 4);
+        } else {
+            const float* p = lds + (8 * step + 4 * half) * K_STRIDE + row;
+            return make_float4(p[0], p[K_STRIDE], p[2 * K_STRIDE], p[3 * K_STRIDE]);
+        }
+    }
+};
+
+template <int BM, int BN, int WM, int WN, int LAYOUT, bool HALF_B>
+__global__ __launch_bounds__(256) void gemm_fast_kernel(GemmArgs p) {
+    constexpr bool A_KC = LAYOUT != 2;
+    constexpr bool B_KC = LAYOUT == 1;
+    constexpr int FM = WM / 32, FN = WN / 32;
+    constexpr int WAVES_N = BN / WN;
+    constexpr int STEPS = KQ / 2;
+    static_assert((BM / WM) * (BN / WN) == 4, "4 waves per workgroup");
+    using ATile = FastTile<BM, A_KC>;
+    using BTile = FastTile<BN, B_KC>;
+    using BType = typename std::conditional<HALF_B, _Float16, float>::type;
+
+    __shared__ __attribute__((aligned(16))) float As[2][ATile::LDS_FLOATS];
+    __shared__ __attribute__((aligned(16))) float Bs[2][BTile::LDS_FLOATS];
+
+    const int tile = blockIdx.x;
+    const int m0 = (tile / p.tiles_n) * BM;
+    const int n0 = (tile % p.tiles_n) * BN;
+    const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
+    const int wm0 = (wave / WAVES_N) * WM, wn0 = (wave % WAVES_N) * WN;
+    const int l32 = lane % 32, half = lane / 32;
+
+    floatx16 acc[FM][FN];
+#pragma unroll
+    for (int i = 0; i < FM; i++)
+#pragma unroll
+        for (int j = 0; j < FN; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
+
+    const int nt1 = (p.K + BK - 1) / BK;
+    const int nt2 = (LAYOUT != 2 && p.a2) ? (p.K2 + BK - 1) / BK : 0;
+    const int nt = nt1 + nt2;
+    const BType* bmat = reinterpret_cast<const BType*>(p.b);
+
+    ATile ta;
+    BTile tb;
+    // Tiles past nt1 belong to the second (LoRA) product: f32 operands, same orientation.
+    auto fetch = [&](int t) {
+        if (t < nt1) {
+            ta.load(p.a, p.lda, m0, p.M, t * BK, p.K);
+            tb.load(bmat, p.ldb, n0, p.N, t * BK, p.K);
+        } else if constexpr (LAYOUT != 2) {
+            ta.load(p.a2, p.lda2, m0, p.M, (t - nt1) * BK, p.K2);
+            tb.load(p.b2, p.ldb2, n0, p.N, (t - nt1) * BK, p.K2);
+        }
+    };
+    auto stash = [&](int t, int buf) {
+        ta.template store<float>(As[buf]);
+        if (t < nt1)
+            tb.template store<BType>(Bs[buf]);
+        else
+            tb.template store<float>(Bs[buf]);
+    };
+
+    if (nt > 0) {
+        fetch(0);
+        stash(0, 0);
+    }
+    __syncthreads();
+    for (int t = 0; t < nt; t++) {
+        const int buf = t & 1;
+        // Global loads of the next tile are issued first and consumed only after
+        // the MFMA block: the scheduling barriers keep the compiler from pulling
+        // the f16 conversion (and its wait) in front of the matrix work.
+        if (t + 1 < nt) fetch(t + 1);
+        __builtin_amdgcn_sched_barrier(0);
+        const float* as = As[buf];
+        const float* bs = Bs[buf];
+        float4 af[2][FM], bf[2][FN];
+#pragma unroll
+        for (int i = 0; i < FM; i++) af[0][i] = ATile::frag(as, 0, half, wm0 + i * 32 + l32);
+#pragma unroll
+        for (int j = 0; j < FN; j++) bf[0][j] = BTile::frag(bs, 0, half, wn0 + j * 32 + l32);
+#pragma unroll
+        for (int s = 0; s < STEPS; s++) {
+            const int cur = s & 1, nxt = cur ^ 1;
+            if (s + 1 < STEPS) {
+#pragma unroll
+                for (int i = 0; i < FM; i++) af[nxt][i] = ATile::frag(as, s + 1, half, wm0 + i * 32 + l32);
+#pragma unroll
+                for (int j = 0; j < FN; j++) bf[nxt][j] = BTile::frag(bs, s + 1, half, wn0 + j * 32 + l32);
+            }
+#pragma unroll
+            for (int i = 0; i < FM; i++)
+#pragma unroll
+                for (int j = 0; j < FN; j++) {
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[cur][i].x, bf[cur][j].x, acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[cur][i].y, bf[cur][j].y, acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[cur][i].z, bf[cur][j].z, acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[cur][i].w, bf[cur][j].w, acc[i][j], 0, 0, 0);
+                }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        if (t + 1 < nt) stash(t + 1, buf ^ 1);
+        __syncthreads();
+    }
+
+#pragma unroll
+    for (int i = 0; i < FM; i++)
+#pragma unroll
+        for (int j = 0; j < FN; j++) {
+            const int col = n0 + wn0 + j * 32 + l32;
+            if (col >= p.N) continue;
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int row = m0 + wm0 + i * 32 + (r / 4) * 8 + half * 4 + (r % 4);
+                if (row < p.M) p.out[(long)row * p.ldc + col] = acc[i][j][r];
+            }
+        }
+}
+
+// ---------------------------------------------------------------------------
 // out[R, C] (C <= 32) = scale * X[R, Kr] @ Y[Kr, C].
 //   XT:  X is stored [Kr, R] (element (row,k) at x[k*ldx + row])
 //   YT:  Y is stored [C, Kr] (element (k,col) at y[col*ldy + k])
@@ -355,19 +572,24 @@ struct TileCfg {
 };
 
 template <int BM, int BN, int WM, int WN>
-int launch_cfg(ft_context* ctx, GemmArgs p, int layout, bool half_b) {
+int launch_cfg(ft_context* ctx, GemmArgs p, int layout, bool half_b, bool fast) {
     const int tiles_m = (p.M + BM - 1) / BM;
     p.tiles_n = (p.N + BN - 1) / BN;
     const dim3 grid((unsigned)(tiles_m * p.tiles_n));
     char name[96];
-    snprintf(name, sizeof(name), "gemm_kernel<%d, %d, %d, %d, %d, %s>", BM, BN, WM, WN, layout,
-             half_b ? "true" : "false");
+    snprintf(name, sizeof(name), "%s<%d, %d, %d, %d, %d, %s>", fast ? "gemm_fast_kernel" : "gemm_kernel", BM, BN, WM,
+             WN, layout, half_b ? "true" : "false");
     const double kk = (double)p.K + (p.a2 ? (double)p.K2 : 0.0);
     ft_prof_scope prof(ctx, name, 2.0 * p.M * (double)p.N * kk,
                        4.0 * p.M * kk + (half_b ? 2.0 : 4.0) * p.N * (double)p.K + 4.0 * p.N * (p.a2 ? p.K2 : 0) +
                            4.0 * p.M * (double)p.N);
-#define FT_GEMM_LAUNCH(L, H) \
-    hipLaunchKernelGGL((gemm_kernel<BM, BN, WM, WN, L, H>), grid, dim3(256), 0, ctx->stream, p)
+#define FT_GEMM_LAUNCH(L, H)                                                                             \
+    do {                                                                                                 \
+        if (fast)                                                                                        \
+            hipLaunchKernelGGL((gemm_fast_kernel<BM, BN, WM, WN, L, H>), grid, dim3(256), 0, ctx->stream, p); \
+        else                                                                                             \
+            hipLaunchKernelGGL((gemm_kernel<BM, BN, WM, WN, L, H>), grid, dim3(256), 0, ctx->stream, p);      \
+    } while (0)
     if (layout == 0) {
         if (half_b) FT_GEMM_LAUNCH(0, true); else FT_GEMM_LAUNCH(0, false);
     } else if (layout == 1) {
@@ -417,9 +639,16 @@ int gemm_dispatch(ft_context* ctx, const char* who, int layout, bool half_b, con
             best_cost = cost;
         }
     }
-    if (best == 0) return launch_cfg<128, 128, 64, 64>(ctx, p, layout, half_b);
-    if (best == 1) return launch_cfg<128, 64, 64, 32>(ctx, p, layout, half_b);
-    return launch_cfg<64, 64, 32, 32>(ctx, p, layout, half_b);
+    // The branch-free kernel needs aligned operands and whole float4 groups.
+    auto al16 = [](const void* q) { return (((uintptr_t)q) & 15) == 0; };
+    bool fast = al16(a) && al16(b) && al16(out) && K % 4 == 0 && K >= 4 && (p.lda % 4 == 0) && (p.ldb % 4 == 0);
+    if (layout != 1) fast = fast && N % 4 == 0 && N >= 4;   // b rows run along n
+    if (layout == 2) fast = fast && M % 4 == 0 && M >= 4;   // a rows run along m
+    if (half_b) fast = fast && (p.ldb % 8 == 0 || layout == 1);
+    if (p.a2) fast = fast && al16(a2) && al16(b2) && K2 % 4 == 0 && K2 >= 4;
+    if (best == 0) return launch_cfg<128, 128, 64, 64>(ctx, p, layout, half_b, fast);
+    if (best == 1) return launch_cfg<128, 64, 64, 32>(ctx, p, layout, half_b, fast);
+    return launch_cfg<64, 64, 32, 32>(ctx, p, layout, half_b, fast);
 }
 
 template <bool XT, bool YT, bool OT>
