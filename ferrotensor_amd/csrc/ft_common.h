@@ -25,6 +25,9 @@ struct ft_context {
     size_t live_bytes = 0, idle_bytes = 0;
     int num_cus = 256;
 
+    // Partial sums of the sliced thin products (LoRA dA, dB); allocated on first use.
+    float* thin_scratch = nullptr;
+
     // Per-kernel timing with HIP events on the context's stream (off by default).
     struct ProfRecord {
         int key;

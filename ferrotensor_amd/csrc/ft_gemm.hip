@@ -17,6 +17,7 @@
 // and dB products), operands read straight from global memory into MFMA
 // operand registers, the reduction dimension split across the 4 waves.
 #include "ft_common.h"
+#include "ft_thin.h"
 
 namespace {
 
@@ -482,8 +483,9 @@ __global__ __launch_bounds__(256) void skinny_kernel(const float* __restrict__ x
     // k range of this wave, in steps of 8
     const int steps = (Kr + 7) / 8;
     const int per = (steps + 3) / 4;
-    const int s_begin = wave * per;
+    int s_begin = wave * per;
     const int s_end = (s_begin + per < steps) ? s_begin + per : steps;
+    if (s_begin > s_end) s_begin = s_end;
 
     floatx16 acc;
 #pragma unroll
@@ -549,16 +551,18 @@ __global__ __launch_bounds__(256) void skinny_kernel(const float* __restrict__ x
         red[wave][i * 33 + l32] = acc[r];
     }
     __syncthreads();
-    // 1024 outputs, 256 threads: fixed order w0 + w1 + w2 + w3.
-    for (int e = threadIdx.x; e < 32 * 32; e += 256) {
-        const int i = e / 32, j = e % 32;
+    auto emit = [&](int i, int j, float v) {
         if (r0 + i < R && j < C) {
-            const float v = ((red[0][i * 33 + j] + red[1][i * 33 + j]) + red[2][i * 33 + j]) + red[3][i * 33 + j];
             if constexpr (OT)
                 out[(long)j * ldo + r0 + i] = v * scale;
             else
                 out[(long)(r0 + i) * ldo + j] = v * scale;
         }
+    };
+    // 1024 outputs, 256 threads: the 4 waves are added in fixed order.
+    for (int e = threadIdx.x; e < 32 * 32; e += 256) {
+        const int i = e / 32, j = e % 32;
+        emit(i, j, ((red[0][i * 33 + j] + red[1][i * 33 + j]) + red[2][i * 33 + j]) + red[3][i * 33 + j]);
     }
 }
 
@@ -689,6 +693,8 @@ int ft_lora_down(ft_context* ctx, const float* x, const float* a, float* t, size
                  float scale) {
     FT_CHECK_ARG(ctx && x && a && t, "ft_lora_down: NULL argument");
     FT_CHECK_ARG(r >= 1 && r <= 32, "ft_lora_down: rank %zu is outside 1..32", r);
+    ft_thin_problem tp{x, a, t, (int)M, (int)K, 0, (int)r, (long)K, (long)r, (long)r, scale, 0, 0, 0};
+    if (ft_thin_rowwise_ok(tp)) return ft_thin_rowwise(ctx, &tp, 1);
     return skinny_launch<false, false, false>(ctx, x, a, t, M, K, r, (long)K, (long)r, (long)r, scale);
 }
 
@@ -703,6 +709,8 @@ int ft_lora_grad_down(ft_context* ctx, const float* dy, const float* b, float* d
     FT_CHECK_ARG(ctx && dy && b && dt, "ft_lora_grad_down: NULL argument");
     FT_CHECK_ARG(r >= 1 && r <= 32, "ft_lora_grad_down: rank %zu is outside 1..32", r);
     // dt[m][j] = sum_n dy[m][n] * b[j][n]
+    ft_thin_problem tp{dy, b, dt, (int)M, (int)N, 0, (int)r, (long)N, (long)N, (long)r, scale, 1, 0, 0};
+    if (ft_thin_rowwise_ok(tp)) return ft_thin_rowwise(ctx, &tp, 1);
     return skinny_launch<false, true, false>(ctx, dy, b, dt, M, N, r, (long)N, (long)N, (long)r, scale);
 }
 
@@ -717,6 +725,8 @@ int ft_lora_grad_b(ft_context* ctx, const float* t, const float* dy, float* db, 
     FT_CHECK_ARG(ctx && t && dy && db, "ft_lora_grad_b: NULL argument");
     FT_CHECK_ARG(r >= 1 && r <= 32, "ft_lora_grad_b: rank %zu is outside 1..32", r);
     // db^T[n][j] = sum_m dy[m][n] * t[m][j]: rows = n (dy read transposed), output stored transposed.
+    ft_thin_problem tp{dy, t, db, (int)M, 0, (int)N, (int)r, (long)N, (long)r, (long)N, 1.0f, 0, 1, 0};
+    if (ft_thin_colwise_ok(tp)) return ft_thin_colwise(ctx, &tp, 1);
     return skinny_launch<true, false, true>(ctx, dy, t, db, N, M, r, (long)N, (long)r, (long)N, 1.0f);
 }
 
@@ -724,6 +734,8 @@ int ft_lora_grad_a(ft_context* ctx, const float* x, const float* dt, float* da, 
     FT_CHECK_ARG(ctx && x && dt && da, "ft_lora_grad_a: NULL argument");
     FT_CHECK_ARG(r >= 1 && r <= 32, "ft_lora_grad_a: rank %zu is outside 1..32", r);
     // da[k][j] = sum_m x[m][k] * dt[m][j]: rows = k (x read transposed).
+    ft_thin_problem tp{x, dt, da, (int)M, 0, (int)K, (int)r, (long)K, (long)r, (long)r, 1.0f, 0, 0, 0};
+    if (ft_thin_colwise_ok(tp)) return ft_thin_colwise(ctx, &tp, 1);
     return skinny_launch<true, false, false>(ctx, x, dt, da, K, M, r, (long)K, (long)r, (long)r, 1.0f);
 }
 

@@ -156,6 +156,7 @@ int ft_context_destroy(ft_context* ctx) {
         (void)hipEventDestroy(r.e1);
     }
     for (hipEvent_t e : ctx->prof_event_pool) (void)hipEventDestroy(e);
+    if (ctx->thin_scratch) (void)hipFree(ctx->thin_scratch);
     if (ctx->owns_stream) (void)hipStreamDestroy(ctx->stream);
     delete ctx;
     return FT_OK;

@@ -19,6 +19,7 @@
 // per (batch, sequence) shape and kept. Nothing in the step waits for the GPU
 // until the per-row losses and the gradient norm are read back at its end.
 #include "ft_common.h"
+#include "ft_thin.h"
 
 #include <cmath>
 #include <cstring>
@@ -103,7 +104,7 @@ struct ft_model {
     // backward scratch
     float *g0 = nullptr, *g1 = nullptr, *gx = nullptr, *d_act = nullptr, *d_gate = nullptr, *d_up = nullptr,
           *d_h2 = nullptr, *d_h2b = nullptr, *d_attn = nullptr, *dq = nullptr, *dk = nullptr, *dv = nullptr,
-          *d_h1 = nullptr, *d_h1b = nullptr, *dt = nullptr, *gtmp = nullptr;
+          *d_h1 = nullptr, *d_h1b = nullptr, *dt = nullptr, *dt2 = nullptr, *dt3 = nullptr, *gtmp = nullptr;
 
     size_t head_dim() const { return cfg.hidden_size / cfg.num_attention_heads; }
 };
@@ -193,6 +194,8 @@ int ensure_workspace(ft_model* m, size_t B, size_t S) {
     FT_TRY(ws_alloc(m, T * H, &m->d_h1));
     FT_TRY(ws_alloc(m, T * H, &m->d_h1b));
     FT_TRY(ws_alloc(m, T * (rmax ? rmax : 1), &m->dt));
+    FT_TRY(ws_alloc(m, T * (rmax ? rmax : 1), &m->dt2));
+    FT_TRY(ws_alloc(m, T * (rmax ? rmax : 1), &m->dt3));
     size_t gmax = 1;
     for (auto& p : m->params) gmax = p.n > gmax ? p.n : gmax;
     FT_TRY(ws_alloc(m, gmax, &m->gtmp));
@@ -214,14 +217,40 @@ void rebuild_params(ft_model* m) {
     m->params_dirty = false;
 }
 
-// y = x @ W (+ (scale * x @ A) @ B), keeping t = scale * x @ A for backward.
-int linear_forward(ft_context* ctx, const LinearW& l, const float* x, float* t, float* y, size_t T) {
-    FT_CHECK_ARG(l.w, "linear %s has no weight", l.prefix.c_str());
-    if (l.has_lora()) {
-        FT_TRY(ft_lora_down(ctx, x, l.a, t, T, l.in, l.r, l.scale()));
-        return ft_lora_linear(ctx, x, l.w, l.dtype, t, l.b, y, T, l.in, l.out, l.r);
+// t_i = scale_i * x @ A_i for up to 3 linears that read the same x: one
+// launch when the adapters share a rank the vector kernel supports.
+int lora_down_group(ft_context* ctx, LinearW* const* ls, float* const* ts, int n, const float* x, size_t T) {
+    ft_thin_problem probs[3];
+    int cnt = 0;
+    bool batch = true;
+    for (int i = 0; i < n; i++) {
+        if (!ls[i]->has_lora()) continue;
+        const LinearW& l = *ls[i];
+        probs[cnt] = ft_thin_problem{x, l.a, ts[i], (int)T, (int)l.in, 0, (int)l.r, (long)l.in, (long)l.r, (long)l.r,
+                                     l.scale(), 0, 0, 0};
+        batch = batch && ft_thin_rowwise_ok(probs[cnt]) && l.r == ls[0]->r;
+        cnt++;
     }
+    if (cnt == 0) return FT_OK;
+    if (batch && cnt > 1) return ft_thin_rowwise(ctx, probs, cnt);
+    for (int i = 0; i < n; i++)
+        if (ls[i]->has_lora()) FT_TRY(ft_lora_down(ctx, x, ls[i]->a, ts[i], T, ls[i]->in, ls[i]->r, ls[i]->scale()));
+    return FT_OK;
+}
+
+// y = x @ W (+ t @ B) with t = scale * x @ A already computed.
+int linear_gemm(ft_context* ctx, const LinearW& l, const float* x, const float* t, float* y, size_t T) {
+    FT_CHECK_ARG(l.w, "linear %s has no weight", l.prefix.c_str());
+    if (l.has_lora()) return ft_lora_linear(ctx, x, l.w, l.dtype, t, l.b, y, T, l.in, l.out, l.r);
     return ft_lora_linear(ctx, x, l.w, l.dtype, nullptr, nullptr, y, T, l.in, l.out, 0);
+}
+
+// y = x @ W (+ (scale * x @ A) @ B), keeping t = scale * x @ A for backward.
+int linear_forward(ft_context* ctx, LinearW& l, const float* x, float* t, float* y, size_t T) {
+    LinearW* ls[1] = {&l};
+    float* ts[1] = {t};
+    FT_TRY(lora_down_group(ctx, ls, ts, 1, x, T));
+    return linear_gemm(ctx, l, x, t, y, T);
 }
 
 // Gradients of one linear given dy: LoRA factor gradients (written, or added
@@ -231,16 +260,64 @@ int linear_backward(ft_model* m, LinearW& l, const float* x, const float* t, con
     ft_context* ctx = m->ctx;
     if (l.has_lora()) {
         FT_TRY(ft_lora_grad_down(ctx, dy, l.b, m->dt, T, l.out, l.r, l.scale()));
-        float* gb = accumulate ? m->gtmp : l.gb;
-        FT_TRY(ft_lora_grad_b(ctx, t, dy, gb, T, l.out, l.r));
-        if (accumulate) FT_TRY(ft_gradient_accumulate(ctx, l.gb, gb, l.r * l.out));
-        float* ga = accumulate ? m->gtmp : l.ga;
-        FT_TRY(ft_lora_grad_a(ctx, x, m->dt, ga, T, l.in, l.r));
-        if (accumulate) FT_TRY(ft_gradient_accumulate(ctx, l.ga, ga, l.in * l.r));
+        if (accumulate) {
+            FT_TRY(ft_lora_grad_b(ctx, t, dy, m->gtmp, T, l.out, l.r));
+            FT_TRY(ft_gradient_accumulate(ctx, l.gb, m->gtmp, l.r * l.out));
+            FT_TRY(ft_lora_grad_a(ctx, x, m->dt, m->gtmp, T, l.in, l.r));
+            FT_TRY(ft_gradient_accumulate(ctx, l.ga, m->gtmp, l.in * l.r));
+        } else {
+            // dB = t^T dy and dA = x^T dt in one sliced launch when possible.
+            ft_thin_problem pb[2] = {
+                {dy, t, l.gb, (int)T, 0, (int)l.out, (int)l.r, (long)l.out, (long)l.r, (long)l.out, 1.0f, 0, 1, 0},
+                {x, m->dt, l.ga, (int)T, 0, (int)l.in, (int)l.r, (long)l.in, (long)l.r, (long)l.r, 1.0f, 0, 0, 0}};
+            if (ft_thin_colwise_ok(pb[0]) && ft_thin_colwise_ok(pb[1])) {
+                FT_TRY(ft_thin_colwise(ctx, pb, 2));
+            } else {
+                FT_TRY(ft_lora_grad_b(ctx, t, dy, l.gb, T, l.out, l.r));
+                FT_TRY(ft_lora_grad_a(ctx, x, m->dt, l.ga, T, l.in, l.r));
+            }
+        }
         if (dx) FT_TRY(ft_lora_linear_dx(ctx, dy, l.w, l.dtype, m->dt, l.a, dx, T, l.in, l.out, l.r));
     } else if (dx) {
         FT_TRY(ft_lora_linear_dx(ctx, dy, l.w, l.dtype, nullptr, nullptr, dx, T, l.in, l.out, 0));
     }
+    return FT_OK;
+}
+
+// The same for up to 3 linears that share their input x (q/k/v, gate/up): the
+// dT, dA and dB products of all of them go into two batched launches. dxs[i]
+// may be NULL. Falls back to one linear at a time when the adapters cannot be
+// batched or gradients are being accumulated.
+int linear_backward_group(ft_model* m, LinearW* const* ls, const float* const* ts, const float* const* dys,
+                          float* const* dxs, int n, const float* x, size_t T, bool accumulate) {
+    ft_context* ctx = m->ctx;
+    float* dts[3] = {m->dt, m->dt2, m->dt3};
+    bool batch = !accumulate && n <= 3;
+    ft_thin_problem rows[3], cols[6];
+    for (int i = 0; i < n && batch; i++) {
+        const LinearW& l = *ls[i];
+        if (!l.has_lora() || l.r != ls[0]->r) {
+            batch = false;
+            break;
+        }
+        rows[i] = ft_thin_problem{dys[i], l.b, dts[i], (int)T, (int)l.out, 0, (int)l.r, (long)l.out, (long)l.out,
+                                  (long)l.r, l.scale(), 1, 0, 0};
+        cols[2 * i] = ft_thin_problem{dys[i], ts[i], l.gb, (int)T, 0, (int)l.out, (int)l.r, (long)l.out, (long)l.r,
+                                      (long)l.out, 1.0f, 0, 1, 0};
+        cols[2 * i + 1] = ft_thin_problem{x, dts[i], l.ga, (int)T, 0, (int)l.in, (int)l.r, (long)l.in, (long)l.r,
+                                          (long)l.r, 1.0f, 0, 0, 0};
+        batch = ft_thin_rowwise_ok(rows[i]) && ft_thin_colwise_ok(cols[2 * i]) && ft_thin_colwise_ok(cols[2 * i + 1]);
+    }
+    if (!batch) {
+        for (int i = 0; i < n; i++) FT_TRY(linear_backward(m, *ls[i], x, ts[i], dys[i], dxs[i], T, accumulate));
+        return FT_OK;
+    }
+    FT_TRY(ft_thin_rowwise(ctx, rows, n));
+    FT_TRY(ft_thin_colwise(ctx, cols, 2 * n));
+    for (int i = 0; i < n; i++)
+        if (dxs[i])
+            FT_TRY(ft_lora_linear_dx(ctx, dys[i], ls[i]->w, ls[i]->dtype, dts[i], ls[i]->a, dxs[i], T, ls[i]->in,
+                                     ls[i]->out, ls[i]->r));
     return FT_OK;
 }
 
@@ -268,9 +345,14 @@ int model_forward(ft_model* m, const uint32_t* rows_host, size_t B, size_t S) {
         LayerActs& a = m->acts[l];
         float* x_next = l + 1 < m->layers.size() ? m->acts[l + 1].x : m->x_final;
         FT_TRY(ft_rms_norm_eps(ctx, a.x, L.norm1, a.h1, T, H, c.rms_norm_eps));
-        FT_TRY(linear_forward(ctx, L.q, a.h1, a.tq, a.q, T));
-        FT_TRY(linear_forward(ctx, L.k, a.h1, a.tk, a.k, T));
-        FT_TRY(linear_forward(ctx, L.v, a.h1, a.tv, a.v, T));
+        {
+            LinearW* ls[3] = {&L.q, &L.k, &L.v};
+            float* ts[3] = {a.tq, a.tk, a.tv};
+            FT_TRY(lora_down_group(ctx, ls, ts, 3, a.h1, T));
+        }
+        FT_TRY(linear_gemm(ctx, L.q, a.h1, a.tq, a.q, T));
+        FT_TRY(linear_gemm(ctx, L.k, a.h1, a.tk, a.k, T));
+        FT_TRY(linear_gemm(ctx, L.v, a.h1, a.tv, a.v, T));
         FT_TRY(ft_rope_theta(ctx, a.q, B, S, nh * D, D, 0, c.rope_theta));
         FT_TRY(ft_rope_theta(ctx, a.k, B, S, nkv * D, D, 0, c.rope_theta));
         FT_TRY(ft_flash_attention_v2_with_stats(ctx, a.q, a.k, a.v, a.attn, a.stats, B, S, S, nh, nkv, D, &opts));
@@ -278,8 +360,13 @@ int model_forward(ft_model* m, const uint32_t* rows_host, size_t B, size_t S) {
         FT_TRY(linear_forward(ctx, L.o, a.attn, a.to, m->gx, T));
         FT_TRY(ft_add(ctx, a.x, m->gx, a.h, T * H));
         FT_TRY(ft_rms_norm_eps(ctx, a.h, L.norm2, a.h2, T, H, c.rms_norm_eps));
-        FT_TRY(linear_forward(ctx, L.up, a.h2, a.tup, a.up, T));
-        FT_TRY(linear_forward(ctx, L.gate, a.h2, a.tgate, a.gate, T));
+        {
+            LinearW* ls[2] = {&L.up, &L.gate};
+            float* ts[2] = {a.tup, a.tgate};
+            FT_TRY(lora_down_group(ctx, ls, ts, 2, a.h2, T));
+        }
+        FT_TRY(linear_gemm(ctx, L.up, a.h2, a.tup, a.up, T));
+        FT_TRY(linear_gemm(ctx, L.gate, a.h2, a.tgate, a.gate, T));
         FT_TRY(ft_silu_gate_fused(ctx, a.gate, a.up, a.act, T * F));
         FT_TRY(linear_forward(ctx, L.down, a.act, a.tdown, m->gx, T));
         FT_TRY(ft_add(ctx, a.h, m->gx, x_next, T * H));
@@ -308,8 +395,13 @@ int model_backward(ft_model* m, size_t B, size_t S, bool accumulate) {
         // x_next = h + down(silu(gate) * up)
         FT_TRY(linear_backward(m, L.down, a.act, a.tdown, g, m->d_act, T, accumulate));
         FT_TRY(ft_silu_gate_backward(ctx, a.gate, a.up, m->d_act, m->d_gate, m->d_up, T * F));
-        FT_TRY(linear_backward(m, L.up, a.h2, a.tup, m->d_up, m->d_h2, T, accumulate));
-        FT_TRY(linear_backward(m, L.gate, a.h2, a.tgate, m->d_gate, m->d_h2b, T, accumulate));
+        {
+            LinearW* ls[2] = {&L.up, &L.gate};
+            const float* ts[2] = {a.tup, a.tgate};
+            const float* dys[2] = {m->d_up, m->d_gate};
+            float* dxs[2] = {m->d_h2, m->d_h2b};
+            FT_TRY(linear_backward_group(m, ls, ts, dys, dxs, 2, a.h2, T, accumulate));
+        }
         FT_TRY(ft_gradient_accumulate(ctx, m->d_h2, m->d_h2b, T * H));
         FT_TRY(ft_rms_norm_backward(ctx, a.h, L.norm2, m->d_h2, m->gx, nullptr, T, H, c.rms_norm_eps));
         // g_h = g + gx (into g_other)
@@ -324,12 +416,17 @@ int model_backward(ft_model* m, size_t B, size_t S, bool accumulate) {
         // no gradient, so the three input-gradient GEMMs are skipped
         // (MatMulNode::backward, autograd/src/lib.rs:268-287).
         const bool need_dx = li > 0;
-        FT_TRY(linear_backward(m, L.q, a.h1, a.tq, m->dq, need_dx ? m->d_h1 : nullptr, T, accumulate));
-        FT_TRY(linear_backward(m, L.k, a.h1, a.tk, m->dk, need_dx ? m->d_h1b : nullptr, T, accumulate));
-        if (need_dx) FT_TRY(ft_gradient_accumulate(ctx, m->d_h1, m->d_h1b, T * H));
-        FT_TRY(linear_backward(m, L.v, a.h1, a.tv, m->dv, need_dx ? m->d_h1b : nullptr, T, accumulate));
+        {
+            LinearW* ls[3] = {&L.q, &L.k, &L.v};
+            const float* ts[3] = {a.tq, a.tk, a.tv};
+            const float* dys[3] = {m->dq, m->dk, m->dv};
+            // d_h1 = dx_q + dx_k + dx_v: the three land in d_h1, d_h1b and gx.
+            float* dxs[3] = {need_dx ? m->d_h1 : nullptr, need_dx ? m->d_h1b : nullptr, need_dx ? m->gx : nullptr};
+            FT_TRY(linear_backward_group(m, ls, ts, dys, dxs, 3, a.h1, T, accumulate));
+        }
         if (!need_dx) break;
         FT_TRY(ft_gradient_accumulate(ctx, m->d_h1, m->d_h1b, T * H));
+        FT_TRY(ft_gradient_accumulate(ctx, m->d_h1, m->gx, T * H));
         FT_TRY(ft_rms_norm_backward(ctx, a.x, L.norm1, m->d_h1, m->gx, nullptr, T, H, c.rms_norm_eps));
         FT_TRY(ft_add(ctx, g_other, m->gx, g, T * H));
     }
