@@ -62,47 +62,57 @@ __device__ __forceinline__ float4 load_row4(const float* row, int d, int D, bool
 // lane must supply when the register is reused as a B operand.
 __device__ __forceinline__ int row_of(int t, int half) { return (t / 4) * 8 + half * 4 + (t % 4); }
 
-// Stage a 32 x DP tile (rows r0.., head hh of a [.., S, heads, D] tensor) into
-// LDS with row stride DP+4, zero filled outside S or D. NT threads cooperate.
-template <int DP, int NT>
-__device__ __forceinline__ void stage_tile(float* lds, const float* base, int b, int S, int heads, int hh, int D,
-                                           int r0, int tid) {
-    constexpr int LD = DP + 4;
-    constexpr int V4 = 32 * DP / 4;
-    for (int e = tid; e < V4; e += NT) {
-        const int r = e / (DP / 4), c = (e % (DP / 4)) * 4;
-        const int row = r0 + r;
-        const bool ok = row < S;
-        const float* src = base + (((long)b * S + (ok ? row : 0)) * heads + hh) * D;
-        *reinterpret_cast<float4*>(lds + r * LD + c) = load_row4(src, c, D, ok);
-    }
+// Operand fetches straight from global memory into MFMA operand registers. The
+// tiles are small (32 rows x head_dim), every wave needs its own, and they are
+// L2 resident, so there is no LDS staging and no workgroup barrier in the key
+// loop: a wave runs free, with the next tile's loads in flight while it
+// multiplies the current one.
+//   quad: 4 consecutive head-dim values of one row (A operand "row x k" with k
+//         along the head dim: lanes 0-31 take quads 8s.., lanes 32-63 8s+4..)
+//   one:  a single value (A operand with the head dim as the ROW: lane = d)
+template <bool FULL>
+__device__ __forceinline__ float4 ld_quad(const float* row, int d, int D) {
+    if constexpr (FULL) return *reinterpret_cast<const float4*>(row + d);
+    return load_row4(row, d, D, true);
+}
+template <bool FULL>
+__device__ __forceinline__ float ld_one(const float* row, int d, int D) {
+    if constexpr (FULL) return row[d];
+    return d < D ? row[d] : 0.0f;
 }
 
 // ---------------------------------------------------------------------------
-// Forward. Grid (ceil(Sq / (32*NW)), B*H); each wave owns 32 queries.
+// Forward. A workgroup owns 32 queries of one (batch, head); its NSPL waves take
+// every NSPL-th block of 32 keys and merge their partial softmax states through
+// LDS at the end (shorter critical path under the causal mask, and two waves
+// per SIMD to overlap one wave's softmax arithmetic with the other's MFMAs).
+// Grid (ceil(Sq/32), B*H); query blocks are issued last-first: the last block
+// has the longest key loop, so the long ones start first.
 // ---------------------------------------------------------------------------
-template <int DP, int NW>
-__global__ __launch_bounds__(NW * 64) void attn_fwd_kernel(AttnArgs p) {
-    constexpr int LD = DP + 4;
+constexpr int kKeySplit = 2;
+
+template <int DP, bool FULL>
+__global__ __launch_bounds__(kKeySplit * 64) void attn_fwd_kernel(AttnArgs p) {
     constexpr int NF = DP / 32;  // 32-row blocks of the head dim
     constexpr int NS = DP / 8;   // k-steps of 8 over the head dim
-    __shared__ __attribute__((aligned(16))) float Ks[32 * LD];
-    __shared__ __attribute__((aligned(16))) float Vs[32 * LD];
-
-    const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
-    const int l32 = lane % 32, half = lane / 32;
+    constexpr int NSPL = kKeySplit;
+    __shared__ float merge[(NSPL - 1) * 64 * (NF * 16 + 2)];
+    const int lane = threadIdx.x % 64, wave = threadIdx.x / 64, l32 = lane % 32, half = lane / 32;
     const int b = blockIdx.y / p.H, h = blockIdx.y % p.H;
     const int kvh = h / (p.H / p.Hkv);
-    const int q_wg0 = blockIdx.x * (32 * NW);
-    const int q0 = q_wg0 + wave * 32;
+    const int q0 = ((int)gridDim.x - 1 - (int)blockIdx.x) * 32;
     const int qi = q0 + l32;
     const bool q_ok = qi < p.Sq;
-    const float* qrow = p.q + (((long)b * p.Sq + (q_ok ? qi : 0)) * p.H + h) * p.D;
+    const int qc = q_ok ? qi : p.Sq - 1;
+    const float* qrow = p.q + (((long)b * p.Sq + qc) * p.H + h) * p.D;
+    const long kst = (long)p.Hkv * p.D;
+    const float* kbase = p.k + ((long)b * p.Sk * p.Hkv + kvh) * p.D;
+    const float* vbase = p.v + ((long)b * p.Sk * p.Hkv + kvh) * p.D;
 
     float4 qreg[NS];
 #pragma unroll
     for (int s = 0; s < NS; s++) {
-        float4 t = load_row4(qrow, 8 * s + 4 * half, p.D, q_ok);
+        const float4 t = ld_quad<FULL>(qrow, 8 * s + 4 * half, p.D);
         qreg[s] = make_float4(t.x * p.scale, t.y * p.scale, t.z * p.scale, t.w * p.scale);
     }
     floatx16 o[NF];
@@ -110,30 +120,40 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd_kernel(AttnArgs p) {
     for (int f = 0; f < NF; f++) o[f] = zero16();
     float m_run = kMasked, l_run = 0.0f;
 
-    // Keys any query of this workgroup can see (uniform: every wave runs the
-    // same number of tiles and meets the same barriers).
-    int q_last_wg = q_wg0 + 32 * NW - 1;
-    if (q_last_wg > p.Sq - 1) q_last_wg = p.Sq - 1;
     int k_end = p.Sk;
-    if (p.causal && q_last_wg + p.causal_offset + 1 < k_end) k_end = q_last_wg + p.causal_offset + 1;
-    const int q_last_wave = q0 + 31 + p.causal_offset;  // last position this wave can see when causal
+    if (p.causal && q0 + 31 + p.causal_offset + 1 < k_end) k_end = q0 + 31 + p.causal_offset + 1;
     const int q_pos = qi + p.causal_offset;
 
-    for (int kb = 0; kb < k_end; kb += 32) {
-        __syncthreads();
-        stage_tile<DP, NW * 64>(Ks, p.k, b, p.Sk, p.Hkv, kvh, p.D, kb, tid);
-        stage_tile<DP, NW * 64>(Vs, p.v, b, p.Sk, p.Hkv, kvh, p.D, kb, tid);
-        __syncthreads();
-        if (q0 >= p.Sq || (p.causal && kb > q_last_wave)) continue;  // wave-uniform
+    float4 kc[NS], kn[NS];
+    float vc[NF][16], vn[NF][16];
+    auto load_block = [&](int kb, float4 (&kk)[NS], float (&vv)[NF][16]) {
+        int key = kb + l32;
+        key = key < p.Sk ? key : p.Sk - 1;
+        const float* krow = kbase + key * kst;
+#pragma unroll
+        for (int s = 0; s < NS; s++) kk[s] = ld_quad<FULL>(krow, 8 * s + 4 * half, p.D);
+#pragma unroll
+        for (int t = 0; t < 16; t++) {
+            int kt = kb + row_of(t, half);
+            kt = kt < p.Sk ? kt : p.Sk - 1;
+            const float* vrow = vbase + kt * kst;
+#pragma unroll
+            for (int f = 0; f < NF; f++) vv[f][t] = ld_one<FULL>(vrow, f * 32 + l32, p.D);
+        }
+    };
+    const int kb_first = wave * 32;
+    if (kb_first < k_end) load_block(kb_first, kc, vc);
+    for (int kb = kb_first; kb < k_end; kb += 32 * NSPL) {
+        const bool more = kb + 32 * NSPL < k_end;
+        if (more) load_block(kb + 32 * NSPL, kn, vn);
 
         floatx16 s = zero16();
 #pragma unroll
         for (int st = 0; st < NS; st++) {
-            const float4 a = *reinterpret_cast<const float4*>(Ks + l32 * LD + 8 * st + 4 * half);
-            s = MFMA(a.x, qreg[st].x, s);
-            s = MFMA(a.y, qreg[st].y, s);
-            s = MFMA(a.z, qreg[st].z, s);
-            s = MFMA(a.w, qreg[st].w, s);
+            s = MFMA(kc[st].x, qreg[st].x, s);
+            s = MFMA(kc[st].y, qreg[st].y, s);
+            s = MFMA(kc[st].z, qreg[st].z, s);
+            s = MFMA(kc[st].w, qreg[st].w, s);
         }
         float tile_max = kMasked;
 #pragma unroll
@@ -161,10 +181,44 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd_kernel(AttnArgs p) {
 #pragma unroll
             for (int r = 0; r < 16; r++) o[f][r] *= corr;
 #pragma unroll
-            for (int t = 0; t < 16; t++) {
-                const float a = Vs[row_of(t, half) * LD + f * 32 + l32];
-                o[f] = MFMA(a, s[t], o[f]);
-            }
+            for (int t = 0; t < 16; t++) o[f] = MFMA(vc[f][t], s[t], o[f]);
+        }
+        if (more) {
+#pragma unroll
+            for (int st = 0; st < NS; st++) kc[st] = kn[st];
+#pragma unroll
+            for (int f = 0; f < NF; f++)
+#pragma unroll
+                for (int t = 0; t < 16; t++) vc[f][t] = vn[f][t];
+        }
+    }
+
+    // Merge the waves' (m, l, O) into wave 0, in wave order.
+    if constexpr (NSPL > 1) {
+        constexpr int W = NF * 16 + 2;
+        if (wave > 0) {
+            float* dst = merge + ((wave - 1) * 64 + lane) * W;
+            dst[0] = m_run;
+            dst[1] = l_run;
+#pragma unroll
+            for (int f = 0; f < NF; f++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) dst[2 + f * 16 + r] = o[f][r];
+        }
+        __syncthreads();
+        if (wave > 0) return;
+#pragma unroll
+        for (int w = 1; w < NSPL; w++) {
+            const float* src = merge + ((w - 1) * 64 + lane) * W;
+            const float m_o = src[0], l_o = src[1];
+            const float m_new = fmaxf(m_run, m_o);
+            const float c0 = __expf(m_run - m_new), c1 = __expf(m_o - m_new);
+            l_run = l_run * c0 + l_o * c1;
+            m_run = m_new;
+#pragma unroll
+            for (int f = 0; f < NF; f++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) o[f][r] = o[f][r] * c0 + src[2 + f * 16 + r] * c1;
         }
     }
 
@@ -194,71 +248,84 @@ __global__ __launch_bounds__(NW * 64) void attn_fwd_kernel(AttnArgs p) {
 // dQ = scale * sum_j dS_ij K_j with dS = P * (dO.V - Delta), P = exp(S - LSE).
 // Same decomposition as the forward.
 // ---------------------------------------------------------------------------
-template <int DP, int NW>
-__global__ __launch_bounds__(NW * 64) void attn_bwd_dq_kernel(AttnArgs p) {
-    constexpr int LD = DP + 4;
+template <int DP, bool FULL>
+__global__ __launch_bounds__(kKeySplit * 64) void attn_bwd_dq_kernel(AttnArgs p) {
     constexpr int NF = DP / 32;
     constexpr int NS = DP / 8;
-    __shared__ __attribute__((aligned(16))) float Ks[32 * LD];
-    __shared__ __attribute__((aligned(16))) float Vs[32 * LD];
-
-    const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
-    const int l32 = lane % 32, half = lane / 32;
+    constexpr int NSPL = kKeySplit;
+    __shared__ float merge[(NSPL - 1) * 64 * NF * 16];
+    const int lane = threadIdx.x % 64, wave = threadIdx.x / 64, l32 = lane % 32, half = lane / 32;
     const int b = blockIdx.y / p.H, h = blockIdx.y % p.H;
     const int kvh = h / (p.H / p.Hkv);
-    const int q_wg0 = blockIdx.x * (32 * NW);
-    const int q0 = q_wg0 + wave * 32;
+    const int q0 = ((int)gridDim.x - 1 - (int)blockIdx.x) * 32;
     const int qi = q0 + l32;
     const bool q_ok = qi < p.Sq;
-    const long qoff = (((long)b * p.Sq + (q_ok ? qi : 0)) * p.H + h) * p.D;
-    const long srow = ((long)b * p.H + h) * p.Sq + (q_ok ? qi : 0);
+    const int qc = q_ok ? qi : p.Sq - 1;
+    const long qoff = (((long)b * p.Sq + qc) * p.H + h) * p.D;
+    const long srow = ((long)b * p.H + h) * p.Sq + qc;
+    const long kst = (long)p.Hkv * p.D;
+    const float* kbase = p.k + ((long)b * p.Sk * p.Hkv + kvh) * p.D;
+    const float* vbase = p.v + ((long)b * p.Sk * p.Hkv + kvh) * p.D;
 
     float4 qreg[NS], doreg[NS];
     float delta = 0.0f;
 #pragma unroll
     for (int s = 0; s < NS; s++) {
         const int d = 8 * s + 4 * half;
-        const float4 t = load_row4(p.q + qoff, d, p.D, q_ok);
+        const float4 t = ld_quad<FULL>(p.q + qoff, d, p.D);
         qreg[s] = make_float4(t.x * p.scale, t.y * p.scale, t.z * p.scale, t.w * p.scale);
-        doreg[s] = load_row4(p.d_out + qoff, d, p.D, q_ok);
-        const float4 ov = load_row4(p.out + qoff, d, p.D, q_ok);
+        doreg[s] = ld_quad<FULL>(p.d_out + qoff, d, p.D);
+        const float4 ov = ld_quad<FULL>(p.out + qoff, d, p.D);
         delta += doreg[s].x * ov.x + doreg[s].y * ov.y + doreg[s].z * ov.z + doreg[s].w * ov.w;
     }
     delta += __shfl_xor(delta, 32, 64);
     const float lse = q_ok ? p.stats[2 * srow + 1] : kLseEmpty;
-    if (q_ok && half == 0) p.stats[2 * srow] = delta;
+    if (q_ok && half == 0 && wave == 0) p.stats[2 * srow] = delta;
 
     floatx16 acc[NF];
 #pragma unroll
     for (int f = 0; f < NF; f++) acc[f] = zero16();
 
-    int q_last_wg = q_wg0 + 32 * NW - 1;
-    if (q_last_wg > p.Sq - 1) q_last_wg = p.Sq - 1;
     int k_end = p.Sk;
-    if (p.causal && q_last_wg + p.causal_offset + 1 < k_end) k_end = q_last_wg + p.causal_offset + 1;
-    const int q_last_wave = q0 + 31 + p.causal_offset;
+    if (p.causal && q0 + 31 + p.causal_offset + 1 < k_end) k_end = q0 + 31 + p.causal_offset + 1;
     const int q_pos = qi + p.causal_offset;
 
-    for (int kb = 0; kb < k_end; kb += 32) {
-        __syncthreads();
-        stage_tile<DP, NW * 64>(Ks, p.k, b, p.Sk, p.Hkv, kvh, p.D, kb, tid);
-        stage_tile<DP, NW * 64>(Vs, p.v, b, p.Sk, p.Hkv, kvh, p.D, kb, tid);
-        __syncthreads();
-        if (q0 >= p.Sq || (p.causal && kb > q_last_wave)) continue;
+    float4 kc[NS], vc[NS], kn[NS], vn[NS];
+    auto load_quads = [&](int kb, float4 (&kk)[NS], float4 (&vv)[NS]) {
+        int key = kb + l32;
+        key = key < p.Sk ? key : p.Sk - 1;
+#pragma unroll
+        for (int s = 0; s < NS; s++) {
+            kk[s] = ld_quad<FULL>(kbase + key * kst, 8 * s + 4 * half, p.D);
+            vv[s] = ld_quad<FULL>(vbase + key * kst, 8 * s + 4 * half, p.D);
+        }
+    };
+    const int kb_first = wave * 32;
+    if (kb_first < k_end) load_quads(kb_first, kc, vc);
+    for (int kb = kb_first; kb < k_end; kb += 32 * NSPL) {
+        const bool more = kb + 32 * NSPL < k_end;
+        // K^T operand of dQ += K^T dS^T for this block: issued now, used last.
+        float k1[NF][16];
+#pragma unroll
+        for (int t = 0; t < 16; t++) {
+            int kt = kb + row_of(t, half);
+            kt = kt < p.Sk ? kt : p.Sk - 1;
+#pragma unroll
+            for (int f = 0; f < NF; f++) k1[f][t] = ld_one<FULL>(kbase + kt * kst, f * 32 + l32, p.D);
+        }
+        if (more) load_quads(kb + 32 * NSPL, kn, vn);
 
         floatx16 s = zero16(), dp = zero16();
 #pragma unroll
         for (int st = 0; st < NS; st++) {
-            const float4 a = *reinterpret_cast<const float4*>(Ks + l32 * LD + 8 * st + 4 * half);
-            s = MFMA(a.x, qreg[st].x, s);
-            s = MFMA(a.y, qreg[st].y, s);
-            s = MFMA(a.z, qreg[st].z, s);
-            s = MFMA(a.w, qreg[st].w, s);
-            const float4 c = *reinterpret_cast<const float4*>(Vs + l32 * LD + 8 * st + 4 * half);
-            dp = MFMA(c.x, doreg[st].x, dp);
-            dp = MFMA(c.y, doreg[st].y, dp);
-            dp = MFMA(c.z, doreg[st].z, dp);
-            dp = MFMA(c.w, doreg[st].w, dp);
+            s = MFMA(kc[st].x, qreg[st].x, s);
+            s = MFMA(kc[st].y, qreg[st].y, s);
+            s = MFMA(kc[st].z, qreg[st].z, s);
+            s = MFMA(kc[st].w, qreg[st].w, s);
+            dp = MFMA(vc[st].x, doreg[st].x, dp);
+            dp = MFMA(vc[st].y, doreg[st].y, dp);
+            dp = MFMA(vc[st].z, doreg[st].z, dp);
+            dp = MFMA(vc[st].w, doreg[st].w, dp);
         }
 #pragma unroll
         for (int t = 0; t < 16; t++) {
@@ -270,10 +337,36 @@ __global__ __launch_bounds__(NW * 64) void attn_bwd_dq_kernel(AttnArgs p) {
 #pragma unroll
         for (int f = 0; f < NF; f++)
 #pragma unroll
-            for (int t = 0; t < 16; t++) {
-                const float a = Ks[row_of(t, half) * LD + f * 32 + l32];
-                acc[f] = MFMA(a, s[t], acc[f]);
+            for (int t = 0; t < 16; t++) acc[f] = MFMA(k1[f][t], s[t], acc[f]);
+        if (more) {
+#pragma unroll
+            for (int st = 0; st < NS; st++) {
+                kc[st] = kn[st];
+                vc[st] = vn[st];
             }
+        }
+    }
+
+    // Sum of the waves' partial dQ, in wave order.
+    if constexpr (NSPL > 1) {
+        constexpr int W = NF * 16;
+        if (wave > 0) {
+            float* dst = merge + ((wave - 1) * 64 + lane) * W;
+#pragma unroll
+            for (int f = 0; f < NF; f++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) dst[f * 16 + r] = acc[f][r];
+        }
+        __syncthreads();
+        if (wave > 0) return;
+#pragma unroll
+        for (int w = 1; w < NSPL; w++) {
+            const float* src = merge + ((w - 1) * 64 + lane) * W;
+#pragma unroll
+            for (int f = 0; f < NF; f++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) acc[f][r] += src[f * 16 + r];
+        }
     }
 
     if (!q_ok) return;
@@ -298,18 +391,20 @@ __global__ __launch_bounds__(NW * 64) void attn_bwd_dq_kernel(AttnArgs p) {
 // ---------------------------------------------------------------------------
 // Backward, pass 2: dK and dV of 32 keys of one (batch, kv head), summed over
 // the query heads of the group and over the query blocks that can see them.
-// The (head, query block) items are dealt round-robin to the 4 waves, each with
-// its own Q / dO staging area; the 4 partial results are added in wave order
-// through LDS (no atomics: the result is deterministic).
-// Grid (ceil(Sk/32), B*Hkv), 256 threads.
+// The (head, query block) items are dealt round-robin to the NWV waves of the
+// workgroup; the partial results are added in wave order through LDS (no
+// atomics: the result is deterministic). Grid (ceil(Sk/32), B*Hkv), key blocks
+// issued first-first (under the causal mask key block 0 has the most items).
 // ---------------------------------------------------------------------------
-template <int DP>
-__global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(AttnArgs p) {
-    constexpr int LD = DP + 4;
+// 8 waves for head dims up to 64; 4 for 128 (the reduction buffer must fit LDS).
+constexpr int dkdv_waves(int dp) { return dp <= 64 ? 8 : 4; }
+
+template <int DP, bool FULL>
+__global__ __launch_bounds__(dkdv_waves(DP) * 64) void attn_bwd_dkdv_kernel(AttnArgs p) {
     constexpr int NF = DP / 32;
     constexpr int NS = DP / 8;
-    constexpr int REGION = 2 * 32 * LD;  // floats per wave: Q tile + dO tile
-    static_assert(2 * DP * 33 <= REGION, "reduction buffer must fit the staging area");
+    constexpr int NWV = dkdv_waves(DP);
+    constexpr int REGION = 2 * DP * 33;  // floats per wave: dK^T and dV^T, [d][33]
     extern __shared__ __attribute__((aligned(16))) float smem[];
 
     const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
@@ -319,17 +414,16 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(AttnArgs p) {
     const int kb0 = blockIdx.x * 32;
     const int key = kb0 + l32;
     const bool k_ok = key < p.Sk;
-    const long koff = (((long)b * p.Sk + (k_ok ? key : 0)) * p.Hkv + kvh) * p.D;
-    float* Qs = smem + wave * REGION;
-    float* dOs = Qs + 32 * LD;
+    const long koff = (((long)b * p.Sk + (k_ok ? key : p.Sk - 1)) * p.Hkv + kvh) * p.D;
+    const long qst = (long)p.H * p.D;
 
     float4 kreg[NS], vreg[NS];
 #pragma unroll
     for (int s = 0; s < NS; s++) {
         const int d = 8 * s + 4 * half;
-        const float4 t = load_row4(p.k + koff, d, p.D, k_ok);
+        const float4 t = ld_quad<FULL>(p.k + koff, d, p.D);
         kreg[s] = make_float4(t.x * p.scale, t.y * p.scale, t.z * p.scale, t.w * p.scale);
-        vreg[s] = load_row4(p.v + koff, d, p.D, k_ok);
+        vreg[s] = ld_quad<FULL>(p.v + koff, d, p.D);
     }
     floatx16 dk[NF], dv[NF];
 #pragma unroll
@@ -347,45 +441,25 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(AttnArgs p) {
     }
     const int per_head = nqb > qb_start ? nqb - qb_start : 0;
     const int items = per_head * G;
-    const int rounds = (items + 3) / 4;
 
-    for (int it = 0; it < rounds; it++) {
-        const int item = it * 4 + wave;
-        const bool active = item < items;  // wave-uniform
-        const int g = active ? item / per_head : 0;
-        const int qb = active ? qb_start + item % per_head : 0;
+    for (int item = wave; item < items; item += NWV) {
+        const int g = item / per_head;
+        const int q0 = (qb_start + item % per_head) * 32;
         const int h = kvh * G + g;
-        const int q0 = qb * 32;
-        __syncthreads();
-        if (active) {
-            stage_tile<DP, 64>(Qs, p.q, b, p.Sq, p.H, h, p.D, q0, lane);
-            stage_tile<DP, 64>(dOs, p.d_out, b, p.Sq, p.H, h, p.D, q0, lane);
-        }
-        __syncthreads();
-        if (!active) continue;
+        const float* qbase = p.q + ((long)b * p.Sq * p.H + h) * p.D;
+        const float* dobase = p.d_out + ((long)b * p.Sq * p.H + h) * p.D;
+        int qr = q0 + l32;
+        qr = qr < p.Sq ? qr : p.Sq - 1;
 
-        float lse[16], dlt[16];
-#pragma unroll
-        for (int t = 0; t < 16; t++) {
-            const int qi = q0 + row_of(t, half);
-            if (qi < p.Sq) {
-                const float2 st = *reinterpret_cast<const float2*>(p.stats + 2 * (((long)b * p.H + h) * p.Sq + qi));
-                dlt[t] = st.x;
-                lse[t] = st.y;
-            } else {
-                dlt[t] = 0.0f;
-                lse[t] = kLseEmpty;
-            }
-        }
         floatx16 s = zero16(), dp = zero16();
 #pragma unroll
         for (int st = 0; st < NS; st++) {
-            const float4 a = *reinterpret_cast<const float4*>(Qs + l32 * LD + 8 * st + 4 * half);
+            const float4 a = ld_quad<FULL>(qbase + qr * qst, 8 * st + 4 * half, p.D);
+            const float4 c = ld_quad<FULL>(dobase + qr * qst, 8 * st + 4 * half, p.D);
             s = MFMA(a.x, kreg[st].x, s);
             s = MFMA(a.y, kreg[st].y, s);
             s = MFMA(a.z, kreg[st].z, s);
             s = MFMA(a.w, kreg[st].w, s);
-            const float4 c = *reinterpret_cast<const float4*>(dOs + l32 * LD + 8 * st + 4 * half);
             dp = MFMA(c.x, vreg[st].x, dp);
             dp = MFMA(c.y, vreg[st].y, dp);
             dp = MFMA(c.z, vreg[st].z, dp);
@@ -394,23 +468,30 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(AttnArgs p) {
 #pragma unroll
         for (int t = 0; t < 16; t++) {
             const int qi = q0 + row_of(t, half);
+            float lse = kLseEmpty, dlt = 0.0f;
+            if (qi < p.Sq) {
+                const float2 st2 = *reinterpret_cast<const float2*>(p.stats + 2 * (((long)b * p.H + h) * p.Sq + qi));
+                dlt = st2.x;
+                lse = st2.y;
+            }
             const bool vis = k_ok && qi < p.Sq && (!p.causal || key <= qi + p.causal_offset);
-            const float pij = vis ? __expf(s[t] - lse[t]) : 0.0f;
-            s[t] = pij;                       // P
-            dp[t] = pij * (dp[t] - dlt[t]);   // dS
+            const float pij = vis ? __expf(s[t] - lse) : 0.0f;
+            s[t] = pij;                   // P
+            dp[t] = pij * (dp[t] - dlt);  // dS
         }
 #pragma unroll
-        for (int f = 0; f < NF; f++)
+        for (int t = 0; t < 16; t++) {
+            int qt = q0 + row_of(t, half);
+            qt = qt < p.Sq ? qt : p.Sq - 1;
 #pragma unroll
-            for (int t = 0; t < 16; t++) {
-                const int r = row_of(t, half);
-                dv[f] = MFMA(dOs[r * LD + f * 32 + l32], s[t], dv[f]);
-                dk[f] = MFMA(Qs[r * LD + f * 32 + l32], dp[t], dk[f]);
+            for (int f = 0; f < NF; f++) {
+                dv[f] = MFMA(ld_one<FULL>(dobase + qt * qst, f * 32 + l32, p.D), s[t], dv[f]);
+                dk[f] = MFMA(ld_one<FULL>(qbase + qt * qst, f * 32 + l32, p.D), dp[t], dk[f]);
             }
+        }
     }
 
-    // Cross-wave sum. red[wave][which][d][33]
-    __syncthreads();
+    // Cross-wave sum: red[wave][which][d][33]
     float* red = smem + wave * REGION;
 #pragma unroll
     for (int f = 0; f < NF; f++)
@@ -421,60 +502,75 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(AttnArgs p) {
             red[DP * 33 + d * 33 + l32] = dv[f][t];
         }
     __syncthreads();
-    for (int e = tid; e < 32 * DP; e += 256) {
+    for (int e = tid; e < 32 * DP; e += NWV * 64) {
         const int kk = e / DP, d = e % DP;
         const int krow = kb0 + kk;
         if (krow < p.Sk && d < p.D) {
             float sk = 0.0f, sv = 0.0f;
 #pragma unroll
-            for (int w = 0; w < 4; w++) {
+            for (int w = 0; w < NWV; w++) {
                 sk += smem[w * REGION + d * 33 + kk];
                 sv += smem[w * REGION + DP * 33 + d * 33 + kk];
             }
             const long o = (((long)b * p.Sk + krow) * p.Hkv + kvh) * p.D + d;
-            p.dk[o] = sk * p.scale;  // dK = scale * sum dS Q (Q is staged unscaled)
+            p.dk[o] = sk * p.scale;  // dK = scale * sum dS Q (Q is read unscaled)
             p.dv[o] = sv;
         }
     }
 }
 
+// The unguarded vector loads need whole, aligned quads in every row.
+bool attn_full(const AttnArgs& a, int DP) {
+    auto al = [](const void* q) { return q == nullptr || (((uintptr_t)q) & 15) == 0; };
+    return a.D == DP && al(a.q) && al(a.k) && al(a.v) && al(a.out) && al(a.d_out);
+}
+
 template <int DP>
 int launch_fwd(ft_context* ctx, const AttnArgs& a) {
-    constexpr int NW = 2;
-    const dim3 grid(ft_div_up(a.Sq, 32 * NW), (unsigned)(a.B * a.H));
+    const dim3 grid(ft_div_up(a.Sq, 32), (unsigned)(a.B * a.H));
     // flop convention of the reference's benchmarks: causal forward 2*B*H*Sq*Sk*D, full 4*...
     const double fl = (a.causal ? 2.0 : 4.0) * a.B * a.H * (double)a.Sq * a.Sk * a.D;
     const double by = 4.0 * a.B * ((double)a.Sq * a.H * a.D * 2 + (double)a.Sk * a.Hkv * a.D * 2);
     ft_prof_scope prof(ctx, "attn_fwd_kernel", fl, by);
-    hipLaunchKernelGGL((attn_fwd_kernel<DP, NW>), grid, dim3(NW * 64), 0, ctx->stream, a);
+    if (attn_full(a, DP))
+        hipLaunchKernelGGL((attn_fwd_kernel<DP, true>), grid, dim3(kKeySplit * 64), 0, ctx->stream, a);
+    else
+        hipLaunchKernelGGL((attn_fwd_kernel<DP, false>), grid, dim3(kKeySplit * 64), 0, ctx->stream, a);
     FT_LAUNCH_CHECK();
     return FT_OK;
 }
 
 template <int DP>
 int launch_bwd(ft_context* ctx, const AttnArgs& a) {
-    constexpr int NW = 2;
-    const dim3 grid(ft_div_up(a.Sq, 32 * NW), (unsigned)(a.B * a.H));
-    // backward = 2.5x forward by the reference's convention: 1.5x (3 products) in dQ, 2x (4 products)
-    // in dK/dV, minus the shared recomputation -> charged 1.0x and 1.5x.
+    const dim3 grid(ft_div_up(a.Sq, 32), (unsigned)(a.B * a.H));
+    // backward = 2.5x forward by the reference's convention, charged 1.0x to the dQ pass and 1.5x to dK/dV.
     const double fl = (a.causal ? 2.0 : 4.0) * a.B * a.H * (double)a.Sq * a.Sk * a.D;
     const double by = 4.0 * a.B * ((double)a.Sq * a.H * a.D * 4 + (double)a.Sk * a.Hkv * a.D * 4);
+    const bool full = attn_full(a, DP);
     {
         ft_prof_scope prof(ctx, "attn_bwd_dq_kernel", 1.0 * fl, by * 0.5);
-        hipLaunchKernelGGL((attn_bwd_dq_kernel<DP, NW>), grid, dim3(NW * 64), 0, ctx->stream, a);
+        if (full)
+            hipLaunchKernelGGL((attn_bwd_dq_kernel<DP, true>), grid, dim3(kKeySplit * 64), 0, ctx->stream, a);
+        else
+            hipLaunchKernelGGL((attn_bwd_dq_kernel<DP, false>), grid, dim3(kKeySplit * 64), 0, ctx->stream, a);
     }
     FT_LAUNCH_CHECK();
-    constexpr size_t smem = (size_t)4 * 2 * 32 * (DP + 4) * sizeof(float);
+    constexpr size_t smem = (size_t)dkdv_waves(DP) * 2 * DP * 33 * sizeof(float);
     static bool attr_set = false;
     if (!attr_set) {
-        FT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_bwd_dkdv_kernel<DP>),
+        FT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_bwd_dkdv_kernel<DP, true>),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+        FT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_bwd_dkdv_kernel<DP, false>),
                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
         attr_set = true;
     }
     const dim3 grid2(ft_div_up(a.Sk, 32), (unsigned)(a.B * a.Hkv));
     {
         ft_prof_scope prof(ctx, "attn_bwd_dkdv_kernel", 1.5 * fl, by * 0.5);
-        hipLaunchKernelGGL((attn_bwd_dkdv_kernel<DP>), grid2, dim3(256), smem, ctx->stream, a);
+        if (full)
+            hipLaunchKernelGGL((attn_bwd_dkdv_kernel<DP, true>), grid2, dim3(dkdv_waves(DP) * 64), smem, ctx->stream, a);
+        else
+            hipLaunchKernelGGL((attn_bwd_dkdv_kernel<DP, false>), grid2, dim3(dkdv_waves(DP) * 64), smem, ctx->stream, a);
     }
     FT_LAUNCH_CHECK();
     return FT_OK;

@@ -266,46 +266,63 @@ __device__ __attribute__((aligned(16))) float g_zero16[4] = {0.f, 0.f, 0.f, 0.f}
 
 typedef float float2_t __attribute__((ext_vector_type(2)));
 
-template <int ROWS, bool KCONTIG>
+template <int ROWS, bool KCONTIG, int BKT>
 struct FastTile {
+    static constexpr int KQT = BKT / 4;
     static constexpr int PAD = 4;
     static constexpr int KQ_STRIDE = ROWS * 4 + PAD;   // k-quad major: floats per quad row (== 4 mod 32)
     static constexpr int K_STRIDE = ROWS + PAD;        // k-major: floats per k row
-    static constexpr int LDS_FLOATS = KCONTIG ? KQ * KQ_STRIDE : BK * K_STRIDE;
-    static constexpr int SLOTS = KCONTIG ? ROWS * KQ / 256 : BK * (ROWS / 4) / 256;
+    static constexpr int LDS_FLOATS = KCONTIG ? KQT * KQ_STRIDE : BKT * K_STRIDE;
+    static constexpr int SLOTS = KCONTIG ? ROWS * KQT / 256 : BKT * (ROWS / 4) / 256;
     static_assert(SLOTS >= 1, "tile too small for 256 threads");
     // Raw loaded bits: 4 floats, or 4 halfs in .x/.y. Converted when stored to
     // LDS, so nothing between the load and the MFMA block depends on it.
     float4 r[SLOTS];
+    // Byte offset of each slot from the tile's (uniform) base pointer: constant
+    // over the K loop, so a load costs no per-lane address arithmetic.
+    unsigned off[SLOTS];
 
     __device__ __forceinline__ static void slot_coords(int i, int& row, int& k) {
         const int s = threadIdx.x + i * 256;
         if constexpr (KCONTIG) {
-            row = s / KQ;
-            k = (s % KQ) * 4;
+            row = s / KQT;
+            k = (s % KQT) * 4;
         } else {
             row = (s % (ROWS / 4)) * 4;
             k = s / (ROWS / 4);
         }
     }
 
-    template <typename T>
-    __device__ __forceinline__ void load(const T* base, long ld, int row0, int row_limit, int k0, int k_limit) {
+    // Offsets for an operand with leading dimension ld (elements of esize bytes);
+    // rows past row_limit are clamped to a valid row (their results are never stored).
+    __device__ __forceinline__ void set_offsets(long ld, int row0, int row_limit, int esize) {
 #pragma unroll
         for (int i = 0; i < SLOTS; i++) {
             int row, k;
             slot_coords(i, row, k);
             int gr = row0 + row;
-            const int gk = k0 + k;
-            long off;
             if constexpr (KCONTIG) {
                 gr = gr < row_limit ? gr : row_limit - 1;
-                off = (long)gr * ld + gk;
+                off[i] = (unsigned)(((long)gr * ld + k) * esize);
             } else {
                 gr = gr + 4 <= row_limit ? gr : row_limit - 4;
-                off = (long)gk * ld + gr;
+                off[i] = (unsigned)(((long)k * ld + gr) * esize);
             }
-            const T* src = gk < k_limit ? base + off : reinterpret_cast<const T*>(g_zero16);
+        }
+    }
+
+    // tile_base = operand base advanced to k0 (uniform). GUARD: k0 + k may run
+    // past k_limit; such slots read a line of zeros instead.
+    template <typename T, bool GUARD>
+    __device__ __forceinline__ void load(const char* tile_base, int k0, int k_limit) {
+#pragma unroll
+        for (int i = 0; i < SLOTS; i++) {
+            const char* src = tile_base + off[i];
+            if constexpr (GUARD) {
+                int row, k;
+                slot_coords(i, row, k);
+                if (k0 + k >= k_limit) src = reinterpret_cast<const char*>(g_zero16);
+            }
             if constexpr (sizeof(T) == 2) {
                 const float2_t raw = *reinterpret_cast<const float2_t*>(src);
                 r[i].x = raw.x;
@@ -350,16 +367,16 @@ struct FastTile {
     }
 };
 
-template <int BM, int BN, int WM, int WN, int LAYOUT, bool HALF_B>
+template <int BM, int BN, int WM, int WN, int LAYOUT, bool HALF_B, int BKT>
 __global__ __launch_bounds__(256) void gemm_fast_kernel(GemmArgs p) {
     constexpr bool A_KC = LAYOUT != 2;
     constexpr bool B_KC = LAYOUT == 1;
     constexpr int FM = WM / 32, FN = WN / 32;
     constexpr int WAVES_N = BN / WN;
-    constexpr int STEPS = KQ / 2;
+    constexpr int STEPS = BKT / 8;
     static_assert((BM / WM) * (BN / WN) == 4, "4 waves per workgroup");
-    using ATile = FastTile<BM, A_KC>;
-    using BTile = FastTile<BN, B_KC>;
+    using ATile = FastTile<BM, A_KC, BKT>;
+    using BTile = FastTile<BN, B_KC, BKT>;
     using BType = typename std::conditional<HALF_B, _Float16, float>::type;
 
     __shared__ __attribute__((aligned(16))) float As[2][ATile::LDS_FLOATS];
@@ -380,21 +397,36 @@ __global__ __launch_bounds__(256) void gemm_fast_kernel(GemmArgs p) {
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
 
-    const int nt1 = (p.K + BK - 1) / BK;
-    const int nt2 = (LAYOUT != 2 && p.a2) ? (p.K2 + BK - 1) / BK : 0;
+    const int nt1 = (p.K + BKT - 1) / BKT;
+    const int nt1_full = p.K / BKT;  // tiles that need no k guard
+    const int nt2 = (LAYOUT != 2 && p.a2) ? (p.K2 + BKT - 1) / BKT : 0;
     const int nt = nt1 + nt2;
-    const BType* bmat = reinterpret_cast<const BType*>(p.b);
+    const long a_kstep = (A_KC ? 1 : p.lda) * 4;                                // bytes per k
+    const long b_kstep = (B_KC ? 1 : p.ldb) * (long)sizeof(BType);
+    const long b2_kstep = (B_KC ? 1 : p.ldb2) * 4;
 
     ATile ta;
     BTile tb;
-    // Tiles past nt1 belong to the second (LoRA) product: f32 operands, same orientation.
+    ta.set_offsets(p.lda, m0, p.M, 4);
+    tb.set_offsets(p.ldb, n0, p.N, (int)sizeof(BType));
+
+    // Tiles past nt1 belong to the second (LoRA) product: f32 operands, same
+    // orientation, their own leading dimensions (offsets are re-derived once).
     auto fetch = [&](int t) {
-        if (t < nt1) {
-            ta.load(p.a, p.lda, m0, p.M, t * BK, p.K);
-            tb.load(bmat, p.ldb, n0, p.N, t * BK, p.K);
+        if (t < nt1_full) {
+            ta.template load<float, false>(reinterpret_cast<const char*>(p.a) + (long)t * BKT * a_kstep, 0, 0);
+            tb.template load<BType, false>(reinterpret_cast<const char*>(p.b) + (long)t * BKT * b_kstep, 0, 0);
+        } else if (t < nt1) {
+            ta.template load<float, true>(reinterpret_cast<const char*>(p.a) + (long)t * BKT * a_kstep, t * BKT, p.K);
+            tb.template load<BType, true>(reinterpret_cast<const char*>(p.b) + (long)t * BKT * b_kstep, t * BKT, p.K);
         } else if constexpr (LAYOUT != 2) {
-            ta.load(p.a2, p.lda2, m0, p.M, (t - nt1) * BK, p.K2);
-            tb.load(p.b2, p.ldb2, n0, p.N, (t - nt1) * BK, p.K2);
+            const int k0 = (t - nt1) * BKT;
+            if (t == nt1) {
+                ta.set_offsets(p.lda2, m0, p.M, 4);
+                tb.set_offsets(p.ldb2, n0, p.N, 4);
+            }
+            ta.template load<float, true>(reinterpret_cast<const char*>(p.a2) + (long)k0 * 4, k0, p.K2);
+            tb.template load<float, true>(reinterpret_cast<const char*>(p.b2) + (long)k0 * b2_kstep, k0, p.K2);
         }
     };
     auto stash = [&](int t, int buf) {
@@ -404,6 +436,17 @@ __global__ __launch_bounds__(256) void gemm_fast_kernel(GemmArgs p) {
         else
             tb.template store<float>(Bs[buf]);
     };
+    auto mfma_step = [&](const float4 (&af)[FM], const float4 (&bf)[FN]) {
+#pragma unroll
+        for (int i = 0; i < FM; i++)
+#pragma unroll
+            for (int j = 0; j < FN; j++) {
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i].x, bf[j].x, acc[i][j], 0, 0, 0);
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i].y, bf[j].y, acc[i][j], 0, 0, 0);
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i].z, bf[j].z, acc[i][j], 0, 0, 0);
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i].w, bf[j].w, acc[i][j], 0, 0, 0);
+            }
+    };
 
     if (nt > 0) {
         fetch(0);
@@ -412,14 +455,14 @@ __global__ __launch_bounds__(256) void gemm_fast_kernel(GemmArgs p) {
     __syncthreads();
     for (int t = 0; t < nt; t++) {
         const int buf = t & 1;
-        // Global loads of the next tile are issued first and consumed only after
-        // the MFMA block: the scheduling barriers keep the compiler from pulling
-        // the f16 conversion (and its wait) in front of the matrix work.
-        if (t + 1 < nt) fetch(t + 1);
-        __builtin_amdgcn_sched_barrier(0);
         const float* as = As[buf];
         const float* bs = Bs[buf];
         float4 af[2][FM], bf[2][FN];
+        // Order inside one K tile (the scheduling barriers pin it): operand
+        // reads of step 0 and 1, MFMAs of step 0, THEN the global loads of the
+        // next tile (their address setup runs under step 0's matrix work
+        // instead of in front of it), remaining steps, and the next tile's LDS
+        // stores (f16 -> f32 conversion included) before the last step.
 #pragma unroll
         for (int i = 0; i < FM; i++) af[0][i] = ATile::frag(as, 0, half, wm0 + i * 32 + l32);
 #pragma unroll
@@ -433,18 +476,18 @@ __global__ __launch_bounds__(256) void gemm_fast_kernel(GemmArgs p) {
 #pragma unroll
                 for (int j = 0; j < FN; j++) bf[nxt][j] = BTile::frag(bs, s + 1, half, wn0 + j * 32 + l32);
             }
-#pragma unroll
-            for (int i = 0; i < FM; i++)
-#pragma unroll
-                for (int j = 0; j < FN; j++) {
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[cur][i].x, bf[cur][j].x, acc[i][j], 0, 0, 0);
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[cur][i].y, bf[cur][j].y, acc[i][j], 0, 0, 0);
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[cur][i].z, bf[cur][j].z, acc[i][j], 0, 0, 0);
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[cur][i].w, bf[cur][j].w, acc[i][j], 0, 0, 0);
-                }
+            __builtin_amdgcn_sched_barrier(0);
+            mfma_step(af[cur], bf[cur]);
+            __builtin_amdgcn_sched_barrier(0);
+            if (s == 0 && t + 1 < nt) {
+                fetch(t + 1);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            if (s == STEPS - 2 && t + 1 < nt) {
+                stash(t + 1, buf ^ 1);
+                __builtin_amdgcn_sched_barrier(0);
+            }
         }
-        __builtin_amdgcn_sched_barrier(0);
-        if (t + 1 < nt) stash(t + 1, buf ^ 1);
         __syncthreads();
     }
 
@@ -570,19 +613,18 @@ __global__ __launch_bounds__(256) void skinny_kernel(const float* __restrict__ x
 // Host side
 // ---------------------------------------------------------------------------
 
-struct TileCfg {
-    int bm, bn;
-    float eff;  // relative per-tile efficiency used only to rank configurations
-};
-
-template <int BM, int BN, int WM, int WN>
+template <int BM, int BN, int WM, int WN, int BKF = 32>
 int launch_cfg(ft_context* ctx, GemmArgs p, int layout, bool half_b, bool fast) {
     const int tiles_m = (p.M + BM - 1) / BM;
     p.tiles_n = (p.N + BN - 1) / BN;
     const dim3 grid((unsigned)(tiles_m * p.tiles_n));
     char name[96];
-    snprintf(name, sizeof(name), "%s<%d, %d, %d, %d, %d, %s>", fast ? "gemm_fast_kernel" : "gemm_kernel", BM, BN, WM,
-             WN, layout, half_b ? "true" : "false");
+    if (fast)
+        snprintf(name, sizeof(name), "gemm_fast_kernel<%d, %d, %d, %d, %d, %s, %d>", BM, BN, WM, WN, layout,
+                 half_b ? "true" : "false", BKF);
+    else
+        snprintf(name, sizeof(name), "gemm_kernel<%d, %d, %d, %d, %d, %s>", BM, BN, WM, WN, layout,
+                 half_b ? "true" : "false");
     const double kk = (double)p.K + (p.a2 ? (double)p.K2 : 0.0);
     ft_prof_scope prof(ctx, name, 2.0 * p.M * (double)p.N * kk,
                        4.0 * p.M * kk + (half_b ? 2.0 : 4.0) * p.N * (double)p.K + 4.0 * p.N * (p.a2 ? p.K2 : 0) +
@@ -590,7 +632,7 @@ int launch_cfg(ft_context* ctx, GemmArgs p, int layout, bool half_b, bool fast) 
 #define FT_GEMM_LAUNCH(L, H)                                                                             \
     do {                                                                                                 \
         if (fast)                                                                                        \
-            hipLaunchKernelGGL((gemm_fast_kernel<BM, BN, WM, WN, L, H>), grid, dim3(256), 0, ctx->stream, p); \
+            hipLaunchKernelGGL((gemm_fast_kernel<BM, BN, WM, WN, L, H, BKF>), grid, dim3(256), 0, ctx->stream, p); \
         else                                                                                             \
             hipLaunchKernelGGL((gemm_kernel<BM, BN, WM, WN, L, H>), grid, dim3(256), 0, ctx->stream, p);      \
     } while (0)
@@ -629,20 +671,15 @@ int gemm_dispatch(ft_context* ctx, const char* who, int layout, bool half_b, con
     p.ldc = (long)N;
     p.lda2 = (long)K2;
     p.ldb2 = layout == 1 ? (long)K2 : (long)N;
-    // Pick the tile that needs the fewest rounds over the CUs, weighted by how
-    // well each shape amortises its loads.
-    const TileCfg cfgs[3] = {{128, 128, 1.00f}, {128, 64, 0.95f}, {64, 64, 0.88f}};
-    int best = 0;
-    float best_cost = 0.0f;
-    for (int c = 0; c < 3; c++) {
-        const size_t tiles = ((M + cfgs[c].bm - 1) / cfgs[c].bm) * ((N + cfgs[c].bn - 1) / cfgs[c].bn);
-        const size_t rounds = (tiles + ctx->num_cus - 1) / ctx->num_cus;
-        const float cost = (float)rounds * (float)(cfgs[c].bm * cfgs[c].bn) / cfgs[c].eff;
-        if (c == 0 || cost < best_cost) {
-            best = c;
-            best_cost = cost;
-        }
-    }
+    // Tile choice, from measurements on MI355X at M = 2048: 128x128 tiles (64x64
+    // per wave) reach the highest MFMA occupancy but only pay off when there are
+    // many of them per CU (the vocabulary head); everything smaller runs best as
+    // 64x64 tiles, which keep several workgroups resident per CU. A deep K loop
+    // on few tiles prefers BK = 64 (half the barriers per MFMA).
+    const size_t tiles128 = ((M + 127) / 128) * ((N + 127) / 128);
+    const size_t tiles64 = ((M + 63) / 64) * ((N + 63) / 64);
+    int best = tiles128 >= 8 * (size_t)ctx->num_cus ? 0 : 2;
+    if (best == 2 && K >= 4096 && tiles64 <= 2 * (size_t)ctx->num_cus) best = 3;
     // The branch-free kernel needs aligned operands and whole float4 groups.
     auto al16 = [](const void* q) { return (((uintptr_t)q) & 15) == 0; };
     bool fast = al16(a) && al16(b) && al16(out) && K % 4 == 0 && K >= 4 && (p.lda % 4 == 0) && (p.ldb % 4 == 0);
@@ -650,8 +687,12 @@ int gemm_dispatch(ft_context* ctx, const char* who, int layout, bool half_b, con
     if (layout == 2) fast = fast && M % 4 == 0 && M >= 4;   // a rows run along m
     if (half_b) fast = fast && (p.ldb % 8 == 0 || layout == 1);
     if (p.a2) fast = fast && al16(a2) && al16(b2) && K2 % 4 == 0 && K2 >= 4;
+    // Per-lane operand offsets are 32-bit byte offsets from a uniform base.
+    const double lim = 4294967296.0;
+    fast = fast && 4.0 * (double)M * (double)(layout == 2 ? 1 : K) + 4.0 * 64 * (double)p.lda < lim &&
+           4.0 * (double)N * (double)(layout == 1 ? K : 1) + 4.0 * 64 * (double)p.ldb < lim;
     if (best == 0) return launch_cfg<128, 128, 64, 64>(ctx, p, layout, half_b, fast);
-    if (best == 1) return launch_cfg<128, 64, 64, 32>(ctx, p, layout, half_b, fast);
+    if (best == 3) return launch_cfg<64, 64, 32, 32, 64>(ctx, p, layout, half_b, fast);
     return launch_cfg<64, 64, 32, 32>(ctx, p, layout, half_b, fast);
 }
 
