@@ -506,6 +506,234 @@ __global__ __launch_bounds__(256) void gemm_fast_kernel(GemmArgs p) {
 }
 
 // ---------------------------------------------------------------------------
+// Asynchronous path for the shapes the training step is made of: f32 a[M,K],
+// packed f16 b, K a multiple of 32. Both operand tiles go from global memory
+// straight into LDS with global_load_lds_dwordx4 (no VGPR staging, no LDS
+// stores, no per-tile address arithmetic), NST tiles deep, so a workgroup
+// always has NST-1 tiles of loads in flight behind the one it multiplies.
+// b stays f16 in LDS and is converted as it is read into MFMA operands.
+//
+// A lane's 16 bytes land at (LDS base of the instruction) + 16 * lane, so the
+// LDS image of a tile is fixed by which global address each lane is given:
+//   a tile   [BM rows][32 k] f32, 128 B per row, 8 rows per instruction; the
+//            16-byte column c of row r holds k-quad c ^ (r & 7), which makes the
+//            ds_read_b128 of 8 consecutive rows hit 8 different bank groups.
+//   b tile   layout 1 (b[N,K]): [BN rows][32 k] f16, 64 B per row, 16 rows per
+//            instruction, 16-byte column c holds k-octet c ^ ((r >> 1) & 3).
+//            layout 0 (b[K,N]): [32 k][BN n] f16 exactly as in memory; a lane
+//            reads its column's 4 k values as four 16-bit loads.
+// The K loop is unrolled over the stages; the waits are explicit (s_waitcnt
+// vmcnt(n) + s_barrier, not __syncthreads, whose fence would drain every
+// outstanding load).
+// The rank-r second product is loaded into registers before the loop and
+// multiplied from a small LDS tile after it (K2 <= 16).
+// ---------------------------------------------------------------------------
+
+// global_load_lds_dwordx4 with a uniform 64-bit base, a per-lane 32-bit byte
+// offset and a uniform LDS destination (M0). Written as inline assembly so the
+// compiler does not track it: with the builtin it drains every outstanding
+// LDS-DMA load (vmcnt(0)) in front of the first LDS read after the loop
+// back-edge, which defeats the multi-stage pipeline. The waits are explicit.
+__device__ __forceinline__ void glds16(const char* base, unsigned voff, const float* lds_dst) {
+    const unsigned l = __builtin_amdgcn_readfirstlane((unsigned)(uintptr_t)lds_dst);
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(base), "s"(l) : "memory", "m0");
+}
+
+template <int BM, int BN, int WM, int WN, int LAYOUT, int NST>
+__global__ __launch_bounds__(256) void gemm_async_kernel(GemmArgs p) {
+    static_assert(LAYOUT == 0 || LAYOUT == 1, "a is k-contiguous on this path");
+    static_assert(NST == 3 || NST == 4, "3 or 4 stages");
+    constexpr int FM = WM / 32, FN = WN / 32;
+    constexpr int WAVES_N = BN / WN;
+    static_assert((BM / WM) * (BN / WN) == 4, "4 waves per workgroup");
+    constexpr int A_FLOATS = BM * 32;             // f32 tile
+    constexpr int B_FLOATS = BN * 16;             // f16 tile, in float units
+    constexpr int STAGE = A_FLOATS + B_FLOATS;
+    constexpr int A_CH = BM / 8 / 4;              // 1 KiB chunks per wave
+    constexpr int B_CH = BN / 16 / 4;
+    constexpr int LPT = A_CH + B_CH;              // load instructions per wave per tile
+    constexpr int WAIT = (NST - 2) * LPT;         // loads that may still be in flight when tile t is needed
+    using ExA = FastTile<BM, true, 16>;
+    using ExB = FastTile<BN, LAYOUT == 1, 16>;
+
+    __shared__ __attribute__((aligned(16))) float St0[STAGE];
+    __shared__ __attribute__((aligned(16))) float St1[STAGE];
+    __shared__ __attribute__((aligned(16))) float St2[STAGE];
+    __shared__ __attribute__((aligned(16))) float St3[NST == 4 ? STAGE : 4];
+    __shared__ __attribute__((aligned(16))) float ExAs[ExA::LDS_FLOATS];
+    __shared__ __attribute__((aligned(16))) float ExBs[ExB::LDS_FLOATS];
+
+    const int tile = blockIdx.x;
+    const int m0 = (tile / p.tiles_n) * BM;
+    const int n0 = (tile % p.tiles_n) * BN;
+    const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
+    const int wm0 = (wave / WAVES_N) * WM, wn0 = (wave % WAVES_N) * WN;
+    const int l32 = lane % 32, half = lane / 32;
+
+    floatx16 acc[FM][FN];
+#pragma unroll
+    for (int i = 0; i < FM; i++)
+#pragma unroll
+        for (int j = 0; j < FN; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
+
+    const int nt = p.K / 32;
+    const bool has_ext = p.a2 != nullptr;
+
+    // The rank-r product's operands: ordinary loads, issued first, consumed last.
+    ExA xa;
+    ExB xb;
+    if (has_ext) {
+        xa.set_offsets(p.lda2, m0, p.M, 4);
+        xb.set_offsets(p.ldb2, n0, p.N, 4);
+        xa.template load<float, true>(reinterpret_cast<const char*>(p.a2), 0, p.K2);
+        xb.template load<float, true>(reinterpret_cast<const char*>(p.b2), 0, p.K2);
+    }
+
+    // Per-lane source offsets (bytes), constant over the K loop.
+    unsigned offA[A_CH], offB[B_CH];
+#pragma unroll
+    for (int j = 0; j < A_CH; j++) {
+        const int c = wave + 4 * j, r = lane / 8, cs = lane % 8;
+        int row = m0 + 8 * c + r;
+        row = row < p.M ? row : p.M - 1;
+        offA[j] = (unsigned)(((long)row * p.lda + ((cs ^ r) * 4)) * 4);
+    }
+    long b_step;
+#pragma unroll
+    for (int j = 0; j < B_CH; j++) {
+        const int c = wave + 4 * j;
+        if constexpr (LAYOUT == 1) {
+            const int r = lane / 4, cs = lane % 4;
+            int n = n0 + 16 * c + r;
+            n = n < p.N ? n : p.N - 1;
+            offB[j] = (unsigned)(((long)n * p.ldb + ((cs ^ ((r >> 1) & 3)) * 8)) * 2);
+        } else {
+            constexpr int LPR = BN / 8, RPC = 64 / LPR;
+            const int kr = lane / LPR, cs = lane % LPR;
+            int col = n0 + cs * 8;
+            col = col + 8 <= p.N ? col : p.N - 8;
+            offB[j] = (unsigned)(((long)(c * RPC + kr) * p.ldb + col) * 2);
+        }
+    }
+    b_step = LAYOUT == 1 ? 64 : 64 * p.ldb;  // bytes per K tile
+    const char* abase = reinterpret_cast<const char*>(p.a);
+    const char* bbase = reinterpret_cast<const char*>(p.b);
+
+    auto issue = [&](int t, float* st) {
+        t = t < nt ? t : nt - 1;  // past the end: re-read the last tile into a stage nobody reads
+        const char* at = abase + (long)t * 128;
+        const char* bt = bbase + (long)t * b_step;
+#pragma unroll
+        for (int j = 0; j < A_CH; j++) glds16(at, offA[j], st + (wave + 4 * j) * 256);
+#pragma unroll
+        for (int j = 0; j < B_CH; j++) glds16(bt, offB[j], st + A_FLOATS + (wave + 4 * j) * 256);
+    };
+    auto a_frag = [&](const float* st, int s, int row) -> float4 {
+        const int kq = 2 * s + half;
+        return *reinterpret_cast<const float4*>(st + row * 32 + ((kq ^ (row & 7)) * 4));
+    };
+    auto b_frag = [&](const float* st, int s, int n) -> float4 {
+        const char* bs = reinterpret_cast<const char*>(st + A_FLOATS);
+        if constexpr (LAYOUT == 1) {
+            const int kq = 2 * s + half;
+            const int col = (kq >> 1) ^ ((n >> 1) & 3);
+            const half4_t h = *reinterpret_cast<const half4_t*>(bs + n * 64 + col * 16 + (kq & 1) * 8);
+            return make_float4((float)h.x, (float)h.y, (float)h.z, (float)h.w);
+        } else {
+            const _Float16* q = reinterpret_cast<const _Float16*>(bs) + (8 * s + 4 * half) * BN + n;
+            return make_float4((float)q[0], (float)q[BN], (float)q[2 * BN], (float)q[3 * BN]);
+        }
+    };
+    auto mfma_step = [&](const float4 (&af)[FM], const float4 (&bf)[FN]) {
+#pragma unroll
+        for (int i = 0; i < FM; i++)
+#pragma unroll
+            for (int j = 0; j < FN; j++) {
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i].x, bf[j].x, acc[i][j], 0, 0, 0);
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i].y, bf[j].y, acc[i][j], 0, 0, 0);
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i].z, bf[j].z, acc[i][j], 0, 0, 0);
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i].w, bf[j].w, acc[i][j], 0, 0, 0);
+            }
+    };
+    // One K tile: wait for it, let everybody leave the stage that is about to
+    // be refilled, refill it (tile t + NST - 1), multiply tile t.
+    auto iter = [&](int t, const float* cur, float* refill) {
+        __builtin_amdgcn_s_waitcnt(0x0F70 | (WAIT & 15) | ((WAIT >> 4) << 14));
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+        issue(t + NST - 1, refill);
+        __builtin_amdgcn_sched_barrier(0);
+        float4 af[2][FM], bf[2][FN];
+#pragma unroll
+        for (int i = 0; i < FM; i++) af[0][i] = a_frag(cur, 0, wm0 + i * 32 + l32);
+#pragma unroll
+        for (int j = 0; j < FN; j++) bf[0][j] = b_frag(cur, 0, wn0 + j * 32 + l32);
+#pragma unroll
+        for (int s = 0; s < 4; s++) {
+            const int c = s & 1, nx = c ^ 1;
+            if (s + 1 < 4) {
+#pragma unroll
+                for (int i = 0; i < FM; i++) af[nx][i] = a_frag(cur, s + 1, wm0 + i * 32 + l32);
+#pragma unroll
+                for (int j = 0; j < FN; j++) bf[nx][j] = b_frag(cur, s + 1, wn0 + j * 32 + l32);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            mfma_step(af[c], bf[c]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+
+    // Prologue: tiles 0 .. NST-2 in flight.
+    issue(0, St0);
+    issue(1, St1);
+    if constexpr (NST == 4) issue(2, St2);
+    for (int t = 0; t < nt; t += NST) {
+        if constexpr (NST == 3) {
+            iter(t, St0, St2);
+            if (t + 1 < nt) iter(t + 1, St1, St0);
+            if (t + 2 < nt) iter(t + 2, St2, St1);
+        } else {
+            iter(t, St0, St3);
+            if (t + 1 < nt) iter(t + 1, St1, St0);
+            if (t + 2 < nt) iter(t + 2, St2, St1);
+            if (t + 3 < nt) iter(t + 3, St3, St2);
+        }
+    }
+
+    if (has_ext) {
+        xa.template store<float>(ExAs);
+        xb.template store<float>(ExBs);
+        __syncthreads();
+#pragma unroll
+        for (int s = 0; s < 2; s++) {
+            float4 af[FM], bf[FN];
+#pragma unroll
+            for (int i = 0; i < FM; i++) af[i] = ExA::frag(ExAs, s, half, wm0 + i * 32 + l32);
+#pragma unroll
+            for (int j = 0; j < FN; j++) bf[j] = ExB::frag(ExBs, s, half, wn0 + j * 32 + l32);
+            mfma_step(af, bf);
+        }
+    }
+    // Nothing may still be landing in LDS when the workgroup retires.
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+
+#pragma unroll
+    for (int i = 0; i < FM; i++)
+#pragma unroll
+        for (int j = 0; j < FN; j++) {
+            const int col = n0 + wn0 + j * 32 + l32;
+            if (col >= p.N) continue;
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int row = m0 + wm0 + i * 32 + (r / 4) * 8 + half * 4 + (r % 4);
+                if (row < p.M) p.out[(long)row * p.ldc + col] = acc[i][j][r];
+            }
+        }
+}
+
+// ---------------------------------------------------------------------------
 // out[R, C] (C <= 32) = scale * X[R, Kr] @ Y[Kr, C].
 //   XT:  X is stored [Kr, R] (element (row,k) at x[k*ldx + row])
 //   YT:  Y is stored [C, Kr] (element (k,col) at y[col*ldy + k])
@@ -613,6 +841,24 @@ __global__ __launch_bounds__(256) void skinny_kernel(const float* __restrict__ x
 // Host side
 // ---------------------------------------------------------------------------
 
+template <int BM, int BN, int WM, int WN, int NST>
+int launch_async(ft_context* ctx, GemmArgs p, int layout) {
+    const int tiles_m = (p.M + BM - 1) / BM;
+    p.tiles_n = (p.N + BN - 1) / BN;
+    const dim3 grid((unsigned)(tiles_m * p.tiles_n));
+    char name[96];
+    snprintf(name, sizeof(name), "gemm_async_kernel<%d, %d, %d, %d, %d, %d>", BM, BN, WM, WN, layout, NST);
+    const double kk = (double)p.K + (p.a2 ? (double)p.K2 : 0.0);
+    ft_prof_scope prof(ctx, name, 2.0 * p.M * (double)p.N * kk,
+                       4.0 * p.M * kk + 2.0 * p.N * (double)p.K + 4.0 * p.N * (p.a2 ? p.K2 : 0) + 4.0 * p.M * (double)p.N);
+    if (layout == 0)
+        hipLaunchKernelGGL((gemm_async_kernel<BM, BN, WM, WN, 0, NST>), grid, dim3(256), 0, ctx->stream, p);
+    else
+        hipLaunchKernelGGL((gemm_async_kernel<BM, BN, WM, WN, 1, NST>), grid, dim3(256), 0, ctx->stream, p);
+    FT_LAUNCH_CHECK();
+    return FT_OK;
+}
+
 template <int BM, int BN, int WM, int WN, int BKF = 32>
 int launch_cfg(ft_context* ctx, GemmArgs p, int layout, bool half_b, bool fast) {
     const int tiles_m = (p.M + BM - 1) / BM;
@@ -691,6 +937,17 @@ int gemm_dispatch(ft_context* ctx, const char* who, int layout, bool half_b, con
     const double lim = 4294967296.0;
     fast = fast && 4.0 * (double)M * (double)(layout == 2 ? 1 : K) + 4.0 * 64 * (double)p.lda < lim &&
            4.0 * (double)N * (double)(layout == 1 ? K : 1) + 4.0 * 64 * (double)p.ldb < lim;
+    // Asynchronous global->LDS path: f16 b, K in whole tiles, rank-r term at most 16 wide.
+    const bool async_ok = fast && half_b && layout != 2 && K % 32 == 0 && K >= 32 && (!p.a2 || K2 <= 16) &&
+                          (layout == 1 || (N % 8 == 0 && N >= 8)) && p.ldb % 8 == 0 &&
+                          2.0 * (double)p.ldb * (double)(layout == 1 ? N : K) < lim;
+    if (async_ok && !getenv("FT_GEMM_NO_ASYNC")) {
+        const char* st = getenv("FT_GEMM_STAGES");
+        const int nst = st ? atoi(st) : 3;
+        if (best == 0) return launch_async<128, 128, 64, 64, 3>(ctx, p, layout);
+        if (nst == 4) return launch_async<64, 64, 32, 32, 4>(ctx, p, layout);
+        return launch_async<64, 64, 32, 32, 3>(ctx, p, layout);
+    }
     if (best == 0) return launch_cfg<128, 128, 64, 64>(ctx, p, layout, half_b, fast);
     if (best == 3) return launch_cfg<64, 64, 32, 32, 64>(ctx, p, layout, half_b, fast);
     return launch_cfg<64, 64, 32, 32>(ctx, p, layout, half_b, fast);
