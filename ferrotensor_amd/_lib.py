@@ -76,9 +76,9 @@ SIGNATURES = {
     "ft_matmul_f16b": [_P, _P, _P, _P, _SZ, _SZ, _SZ],
     "ft_matmul_bt_f16b": [_P, _P, _P, _P, _SZ, _SZ, _SZ],
     "ft_lora_down": [_P, _P, _P, _P, _SZ, _SZ, _SZ, _F],
-    "ft_lora_linear": [_P, _P, _P, _I, _P, _P, _P, _SZ, _SZ, _SZ, _SZ],
+    "ft_lora_linear": [_P, _P, _P, _I, _P, _P, _P, _P, _SZ, _SZ, _SZ, _SZ],
     "ft_lora_grad_down": [_P, _P, _P, _P, _SZ, _SZ, _SZ, _F],
-    "ft_lora_linear_dx": [_P, _P, _P, _I, _P, _P, _P, _SZ, _SZ, _SZ, _SZ],
+    "ft_lora_linear_dx": [_P, _P, _P, _I, _P, _P, _P, _P, _SZ, _SZ, _SZ, _SZ],
     "ft_lora_grad_b": [_P, _P, _P, _P, _SZ, _SZ, _SZ],
     "ft_lora_grad_a": [_P, _P, _P, _P, _SZ, _SZ, _SZ],
     "ft_rms_norm_eps": [_P, _P, _P, _P, _SZ, _SZ, _F],

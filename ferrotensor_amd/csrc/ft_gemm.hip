@@ -34,6 +34,7 @@ struct GemmArgs {
     float* out;
     const float* a2;
     const float* b2;
+    const float* add;  // optional [M,N] term added in the epilogue (may be `out` itself)
     int M, N, K, K2;
     long lda, ldb, ldc, lda2, ldb2;
     int tiles_n;
@@ -240,7 +241,10 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs p) {
 #pragma unroll
             for (int r = 0; r < 16; r++) {
                 const int row = m0 + wm0 + i * 32 + (r / 4) * 8 + half * 4 + (r % 4);
-                if (row < p.M) p.out[(long)row * p.ldc + col] = acc[i][j][r];
+                if (row < p.M) {
+                    const long o = (long)row * p.ldc + col;
+                    p.out[o] = p.add ? acc[i][j][r] + p.add[o] : acc[i][j][r];
+                }
             }
         }
 }
@@ -500,7 +504,10 @@ __global__ __launch_bounds__(256) void gemm_fast_kernel(GemmArgs p) {
 #pragma unroll
             for (int r = 0; r < 16; r++) {
                 const int row = m0 + wm0 + i * 32 + (r / 4) * 8 + half * 4 + (r % 4);
-                if (row < p.M) p.out[(long)row * p.ldc + col] = acc[i][j][r];
+                if (row < p.M) {
+                    const long o = (long)row * p.ldc + col;
+                    p.out[o] = p.add ? acc[i][j][r] + p.add[o] : acc[i][j][r];
+                }
             }
         }
 }
@@ -728,7 +735,10 @@ __global__ __launch_bounds__(256) void gemm_async_kernel(GemmArgs p) {
 #pragma unroll
             for (int r = 0; r < 16; r++) {
                 const int row = m0 + wm0 + i * 32 + (r / 4) * 8 + half * 4 + (r % 4);
-                if (row < p.M) p.out[(long)row * p.ldc + col] = acc[i][j][r];
+                if (row < p.M) {
+                    const long o = (long)row * p.ldc + col;
+                    p.out[o] = p.add ? acc[i][j][r] + p.add[o] : acc[i][j][r];
+                }
             }
         }
 }
@@ -895,7 +905,8 @@ int launch_cfg(ft_context* ctx, GemmArgs p, int layout, bool half_b, bool fast) 
 }
 
 int gemm_dispatch(ft_context* ctx, const char* who, int layout, bool half_b, const float* a, const void* b,
-                  float* out, size_t M, size_t K, size_t N, const float* a2, const float* b2, size_t K2) {
+                  float* out, size_t M, size_t K, size_t N, const float* a2, const float* b2, size_t K2,
+                  const float* add = nullptr) {
     FT_CHECK_ARG(ctx, "%s: ctx is NULL", who);
     FT_CHECK_ARG(M < (1u << 30) && N < (1u << 30) && K < (1u << 30) && K2 < (1u << 30), "%s: dimension too large", who);
     if (M == 0 || N == 0) return FT_OK;
@@ -906,6 +917,7 @@ int gemm_dispatch(ft_context* ctx, const char* who, int layout, bool half_b, con
     p.a = a;
     p.b = b;
     p.out = out;
+    p.add = add;
     p.a2 = K2 > 0 ? a2 : nullptr;
     p.b2 = K2 > 0 ? b2 : nullptr;
     p.M = (int)M;
@@ -997,9 +1009,9 @@ int ft_lora_down(ft_context* ctx, const float* x, const float* a, float* t, size
 }
 
 int ft_lora_linear(ft_context* ctx, const float* x, const void* w, int w_dtype, const float* t, const float* b,
-                   float* y, size_t M, size_t K, size_t N, size_t r) {
+                   const float* residual, float* y, size_t M, size_t K, size_t N, size_t r) {
     FT_CHECK_ARG(w_dtype == FT_DTYPE_F32 || w_dtype == FT_DTYPE_F16, "ft_lora_linear: dtype %d", w_dtype);
-    return gemm_dispatch(ctx, "ft_lora_linear", 0, w_dtype == FT_DTYPE_F16, x, w, y, M, K, N, t, b, r);
+    return gemm_dispatch(ctx, "ft_lora_linear", 0, w_dtype == FT_DTYPE_F16, x, w, y, M, K, N, t, b, r, residual);
 }
 
 int ft_lora_grad_down(ft_context* ctx, const float* dy, const float* b, float* dt, size_t M, size_t N, size_t r,
@@ -1013,10 +1025,10 @@ int ft_lora_grad_down(ft_context* ctx, const float* dy, const float* b, float* d
 }
 
 int ft_lora_linear_dx(ft_context* ctx, const float* dy, const void* w, int w_dtype, const float* dt,
-                      const float* a, float* dx, size_t M, size_t K, size_t N, size_t r) {
+                      const float* a, const float* residual, float* dx, size_t M, size_t K, size_t N, size_t r) {
     FT_CHECK_ARG(w_dtype == FT_DTYPE_F32 || w_dtype == FT_DTYPE_F16, "ft_lora_linear_dx: dtype %d", w_dtype);
     // dx[M,K] = dy[M,N] @ w[K,N]^T + dt[M,r] @ a[K,r]^T: layout 1 with output width K, reduction N.
-    return gemm_dispatch(ctx, "ft_lora_linear_dx", 1, w_dtype == FT_DTYPE_F16, dy, w, dx, M, N, K, dt, a, r);
+    return gemm_dispatch(ctx, "ft_lora_linear_dx", 1, w_dtype == FT_DTYPE_F16, dy, w, dx, M, N, K, dt, a, r, residual);
 }
 
 int ft_lora_grad_b(ft_context* ctx, const float* t, const float* dy, float* db, size_t M, size_t N, size_t r) {

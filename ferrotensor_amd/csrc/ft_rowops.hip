@@ -307,6 +307,140 @@ __global__ __launch_bounds__(256) void column_sum_kernel(const float* __restrict
 }
 
 // ---------------------------------------------------------------------------
+// RMSNorm, one wave per row: the row (up to 64*4*NV floats) lives in registers
+// between the reduction and the output, so every array is touched once and no
+// workgroup barrier is needed. 4 rows per 256-thread workgroup.
+// ---------------------------------------------------------------------------
+template <int NV>
+__global__ __launch_bounds__(256) void rms_norm_wave_kernel(const float* __restrict__ x, const float* __restrict__ w,
+                                                            float* __restrict__ out, int rows, int size, float eps) {
+    const int row = blockIdx.x * 4 + threadIdx.x / kWave;
+    if (row >= rows) return;
+    const int lane = threadIdx.x % kWave;
+    const int n4 = size / 4;
+    const float4* x4 = reinterpret_cast<const float4*>(x + (size_t)row * size);
+    float4 v[NV];
+    float ss = 0.0f;
+#pragma unroll
+    for (int j = 0; j < NV; j++) {
+        const int i = lane + j * kWave;
+        v[j] = i < n4 ? x4[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+        ss += v[j].x * v[j].x + v[j].y * v[j].y + v[j].z * v[j].z + v[j].w * v[j].w;
+    }
+    ss = wave_sum(ss);
+    const float inv = 1.0f / sqrtf(ss / (float)size + eps);
+    const float4* w4 = reinterpret_cast<const float4*>(w);
+    float4* o4 = reinterpret_cast<float4*>(out + (size_t)row * size);
+#pragma unroll
+    for (int j = 0; j < NV; j++) {
+        const int i = lane + j * kWave;
+        if (i < n4) {
+            const float4 g = w4[i];
+            o4[i] = make_float4(v[j].x * inv * g.x, v[j].y * inv * g.y, v[j].z * inv * g.z, v[j].w * inv * g.w);
+        }
+    }
+}
+
+// gx = g*w*inv - x*coef (+ add): the input gradient of RMSNorm, optionally
+// summed with the gradient arriving over the residual connection.
+template <int NV>
+__global__ __launch_bounds__(256) void rms_norm_backward_wave_kernel(
+    const float* __restrict__ x, const float* __restrict__ w, const float* __restrict__ g, const float* add,
+    float* gx, int rows, int size, float eps) {
+    const int row = blockIdx.x * 4 + threadIdx.x / kWave;
+    if (row >= rows) return;
+    const int lane = threadIdx.x % kWave;
+    const int n4 = size / 4;
+    const float4* x4 = reinterpret_cast<const float4*>(x + (size_t)row * size);
+    const float4* g4 = reinterpret_cast<const float4*>(g + (size_t)row * size);
+    const float4* w4 = reinterpret_cast<const float4*>(w);
+    float4 xv[NV], gv[NV];
+    float ss = 0.0f, gwx = 0.0f;
+#pragma unroll
+    for (int j = 0; j < NV; j++) {
+        const int i = lane + j * kWave;
+        if (i < n4) {
+            xv[j] = x4[i];
+            const float4 gg = g4[i], ww = w4[i];
+            gv[j] = make_float4(gg.x * ww.x, gg.y * ww.y, gg.z * ww.z, gg.w * ww.w);  // g*w
+        } else {
+            xv[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+            gv[j] = xv[j];
+        }
+        ss += xv[j].x * xv[j].x + xv[j].y * xv[j].y + xv[j].z * xv[j].z + xv[j].w * xv[j].w;
+        gwx += gv[j].x * xv[j].x + gv[j].y * xv[j].y + gv[j].z * xv[j].z + gv[j].w * xv[j].w;
+    }
+    ss = wave_sum(ss);
+    gwx = wave_sum(gwx);
+    const float inv = 1.0f / sqrtf(ss / (float)size + eps);
+    const float coef = gwx * inv * inv * inv / (float)size;
+    const float4* a4 = reinterpret_cast<const float4*>(add ? add + (size_t)row * size : nullptr);
+    float4* o4 = reinterpret_cast<float4*>(gx + (size_t)row * size);
+#pragma unroll
+    for (int j = 0; j < NV; j++) {
+        const int i = lane + j * kWave;
+        if (i < n4) {
+            float4 r = make_float4(gv[j].x * inv - xv[j].x * coef, gv[j].y * inv - xv[j].y * coef,
+                                   gv[j].z * inv - xv[j].z * coef, gv[j].w * inv - xv[j].w * coef);
+            if (add) {
+                const float4 a = a4[i];
+                r = make_float4(a.x + r.x, a.y + r.y, a.z + r.z, a.w + r.w);
+            }
+            o4[i] = r;
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// RoPE through a (cos, sin) table: the angles of a step depend only on
+// (position, i), so they are computed once (exactly as rope_kernel computes
+// them) and the rotation itself becomes a pure streaming pass. One launch
+// rotates two tensors (q and k).
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void rope_table_kernel(float2* __restrict__ table, unsigned seq, unsigned head_dim,
+                                                         unsigned pos0, float theta) {
+    const unsigned half = head_dim / 2;
+    const unsigned idx = blockIdx.x * 256 + threadIdx.x;
+    if (idx >= seq * half) return;
+    const unsigned t = idx / half, i = idx % half;
+    const float pos = (float)(pos0 + t);
+    const float freq_exp = -2.0f * (float)i / (float)head_dim;
+    const float angle = pos * powf(theta, freq_exp);
+    float s, c;
+    sincosf(angle, &s, &c);
+    table[idx] = make_float2(c, s);
+}
+
+struct RopeJob {
+    const float* src;
+    float* dst;
+    unsigned heads;      // head vectors per token
+    size_t quads;        // tokens * heads * head_dim / 8 (4 pairs per thread)
+};
+
+__global__ __launch_bounds__(256) void rope_apply_kernel(RopeJob j0, RopeJob j1, const float2* __restrict__ table,
+                                                         unsigned seq, unsigned head_dim, float dir) {
+    const RopeJob& j = blockIdx.y == 0 ? j0 : j1;
+    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= j.quads) return;
+    const unsigned half = head_dim / 2, qpv = half / 4;   // quads per head vector
+    const size_t vec = idx / qpv;
+    const unsigned i = (unsigned)(idx % qpv) * 4;
+    const unsigned t = (unsigned)((vec / j.heads) % seq);
+    const float2* tb = table + (size_t)t * half + i;
+    const float4 v1 = *reinterpret_cast<const float4*>(j.src + vec * head_dim + i);
+    const float4 v2 = *reinterpret_cast<const float4*>(j.src + vec * head_dim + i + half);
+    const float2 c0 = tb[0], c1 = tb[1], c2 = tb[2], c3 = tb[3];
+    float4 o1, o2;
+    o1.x = v1.x * c0.x - v2.x * (dir * c0.y);  o2.x = v1.x * (dir * c0.y) + v2.x * c0.x;
+    o1.y = v1.y * c1.x - v2.y * (dir * c1.y);  o2.y = v1.y * (dir * c1.y) + v2.y * c1.x;
+    o1.z = v1.z * c2.x - v2.z * (dir * c2.y);  o2.z = v1.z * (dir * c2.y) + v2.z * c2.x;
+    o1.w = v1.w * c3.x - v2.w * (dir * c3.y);  o2.w = v1.w * (dir * c3.y) + v2.w * c3.x;
+    *reinterpret_cast<float4*>(j.dst + vec * head_dim + i) = o1;
+    *reinterpret_cast<float4*>(j.dst + vec * head_dim + i + half) = o2;
+}
+
+// ---------------------------------------------------------------------------
 // RoPE (rotate-half). One thread per (token, head, i < head_dim/2) pair.
 // Angles in f32 exactly as pos * powf(theta, -2i/head_dim), precise sin/cos.
 // ---------------------------------------------------------------------------
@@ -583,6 +717,60 @@ __global__ __launch_bounds__(256) void multi_adamw_kernel(const ft_segment* __re
 }  // namespace
 
 // Internal entry points used by the step driver (ft_step.cpp).
+// gx = rms_norm_backward(x, w, g) (+ add); add may be NULL or alias gx. No weight gradient.
+int ft_internal_rms_norm_backward_add(ft_context* ctx, const float* x, const float* w, const float* g,
+                                      const float* add, float* gx, size_t rows, size_t size, float eps) {
+    FT_CHECK_ARG(ctx && x && w && g && gx, "rms_norm_backward: NULL argument");
+    FT_CHECK_ARG(size > 0, "rms_norm_backward: size is 0");
+    if (rows == 0) return FT_OK;
+    const bool vec = (size % 4 == 0) && aligned16(x) && aligned16(w) && aligned16(g) && aligned16(gx) &&
+                     aligned16(add) && size <= 2048 && rows < (1u << 30);
+    if (!vec) {
+        FT_TRY(ft_rms_norm_backward(ctx, x, w, g, gx, nullptr, rows, size, eps));
+        if (add) return ft_add(ctx, add, gx, gx, rows * size);
+        return FT_OK;
+    }
+    ft_prof_scope prof(ctx, "rms_norm_backward_kernel", 0.0, (add ? 16.0 : 12.0) * (double)rows * size);
+    const dim3 grid(ft_div_up(rows, 4));
+    if (size <= 1024)
+        hipLaunchKernelGGL((rms_norm_backward_wave_kernel<4>), grid, dim3(256), 0, ctx->stream, x, w, g, add, gx,
+                           (int)rows, (int)size, eps);
+    else
+        hipLaunchKernelGGL((rms_norm_backward_wave_kernel<8>), grid, dim3(256), 0, ctx->stream, x, w, g, add, gx,
+                           (int)rows, (int)size, eps);
+    FT_LAUNCH_CHECK();
+    return FT_OK;
+}
+
+// (cos, sin) of pos * theta^(-2i/head_dim) for seq positions; table holds seq * head_dim/2 float2.
+int ft_internal_rope_table(ft_context* ctx, float* table, size_t seq, size_t head_dim, size_t pos, float theta) {
+    const size_t n = seq * head_dim / 2;
+    if (n == 0) return FT_OK;
+    hipLaunchKernelGGL(rope_table_kernel, dim3(ft_div_up(n, 256)), dim3(256), 0, ctx->stream,
+                       reinterpret_cast<float2*>(table), (unsigned)seq, (unsigned)head_dim, (unsigned)pos, theta);
+    FT_LAUNCH_CHECK();
+    return FT_OK;
+}
+
+// Rotates a [batch, seq, heads_a*head_dim] and a [batch, seq, heads_b*head_dim] tensor in one
+// launch (src may equal dst). head_dim must be a multiple of 8 and the tensors 16-byte aligned.
+int ft_internal_rope_pair(ft_context* ctx, const float* a_src, float* a_dst, size_t heads_a, const float* b_src,
+                          float* b_dst, size_t heads_b, const float* table, size_t batch, size_t seq,
+                          size_t head_dim, int inverse) {
+    FT_CHECK_ARG(head_dim % 8 == 0 && aligned16(a_src) && aligned16(a_dst) && aligned16(b_src) && aligned16(b_dst),
+                 "rope pair: head_dim %zu must be a multiple of 8 and the tensors aligned", head_dim);
+    RopeJob j0{a_src, a_dst, (unsigned)heads_a, batch * seq * heads_a * head_dim / 8};
+    RopeJob j1{b_src, b_dst, (unsigned)heads_b, batch * seq * heads_b * head_dim / 8};
+    const size_t qmax = j0.quads > j1.quads ? j0.quads : j1.quads;
+    if (qmax == 0) return FT_OK;
+    ft_prof_scope prof(ctx, "rope_apply_kernel", 0.0, 8.0 * (double)(j0.quads + j1.quads) * 8);
+    hipLaunchKernelGGL(rope_apply_kernel, dim3(ft_div_up(qmax, 256), 2), dim3(256), 0, ctx->stream, j0, j1,
+                       reinterpret_cast<const float2*>(table), (unsigned)seq, (unsigned)head_dim,
+                       inverse ? -1.0f : 1.0f);
+    FT_LAUNCH_CHECK();
+    return FT_OK;
+}
+
 int ft_internal_multi_grad_norm(ft_context* ctx, const ft_segment* segs_dev, size_t nseg, float* partials_dev,
                                 float max_norm, float* control_dev) {
     if (nseg == 0) return FT_OK;
@@ -675,6 +863,17 @@ int ft_rms_norm_eps(ft_context* ctx, const float* x, const float* w, float* out,
     if (rows == 0) return FT_OK;
     const int vec = (size % 4 == 0) && aligned16(x) && aligned16(w) && aligned16(out);
     ft_prof_scope prof(ctx, "rms_norm_kernel", 0.0, 8.0 * (double)rows * size);
+    if (vec && size <= 2048 && rows < (1u << 30)) {
+        const dim3 grid(ft_div_up(rows, 4));
+        if (size <= 1024)
+            hipLaunchKernelGGL((rms_norm_wave_kernel<4>), grid, dim3(256), 0, ctx->stream, x, w, out, (int)rows,
+                               (int)size, eps);
+        else
+            hipLaunchKernelGGL((rms_norm_wave_kernel<8>), grid, dim3(256), 0, ctx->stream, x, w, out, (int)rows,
+                               (int)size, eps);
+        FT_LAUNCH_CHECK();
+        return FT_OK;
+    }
     hipLaunchKernelGGL(rms_norm_kernel, dim3((unsigned)rows), dim3(256), 0, ctx->stream, x, w, out, rows, size,
                        eps, vec);
     FT_LAUNCH_CHECK();
@@ -685,6 +884,9 @@ int ft_rms_norm_backward(ft_context* ctx, const float* x, const float* w, const 
                          size_t rows, size_t size, float eps) {
     FT_CHECK_ARG(ctx && x && w && g && gx, "ft_rms_norm_backward: NULL argument");
     FT_CHECK_ARG(size > 0, "ft_rms_norm_backward: size is 0");
+    if (!gw && rows > 0 && size % 4 == 0 && size <= 2048 && aligned16(x) && aligned16(w) && aligned16(g) &&
+        aligned16(gx))
+        return ft_internal_rms_norm_backward_add(ctx, x, w, g, nullptr, gx, rows, size, eps);
     if (rows == 0) {
         if (gw) return ft_zero(ctx, gw, size * 4);
         return FT_OK;

@@ -36,6 +36,12 @@ struct ft_segment {
 };
 int ft_internal_multi_grad_norm(ft_context* ctx, const ft_segment* segs_dev, size_t nseg, float* partials_dev,
                                 float max_norm, float* control_dev);
+int ft_internal_rms_norm_backward_add(ft_context* ctx, const float* x, const float* w, const float* g,
+                                      const float* add, float* gx, size_t rows, size_t size, float eps);
+int ft_internal_rope_table(ft_context* ctx, float* table, size_t seq, size_t head_dim, size_t pos, float theta);
+int ft_internal_rope_pair(ft_context* ctx, const float* a_src, float* a_dst, size_t heads_a, const float* b_src,
+                          float* b_dst, size_t heads_b, const float* table, size_t batch, size_t seq,
+                          size_t head_dim, int inverse);
 int ft_internal_multi_adamw(ft_context* ctx, const ft_segment* segs_dev, size_t nseg, const ft_adam_params* p,
                             float grad_scale, const float* control_dev);
 
@@ -102,9 +108,9 @@ struct ft_model {
     uint32_t *ids_dev = nullptr, *targets_dev = nullptr;
     float *weights_dev = nullptr, *row_loss = nullptr;
     // backward scratch
-    float *g0 = nullptr, *g1 = nullptr, *gx = nullptr, *d_act = nullptr, *d_gate = nullptr, *d_up = nullptr,
-          *d_h2 = nullptr, *d_h2b = nullptr, *d_attn = nullptr, *dq = nullptr, *dk = nullptr, *dv = nullptr,
-          *d_h1 = nullptr, *d_h1b = nullptr, *dt = nullptr, *dt2 = nullptr, *dt3 = nullptr, *gtmp = nullptr;
+    float *g0 = nullptr, *g1 = nullptr, *d_act = nullptr, *d_gate = nullptr, *d_up = nullptr, *d_h2 = nullptr,
+          *d_attn = nullptr, *dq = nullptr, *dk = nullptr, *dv = nullptr, *d_h1 = nullptr, *dt = nullptr,
+          *dt2 = nullptr, *dt3 = nullptr, *gtmp = nullptr, *rope_table = nullptr;
 
     size_t head_dim() const { return cfg.hidden_size / cfg.num_attention_heads; }
 };
@@ -181,18 +187,21 @@ int ensure_workspace(ft_model* m, size_t B, size_t S) {
     FT_TRY(ws_alloc(m, T, &m->row_loss));
     FT_TRY(ws_alloc(m, T * H, &m->g0));
     FT_TRY(ws_alloc(m, T * H, &m->g1));
-    FT_TRY(ws_alloc(m, T * H, &m->gx));
     FT_TRY(ws_alloc(m, T * F, &m->d_act));
     FT_TRY(ws_alloc(m, T * F, &m->d_gate));
     FT_TRY(ws_alloc(m, T * F, &m->d_up));
     FT_TRY(ws_alloc(m, T * H, &m->d_h2));
-    FT_TRY(ws_alloc(m, T * H, &m->d_h2b));
     FT_TRY(ws_alloc(m, T * QD, &m->d_attn));
     FT_TRY(ws_alloc(m, T * QD, &m->dq));
     FT_TRY(ws_alloc(m, T * KD, &m->dk));
     FT_TRY(ws_alloc(m, T * KD, &m->dv));
     FT_TRY(ws_alloc(m, T * H, &m->d_h1));
-    FT_TRY(ws_alloc(m, T * H, &m->d_h1b));
+    // (cos, sin) table of the rotary embedding; the vector kernel needs head_dim % 8 == 0
+    m->rope_table = nullptr;
+    if (m->head_dim() % 8 == 0) {
+        FT_TRY(ws_alloc(m, S * m->head_dim(), &m->rope_table));
+        FT_TRY(ft_internal_rope_table(m->ctx, m->rope_table, S, m->head_dim(), 0, c.rope_theta));
+    }
     FT_TRY(ws_alloc(m, T * (rmax ? rmax : 1), &m->dt));
     FT_TRY(ws_alloc(m, T * (rmax ? rmax : 1), &m->dt2));
     FT_TRY(ws_alloc(m, T * (rmax ? rmax : 1), &m->dt3));
@@ -239,24 +248,26 @@ int lora_down_group(ft_context* ctx, LinearW* const* ls, float* const* ts, int n
 }
 
 // y = x @ W (+ t @ B) with t = scale * x @ A already computed.
-int linear_gemm(ft_context* ctx, const LinearW& l, const float* x, const float* t, float* y, size_t T) {
+int linear_gemm(ft_context* ctx, const LinearW& l, const float* x, const float* t, float* y, size_t T,
+                const float* residual = nullptr) {
     FT_CHECK_ARG(l.w, "linear %s has no weight", l.prefix.c_str());
-    if (l.has_lora()) return ft_lora_linear(ctx, x, l.w, l.dtype, t, l.b, y, T, l.in, l.out, l.r);
-    return ft_lora_linear(ctx, x, l.w, l.dtype, nullptr, nullptr, y, T, l.in, l.out, 0);
+    if (l.has_lora()) return ft_lora_linear(ctx, x, l.w, l.dtype, t, l.b, residual, y, T, l.in, l.out, l.r);
+    return ft_lora_linear(ctx, x, l.w, l.dtype, nullptr, nullptr, residual, y, T, l.in, l.out, 0);
 }
 
-// y = x @ W (+ (scale * x @ A) @ B), keeping t = scale * x @ A for backward.
-int linear_forward(ft_context* ctx, LinearW& l, const float* x, float* t, float* y, size_t T) {
+// y = x @ W (+ (scale * x @ A) @ B) (+ residual), keeping t = scale * x @ A for backward.
+int linear_forward(ft_context* ctx, LinearW& l, const float* x, float* t, float* y, size_t T,
+                   const float* residual = nullptr) {
     LinearW* ls[1] = {&l};
     float* ts[1] = {t};
     FT_TRY(lora_down_group(ctx, ls, ts, 1, x, T));
-    return linear_gemm(ctx, l, x, t, y, T);
+    return linear_gemm(ctx, l, x, t, y, T, residual);
 }
 
 // Gradients of one linear given dy: LoRA factor gradients (written, or added
-// when `accumulate`), and dx when wanted.
+// when `accumulate`), and dx when wanted (added to what dx holds when `dx_add`).
 int linear_backward(ft_model* m, LinearW& l, const float* x, const float* t, const float* dy, float* dx, size_t T,
-                    bool accumulate) {
+                    bool accumulate, bool dx_add = false) {
     ft_context* ctx = m->ctx;
     if (l.has_lora()) {
         FT_TRY(ft_lora_grad_down(ctx, dy, l.b, m->dt, T, l.out, l.r, l.scale()));
@@ -277,19 +288,23 @@ int linear_backward(ft_model* m, LinearW& l, const float* x, const float* t, con
                 FT_TRY(ft_lora_grad_a(ctx, x, m->dt, l.ga, T, l.in, l.r));
             }
         }
-        if (dx) FT_TRY(ft_lora_linear_dx(ctx, dy, l.w, l.dtype, m->dt, l.a, dx, T, l.in, l.out, l.r));
+        if (dx)
+            FT_TRY(ft_lora_linear_dx(ctx, dy, l.w, l.dtype, m->dt, l.a, dx_add ? dx : nullptr, dx, T, l.in, l.out,
+                                     l.r));
     } else if (dx) {
-        FT_TRY(ft_lora_linear_dx(ctx, dy, l.w, l.dtype, nullptr, nullptr, dx, T, l.in, l.out, 0));
+        FT_TRY(ft_lora_linear_dx(ctx, dy, l.w, l.dtype, nullptr, nullptr, dx_add ? dx : nullptr, dx, T, l.in, l.out,
+                                 0));
     }
     return FT_OK;
 }
 
 // The same for up to 3 linears that share their input x (q/k/v, gate/up): the
-// dT, dA and dB products of all of them go into two batched launches. dxs[i]
-// may be NULL. Falls back to one linear at a time when the adapters cannot be
-// batched or gradients are being accumulated.
+// dT, dA and dB products of all of them go into two batched launches. The input
+// gradients are summed into dx (NULL: not wanted): the first GEMM writes it, the
+// others add to it in their epilogue. Falls back to one linear at a time when the
+// adapters cannot be batched or gradients are being accumulated.
 int linear_backward_group(ft_model* m, LinearW* const* ls, const float* const* ts, const float* const* dys,
-                          float* const* dxs, int n, const float* x, size_t T, bool accumulate) {
+                          float* dx, int n, const float* x, size_t T, bool accumulate) {
     ft_context* ctx = m->ctx;
     float* dts[3] = {m->dt, m->dt2, m->dt3};
     bool batch = !accumulate && n <= 3;
@@ -309,15 +324,14 @@ int linear_backward_group(ft_model* m, LinearW* const* ls, const float* const* t
         batch = ft_thin_rowwise_ok(rows[i]) && ft_thin_colwise_ok(cols[2 * i]) && ft_thin_colwise_ok(cols[2 * i + 1]);
     }
     if (!batch) {
-        for (int i = 0; i < n; i++) FT_TRY(linear_backward(m, *ls[i], x, ts[i], dys[i], dxs[i], T, accumulate));
+        for (int i = 0; i < n; i++) FT_TRY(linear_backward(m, *ls[i], x, ts[i], dys[i], dx, T, accumulate, i > 0));
         return FT_OK;
     }
     FT_TRY(ft_thin_rowwise(ctx, rows, n));
     FT_TRY(ft_thin_colwise(ctx, cols, 2 * n));
-    for (int i = 0; i < n; i++)
-        if (dxs[i])
-            FT_TRY(ft_lora_linear_dx(ctx, dys[i], ls[i]->w, ls[i]->dtype, dts[i], ls[i]->a, dxs[i], T, ls[i]->in,
-                                     ls[i]->out, ls[i]->r));
+    for (int i = 0; i < n && dx; i++)
+        FT_TRY(ft_lora_linear_dx(ctx, dys[i], ls[i]->w, ls[i]->dtype, dts[i], ls[i]->a, i > 0 ? dx : nullptr, dx, T,
+                                 ls[i]->in, ls[i]->out, ls[i]->r));
     return FT_OK;
 }
 
@@ -353,12 +367,15 @@ int model_forward(ft_model* m, const uint32_t* rows_host, size_t B, size_t S) {
         FT_TRY(linear_gemm(ctx, L.q, a.h1, a.tq, a.q, T));
         FT_TRY(linear_gemm(ctx, L.k, a.h1, a.tk, a.k, T));
         FT_TRY(linear_gemm(ctx, L.v, a.h1, a.tv, a.v, T));
-        FT_TRY(ft_rope_theta(ctx, a.q, B, S, nh * D, D, 0, c.rope_theta));
-        FT_TRY(ft_rope_theta(ctx, a.k, B, S, nkv * D, D, 0, c.rope_theta));
+        if (m->rope_table) {
+            FT_TRY(ft_internal_rope_pair(ctx, a.q, a.q, nh, a.k, a.k, nkv, m->rope_table, B, S, D, 0));
+        } else {
+            FT_TRY(ft_rope_theta(ctx, a.q, B, S, nh * D, D, 0, c.rope_theta));
+            FT_TRY(ft_rope_theta(ctx, a.k, B, S, nkv * D, D, 0, c.rope_theta));
+        }
         FT_TRY(ft_flash_attention_v2_with_stats(ctx, a.q, a.k, a.v, a.attn, a.stats, B, S, S, nh, nkv, D, &opts));
-        // o_proj output lands in gx (scratch), then h = x + o
-        FT_TRY(linear_forward(ctx, L.o, a.attn, a.to, m->gx, T));
-        FT_TRY(ft_add(ctx, a.x, m->gx, a.h, T * H));
+        // h = x + o_proj(attn): the residual is added in the GEMM epilogue
+        FT_TRY(linear_forward(ctx, L.o, a.attn, a.to, a.h, T, a.x));
         FT_TRY(ft_rms_norm_eps(ctx, a.h, L.norm2, a.h2, T, H, c.rms_norm_eps));
         {
             LinearW* ls[2] = {&L.up, &L.gate};
@@ -368,8 +385,7 @@ int model_forward(ft_model* m, const uint32_t* rows_host, size_t B, size_t S) {
         FT_TRY(linear_gemm(ctx, L.up, a.h2, a.tup, a.up, T));
         FT_TRY(linear_gemm(ctx, L.gate, a.h2, a.tgate, a.gate, T));
         FT_TRY(ft_silu_gate_fused(ctx, a.gate, a.up, a.act, T * F));
-        FT_TRY(linear_forward(ctx, L.down, a.act, a.tdown, m->gx, T));
-        FT_TRY(ft_add(ctx, a.h, m->gx, x_next, T * H));
+        FT_TRY(linear_forward(ctx, L.down, a.act, a.tdown, x_next, T, a.h));
     }
     FT_TRY(ft_rms_norm_eps(ctx, m->x_final, m->norm_f, m->hf, T, H, c.rms_norm_eps));
     FT_TRY(linear_forward(ctx, m->lm_head, m->hf, m->thead, m->logits, T));
@@ -399,19 +415,20 @@ int model_backward(ft_model* m, size_t B, size_t S, bool accumulate) {
             LinearW* ls[2] = {&L.up, &L.gate};
             const float* ts[2] = {a.tup, a.tgate};
             const float* dys[2] = {m->d_up, m->d_gate};
-            float* dxs[2] = {m->d_h2, m->d_h2b};
-            FT_TRY(linear_backward_group(m, ls, ts, dys, dxs, 2, a.h2, T, accumulate));
+            FT_TRY(linear_backward_group(m, ls, ts, dys, m->d_h2, 2, a.h2, T, accumulate));
         }
-        FT_TRY(ft_gradient_accumulate(ctx, m->d_h2, m->d_h2b, T * H));
-        FT_TRY(ft_rms_norm_backward(ctx, a.h, L.norm2, m->d_h2, m->gx, nullptr, T, H, c.rms_norm_eps));
-        // g_h = g + gx (into g_other)
-        FT_TRY(ft_add(ctx, g, m->gx, g_other, T * H));
+        // g_h = g + norm2_backward(d_h2) (into g_other)
+        FT_TRY(ft_internal_rms_norm_backward_add(ctx, a.h, L.norm2, m->d_h2, g, g_other, T, H, c.rms_norm_eps));
         // h = x + o_proj(attn)
         FT_TRY(linear_backward(m, L.o, a.attn, a.to, g_other, m->d_attn, T, accumulate));
         FT_TRY(ft_flash_attention_v2_backward_with_stats(ctx, a.q, a.k, a.v, a.attn, m->d_attn, m->dq, m->dk, m->dv,
                                                          a.stats, B, S, S, nh, nkv, D, &opts));
-        FT_TRY(ft_rope_theta_inverse(ctx, m->dq, B, S, nh * D, D, 0, c.rope_theta));
-        FT_TRY(ft_rope_theta_inverse(ctx, m->dk, B, S, nkv * D, D, 0, c.rope_theta));
+        if (m->rope_table) {
+            FT_TRY(ft_internal_rope_pair(ctx, m->dq, m->dq, nh, m->dk, m->dk, nkv, m->rope_table, B, S, D, 1));
+        } else {
+            FT_TRY(ft_rope_theta_inverse(ctx, m->dq, B, S, nh * D, D, 0, c.rope_theta));
+            FT_TRY(ft_rope_theta_inverse(ctx, m->dk, B, S, nkv * D, D, 0, c.rope_theta));
+        }
         // The first block's input is the frozen embedding: its norm output needs
         // no gradient, so the three input-gradient GEMMs are skipped
         // (MatMulNode::backward, autograd/src/lib.rs:268-287).
@@ -420,15 +437,12 @@ int model_backward(ft_model* m, size_t B, size_t S, bool accumulate) {
             LinearW* ls[3] = {&L.q, &L.k, &L.v};
             const float* ts[3] = {a.tq, a.tk, a.tv};
             const float* dys[3] = {m->dq, m->dk, m->dv};
-            // d_h1 = dx_q + dx_k + dx_v: the three land in d_h1, d_h1b and gx.
-            float* dxs[3] = {need_dx ? m->d_h1 : nullptr, need_dx ? m->d_h1b : nullptr, need_dx ? m->gx : nullptr};
-            FT_TRY(linear_backward_group(m, ls, ts, dys, dxs, 3, a.h1, T, accumulate));
+            // d_h1 = dx_q + dx_k + dx_v
+            FT_TRY(linear_backward_group(m, ls, ts, dys, need_dx ? m->d_h1 : nullptr, 3, a.h1, T, accumulate));
         }
         if (!need_dx) break;
-        FT_TRY(ft_gradient_accumulate(ctx, m->d_h1, m->d_h1b, T * H));
-        FT_TRY(ft_gradient_accumulate(ctx, m->d_h1, m->gx, T * H));
-        FT_TRY(ft_rms_norm_backward(ctx, a.x, L.norm1, m->d_h1, m->gx, nullptr, T, H, c.rms_norm_eps));
-        FT_TRY(ft_add(ctx, g_other, m->gx, g, T * H));
+        // g = g_h + norm1_backward(d_h1)
+        FT_TRY(ft_internal_rms_norm_backward_add(ctx, a.x, L.norm1, m->d_h1, g_other, g, T, H, c.rms_norm_eps));
     }
     return FT_OK;
 }

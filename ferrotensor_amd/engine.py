@@ -288,12 +288,12 @@ class ComputeEngine:
         assert K == K2 and t.numel() == M * r
         check(self._lib.ft_lora_down(ctx.handle, _p(x), _p(a), _p(t), M, K, r, scale))
 
-    def lora_linear(self, ctx, x, w, t, b, y):
+    def lora_linear(self, ctx, x, w, t, b, y, residual=None):
         M, K = x.shape
         K2, N = w.shape
         r = b.shape[0] if b is not None else 0
         assert K == K2 and y.numel() == M * N
-        check(self._lib.ft_lora_linear(ctx.handle, _p(x), _p(w), w.dtype, _p(t), _p(b), _p(y), M, K, N, r))
+        check(self._lib.ft_lora_linear(ctx.handle, _p(x), _p(w), w.dtype, _p(t), _p(b), _p(residual), _p(y), M, K, N, r))
 
     def lora_grad_down(self, ctx, dy, b, dt, scale):
         M, N = dy.shape
@@ -301,12 +301,12 @@ class ComputeEngine:
         assert N == N2 and dt.numel() == M * r
         check(self._lib.ft_lora_grad_down(ctx.handle, _p(dy), _p(b), _p(dt), M, N, r, scale))
 
-    def lora_linear_dx(self, ctx, dy, w, dt, a, dx):
+    def lora_linear_dx(self, ctx, dy, w, dt, a, dx, residual=None):
         M, N = dy.shape
         K, N2 = w.shape
         r = a.shape[1] if a is not None else 0
         assert N == N2 and dx.numel() == M * K
-        check(self._lib.ft_lora_linear_dx(ctx.handle, _p(dy), _p(w), w.dtype, _p(dt), _p(a), _p(dx), M, K, N, r))
+        check(self._lib.ft_lora_linear_dx(ctx.handle, _p(dy), _p(w), w.dtype, _p(dt), _p(a), _p(residual), _p(dx), M, K, N, r))
 
     def lora_grad_b(self, ctx, t, dy, db):
         M, r = t.shape

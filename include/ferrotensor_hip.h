@@ -136,17 +136,23 @@ int ft_matmul_bt_f16b(ft_context* ctx, const float* a, const uint16_t* b, float*
  * r <= 32. */
 int ft_lora_down(ft_context* ctx, const float* x, const float* a, float* t, size_t M, size_t K,
                  size_t r, float scale);
-/* y[M,N] = x[M,K] @ w[K,N] + t[M,r] @ b[r,N]; w is f32 (w_dtype FT_DTYPE_F32)
- * or packed f16. The rank-r product rides in the GEMM's K loop. */
+/* y[M,N] = x[M,K] @ w[K,N] + t[M,r] @ b[r,N] (+ residual[M,N]); w is f32
+ * (w_dtype FT_DTYPE_F32) or packed f16. The rank-r product rides in the GEMM's
+ * K loop; `residual` (NULL = none, may be y itself) is added in the epilogue,
+ * which also absorbs the block's residual add (lfm.rs:116-139). */
 int ft_lora_linear(ft_context* ctx, const float* x, const void* w, int w_dtype, const float* t,
-                   const float* b, float* y, size_t M, size_t K, size_t N, size_t r);
+                   const float* b, const float* residual, float* y, size_t M, size_t K, size_t N,
+                   size_t r);
 /* dt[M,r] = scale * (dy[M,N] @ b[r,N]^T): gradient of the scaled `x @ A`. */
 int ft_lora_grad_down(ft_context* ctx, const float* dy, const float* b, float* dt, size_t M,
                       size_t N, size_t r, float scale);
-/* dx[M,K] = dy[M,N] @ w[K,N]^T + dt[M,r] @ a[K,r]^T (both MatMulNode input
- * gradients and their AddNode sum in one GEMM). */
+/* dx[M,K] = dy[M,N] @ w[K,N]^T + dt[M,r] @ a[K,r]^T (+ residual[M,K]): both
+ * MatMulNode input gradients and their AddNode sum in one GEMM; `residual`
+ * (NULL = none, may be dx itself) carries a gradient that is being
+ * accumulated (accumulate_grad, ferrotensor-autograd/src/lib.rs:206-218). */
 int ft_lora_linear_dx(ft_context* ctx, const float* dy, const void* w, int w_dtype, const float* dt,
-                      const float* a, float* dx, size_t M, size_t K, size_t N, size_t r);
+                      const float* a, const float* residual, float* dx, size_t M, size_t K, size_t N,
+                      size_t r);
 /* db[r,N] = t[M,r]^T @ dy[M,N]  (matmul_at of the scaled x@A and dy). */
 int ft_lora_grad_b(ft_context* ctx, const float* t, const float* dy, float* db, size_t M, size_t N,
                    size_t r);

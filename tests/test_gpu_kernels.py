@@ -133,6 +133,15 @@ def test_fused_lora_linear_forward_and_backward(g, M, K, N, r, f16):
     dx = empty(ctx, M, K)
     eng.lora_linear_dx(ctx, dyt, wt, dt, At, dx)
     assert_close("lora_linear_dx", dx.to_numpy(), want_dx, atol=2e-3, rtol=1e-4)
+    # residual added in the epilogue: a separate tensor, and the output itself (accumulate)
+    res = rnd(6, M, N)
+    y2 = empty(ctx, M, N)
+    eng.lora_linear(ctx, xt, wt, t, Bt, y2, residual=up(ctx, res))
+    assert_close("lora_linear+residual", y2.to_numpy(), want_y + res, atol=1e-3, rtol=1e-4)
+    acc = rnd(7, M, K)
+    dx2 = up(ctx, acc)
+    eng.lora_linear_dx(ctx, dyt, wt, dt, At, dx2, residual=dx2)
+    assert_close("lora_linear_dx accumulate", dx2.to_numpy(), want_dx + acc, atol=2e-3, rtol=1e-4)
     db, da = empty(ctx, r, N), empty(ctx, K, r)
     eng.lora_grad_b(ctx, t, dyt, db)
     eng.lora_grad_a(ctx, xt, dt, da)
@@ -155,7 +164,7 @@ def test_rms_norm_forward_backward(g, rows, size):
     assert_close("rms gw", gw.to_numpy(), want_gw, atol=2e-4)
     gx2 = empty(ctx, rows, size)
     eng.rms_norm_backward(ctx, up(ctx, x), up(ctx, w), up(ctx, gy), gx2, None, eps)
-    np.testing.assert_array_equal(gx2.to_numpy(), gx.to_numpy())
+    assert_close("rms gx (no gw)", gx2.to_numpy(), want_gx)
 
 
 @pytest.mark.parametrize("B,S,heads,D,pos,theta", [(1, 1, 1, 2, 0, 10000.0), (2, 9, 3, 8, 5, 10000.0),
