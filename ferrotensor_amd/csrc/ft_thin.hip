@@ -3,7 +3,8 @@
 // coalesced loads, and several independent products go into one launch.
 //
 //   row-wise   out[M, C] = scale * X[M, K] @ Y        (x@A,  dT = dY@B^T)
-//              two rows per wave, lanes stride over K, butterfly reduction.
+//              16 rows per workgroup, K split over its 4 waves, 16x16x4 MFMA
+//              (the matrix unit does the K reduction, no cross-lane shuffles).
 //   col-wise   out[R, C] = X[M, R]^T @ Y[M, C]        (dA = x^T@dT, dB = T^T@dY)
 //              each thread owns 4 columns of X, the M rows are cut into
 //              slices; a second kernel adds the slices in order (deterministic,
@@ -21,81 +22,86 @@ struct ThinBatch {
 };
 
 // ---- row-wise ---------------------------------------------------------------
-// grid (ceil(M / 8), count); 256 threads = 4 waves x 2 rows.
+// grid (ceil(M / 16), count); 256 threads = 4 waves. A workgroup owns 16 rows;
+// each wave takes a quarter of K through v_mfma_f32_16x16x4_f32 (X rows are the
+// A operand, Y columns the B operand, columns >= C fed with zeros), and the four
+// partial 16x16 tiles are added in wave order through LDS. Every lane reads X in
+// 16-byte pieces: lane (row = l % 16, q = l / 16) takes k = 16*it + 4*q .. +3,
+// so MFMA e of an iteration contracts k = 16*it + 4*q + e.
+typedef float thin_f4 __attribute__((ext_vector_type(4)));
+
 template <int C, bool YT>
 __global__ __launch_bounds__(256) void thin_rowwise_kernel(ThinBatch b) {
     const ft_thin_problem& p = b.p[blockIdx.y];
+    const int row0 = blockIdx.x * 16;
+    if (row0 >= p.M) return;
+    __shared__ float red[4][16][17];
     const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
-    const int row0 = (blockIdx.x * 4 + wave) * 2;
-    if (row0 >= p.M) return;  // wave-uniform
-    const bool two = row0 + 1 < p.M;
-    const float* x0 = p.x + (long)row0 * p.ldx;
-    const float* x1 = p.x + (long)(two ? row0 + 1 : row0) * p.ldx;
-    float acc0[C], acc1[C];
+    const int li = lane % 16, q = lane / 16;
+    const int row = row0 + li < p.M ? row0 + li : p.M - 1;  // clamped rows are computed and dropped
+    const float* xr = p.x + (long)row * p.ldx + 4 * q;
+    const bool col_live = li < C;
+    // K is a multiple of 4; the quarters are multiples of 16, so a 4-run of k is all in or all out.
+    const int part = ((p.K + 63) / 64) * 16;
+    const int k_begin = wave * part;
+    const int k_end = k_begin + part < p.K ? k_begin + part : p.K;
+    thin_f4 acc = {0.f, 0.f, 0.f, 0.f};
+    constexpr int U = 4;  // iterations whose loads are issued together
+    for (int k0 = k_begin; k0 < k_end; k0 += 16 * U) {
+        float4 xa[U];
+        float yb[U][4];
 #pragma unroll
-    for (int j = 0; j < C; j++) acc0[j] = acc1[j] = 0.0f;
-
-    const int K4 = p.K / 4;  // K is a multiple of 4 (checked on the host)
-    for (int q = lane; q < K4; q += kWave) {
-        const int k = q * 4;
-        const float4 a0 = *reinterpret_cast<const float4*>(x0 + k);
-        const float4 a1 = *reinterpret_cast<const float4*>(x1 + k);
-        if constexpr (!YT) {
-            // Y[k..k+3][0..C-1] is one contiguous run of 4*C floats.
-            const float4* y4 = reinterpret_cast<const float4*>(p.y + (long)k * C);
-            float yv[4 * C];
+        for (int u = 0; u < U; u++) {
+            const int k = k0 + 16 * u + 4 * q;
+            const bool in = k < k_end;
+            xa[u] = in ? *reinterpret_cast<const float4*>(xr + k0 + 16 * u) : make_float4(0.f, 0.f, 0.f, 0.f);
+            if constexpr (YT) {
+                const float4 t = (in && col_live) ? *reinterpret_cast<const float4*>(p.y + (long)li * p.ldy + k)
+                                                  : make_float4(0.f, 0.f, 0.f, 0.f);
+                yb[u][0] = t.x, yb[u][1] = t.y, yb[u][2] = t.z, yb[u][3] = t.w;
+            } else {
 #pragma unroll
-            for (int e = 0; e < C; e++) {
-                const float4 t = y4[e];
-                yv[4 * e + 0] = t.x;
-                yv[4 * e + 1] = t.y;
-                yv[4 * e + 2] = t.z;
-                yv[4 * e + 3] = t.w;
+                for (int e = 0; e < 4; e++) yb[u][e] = (in && col_live) ? p.y[(long)(k + e) * C + li] : 0.0f;
             }
+        }
 #pragma unroll
-            for (int j = 0; j < C; j++) {
-                acc0[j] += a0.x * yv[j] + a0.y * yv[C + j] + a0.z * yv[2 * C + j] + a0.w * yv[3 * C + j];
-                acc1[j] += a1.x * yv[j] + a1.y * yv[C + j] + a1.z * yv[2 * C + j] + a1.w * yv[3 * C + j];
-            }
-        } else {
-            // Y is stored [C, K]: row j holds the k run.
-#pragma unroll
-            for (int j = 0; j < C; j++) {
-                const float4 t = *reinterpret_cast<const float4*>(p.y + (long)j * p.ldy + k);
-                acc0[j] += a0.x * t.x + a0.y * t.y + a0.z * t.z + a0.w * t.w;
-                acc1[j] += a1.x * t.x + a1.y * t.y + a1.z * t.z + a1.w * t.w;
-            }
+        for (int u = 0; u < U; u++) {
+            acc = __builtin_amdgcn_mfma_f32_16x16x4f32(xa[u].x, yb[u][0], acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_16x16x4f32(xa[u].y, yb[u][1], acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_16x16x4f32(xa[u].z, yb[u][2], acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_16x16x4f32(xa[u].w, yb[u][3], acc, 0, 0, 0);
         }
     }
+    // accumulator register r holds row 4*q + r, column li
 #pragma unroll
-    for (int j = 0; j < C; j++) {
-#pragma unroll
-        for (int o = kWave / 2; o > 0; o >>= 1) {
-            acc0[j] += __shfl_xor(acc0[j], o, kWave);
-            acc1[j] += __shfl_xor(acc1[j], o, kWave);
-        }
-    }
-    if (lane == 0) {
-#pragma unroll
-        for (int j = 0; j < C; j++) {
-            p.out[(long)row0 * p.ldo + j] = acc0[j] * p.scale;
-            if (two) p.out[(long)(row0 + 1) * p.ldo + j] = acc1[j] * p.scale;
-        }
+    for (int r = 0; r < 4; r++) red[wave][4 * q + r][li] = acc[r];
+    __syncthreads();
+    const int orow = threadIdx.x / 16, ocol = threadIdx.x % 16;
+    if (ocol < C && row0 + orow < p.M) {
+        const float v = ((red[0][orow][ocol] + red[1][orow][ocol]) + red[2][orow][ocol]) + red[3][orow][ocol];
+        p.out[(long)(row0 + orow) * p.ldo + ocol] = v * p.scale;
     }
 }
 
 // ---- col-wise ---------------------------------------------------------------
-// grid (ceil(Rmax / 256), count, slices); 64 threads, each owning 4 columns.
-// partial[((slice * R) + n) * C + j] at p.scratch_offset.
+// grid (ceil(Rmax / 256), count, slices); 256 threads = 4 waves. Every thread owns
+// 4 columns of X (a wave 256 of them); the rows of a slice are dealt to the four
+// waves in contiguous quarters and the four partial results are added in wave
+// order through LDS. partial[((slice * R) + n) * C + j] at p.scratch_offset.
 template <int C>
-__global__ __launch_bounds__(64) void thin_colwise_kernel(ThinBatch b, float* __restrict__ scratch, int slices) {
+__global__ __launch_bounds__(256) void thin_colwise_kernel(ThinBatch b, float* __restrict__ scratch, int slices) {
     const ft_thin_problem& p = b.p[blockIdx.y];
-    const int n = (blockIdx.x * 64 + threadIdx.x) * 4;
     if (blockIdx.x * 256 >= p.R) return;  // whole workgroup past this problem's width
-    const bool live = n < p.R;            // R is a multiple of 4 (checked on the host)
+    __shared__ float red[3][4 * C][kWave + 1];
+    const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+    const int n = (blockIdx.x * 64 + lane) * 4;
+    const bool live = n < p.R;  // R is a multiple of 4 (checked on the host)
     const int per = (p.M + slices - 1) / slices;
-    const int m_begin = blockIdx.z * per;
-    const int m_end = m_begin + per < p.M ? m_begin + per : p.M;
+    const int s_begin = blockIdx.z * per;
+    const int s_end = s_begin + per < p.M ? s_begin + per : p.M;
+    const int quarter = (per + 3) / 4;
+    const int m_begin = s_begin + wave * quarter;
+    const int m_end = m_begin + quarter < s_end ? m_begin + quarter : s_end;
     float acc[4][C];
 #pragma unroll
     for (int e = 0; e < 4; e++)
@@ -103,7 +109,7 @@ __global__ __launch_bounds__(64) void thin_colwise_kernel(ThinBatch b, float* __
         for (int j = 0; j < C; j++) acc[e][j] = 0.0f;
     if (live) {
         const float* xp = p.x + n;
-#pragma unroll 4
+#pragma unroll 8
         for (int m = m_begin; m < m_end; m++) {
             const float4 xv = *reinterpret_cast<const float4*>(xp + (long)m * p.ldx);
             const float* yr = p.y + (long)m * p.ldy;  // uniform across the wave
@@ -116,6 +122,20 @@ __global__ __launch_bounds__(64) void thin_colwise_kernel(ThinBatch b, float* __
                 acc[3][j] += xv.w * yv;
             }
         }
+    }
+    if (wave > 0) {
+#pragma unroll
+        for (int e = 0; e < 4; e++)
+#pragma unroll
+            for (int j = 0; j < C; j++) red[wave - 1][e * C + j][lane] = acc[e][j];
+    }
+    __syncthreads();
+    if (wave == 0 && live) {
+#pragma unroll
+        for (int e = 0; e < 4; e++)
+#pragma unroll
+            for (int j = 0; j < C; j++)
+                acc[e][j] = ((acc[e][j] + red[0][e * C + j][lane]) + red[1][e * C + j][lane]) + red[2][e * C + j][lane];
         float* dst = scratch + p.scratch_offset + ((long)blockIdx.z * p.R + n) * C;
 #pragma unroll
         for (int e = 0; e < 4; e++)
@@ -134,7 +154,15 @@ __global__ __launch_bounds__(256) void thin_finish_kernel(ThinBatch b, const flo
     if (e >= total) return;
     const float* src = scratch + p.scratch_offset + e;
     float v = 0.0f;
-    for (int s = 0; s < slices; s++) v += src[(long)s * total];
+    int s = 0;
+    for (; s + 8 <= slices; s += 8) {
+        float t[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) t[u] = src[(long)(s + u) * total];
+#pragma unroll
+        for (int u = 0; u < 8; u++) v += t[u];
+    }
+    for (; s < slices; s++) v += src[(long)s * total];
     const int n = e / p.C, j = e % p.C;
     if (p.out_transposed)
         p.out[(long)j * p.ldo + n] = v * p.scale;
@@ -182,7 +210,7 @@ int ft_thin_rowwise(ft_context* ctx, const ft_thin_problem* probs, int count) {
         bytes += 4.0 * ((double)p.M * p.K + (double)p.K * p.C + (double)p.M * p.C);
     }
     if (mmax == 0) return FT_OK;
-    const dim3 grid(ft_div_up(mmax, 8), (unsigned)count);
+    const dim3 grid(ft_div_up(mmax, 16), (unsigned)count);
     ft_prof_scope prof(ctx, probs[0].y_transposed ? "thin_rowwise_kernel<YT>" : "thin_rowwise_kernel", 0.0, bytes);
 #define FT_ROW(CC)                                                                                              \
     do {                                                                                                        \
@@ -215,8 +243,8 @@ int ft_thin_colwise(ft_context* ctx, const ft_thin_problem* probs, int count) {
     if (rmax == 0) return FT_OK;
     // Rows per slice: enough slices to fill the chip, few enough that the
     // partial sums stay a fraction of the input traffic.
-    int slices = mmax / 64;
-    if (slices > 32) slices = 32;
+    int slices = mmax / 128;
+    if (slices > 16) slices = 16;
     if (slices < 1) slices = 1;
     size_t off = 0;
     for (int i = 0; i < count; i++) {
@@ -231,11 +259,11 @@ int ft_thin_colwise(ft_context* ctx, const ft_thin_problem* probs, int count) {
     const dim3 fgrid(ft_div_up((size_t)rmax * probs[0].C, 256), (unsigned)count);
     ft_prof_scope prof(ctx, "thin_colwise+finish", 0.0, bytes);
     if (probs[0].C == 4)
-        hipLaunchKernelGGL((thin_colwise_kernel<4>), grid, dim3(64), 0, ctx->stream, b, ctx->thin_scratch, slices);
+        hipLaunchKernelGGL((thin_colwise_kernel<4>), grid, dim3(256), 0, ctx->stream, b, ctx->thin_scratch, slices);
     else if (probs[0].C == 8)
-        hipLaunchKernelGGL((thin_colwise_kernel<8>), grid, dim3(64), 0, ctx->stream, b, ctx->thin_scratch, slices);
+        hipLaunchKernelGGL((thin_colwise_kernel<8>), grid, dim3(256), 0, ctx->stream, b, ctx->thin_scratch, slices);
     else
-        hipLaunchKernelGGL((thin_colwise_kernel<16>), grid, dim3(64), 0, ctx->stream, b, ctx->thin_scratch, slices);
+        hipLaunchKernelGGL((thin_colwise_kernel<16>), grid, dim3(256), 0, ctx->stream, b, ctx->thin_scratch, slices);
     FT_LAUNCH_CHECK();
     hipLaunchKernelGGL(thin_finish_kernel, fgrid, dim3(256), 0, ctx->stream, b, ctx->thin_scratch, slices);
     FT_LAUNCH_CHECK();
