@@ -20,6 +20,16 @@ class AttentionOptionsC(C.Structure):
                 ("dropout_prob", C.c_float), ("seed", C.c_uint64)]
 
 
+class LoraLinearDescC(C.Structure):
+    _fields_ = [("w", C.c_void_p), ("w_dtype", C.c_int32), ("t", C.c_void_p), ("b", C.c_void_p),
+                ("residual", C.c_void_p), ("y", C.c_void_p), ("N", C.c_size_t), ("r", C.c_size_t)]
+
+
+class LoraDxDescC(C.Structure):
+    _fields_ = [("dy", C.c_void_p), ("w", C.c_void_p), ("w_dtype", C.c_int32), ("dt", C.c_void_p),
+                ("a", C.c_void_p), ("N", C.c_size_t), ("r", C.c_size_t)]
+
+
 class AdamParamsC(C.Structure):
     _fields_ = [("lr", C.c_float), ("beta1", C.c_float), ("beta2", C.c_float), ("eps", C.c_float),
                 ("weight_decay", C.c_float), ("t", C.c_float)]
@@ -76,6 +86,8 @@ SIGNATURES = {
     "ft_matmul_f16b": [_P, _P, _P, _P, _SZ, _SZ, _SZ],
     "ft_matmul_bt_f16b": [_P, _P, _P, _P, _SZ, _SZ, _SZ],
     "ft_lora_down": [_P, _P, _P, _P, _SZ, _SZ, _SZ, _F],
+    "ft_lora_linear_group": [_P, _P, C.POINTER(LoraLinearDescC), _SZ, _SZ, _SZ],
+    "ft_lora_linear_dx_group": [_P, C.POINTER(LoraDxDescC), _SZ, _P, _P, _SZ, _SZ],
     "ft_lora_linear": [_P, _P, _P, _I, _P, _P, _P, _P, _SZ, _SZ, _SZ, _SZ],
     "ft_lora_grad_down": [_P, _P, _P, _P, _SZ, _SZ, _SZ, _F],
     "ft_lora_linear_dx": [_P, _P, _P, _I, _P, _P, _P, _P, _SZ, _SZ, _SZ, _SZ],

@@ -546,10 +546,47 @@ __device__ __forceinline__ void glds16(const char* base, unsigned voff, const fl
     asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(base), "s"(l) : "memory", "m0");
 }
 
-template <int BM, int BN, int WM, int WN, int LAYOUT, int NST>
-__global__ __launch_bounds__(256) void gemm_async_kernel(GemmArgs p) {
+// One launch covers up to kAsyncMaxProb products that share M (and usually the a
+// operand): q/k/v or gate/up of one input, each with its own b, output, rank-r
+// term and residual. A product may itself be a sum over up to kAsyncMaxSeg K
+// segments with their own a and b (dx = dq Wq^T + dk Wk^T + dv Wv^T): the tile
+// pipeline runs through the segments without draining.
+constexpr int kAsyncMaxSeg = 3, kAsyncMaxProb = 3;
+
+struct AsyncSeg {
+    const float* a;   // [M, 32 * nt] f32
+    const void* b;    // packed f16: layout 0 [K, N], layout 1 [N, K]
+    const float* a2;  // rank-r term of this segment ([M, K2] and [K2, N] / [N, K2]), or NULL
+    const float* b2;
+    int lda, ldb, lda2, ldb2;
+    int nt;           // K tiles of this segment
+    int K2;
+};
+
+struct AsyncProb {
+    AsyncSeg seg[kAsyncMaxSeg];
+    float* out;
+    const float* add;  // optional [M, N] term added in the epilogue (may be `out` itself)
+    int N, ldc, tiles_n, tile_begin, nseg;
+};
+
+struct AsyncBatch {
+    AsyncProb p[kAsyncMaxProb];
+    int count, M;
+};
+
+template <int NSEG, typename T>
+__device__ __forceinline__ T seg_pick(const T (&v)[NSEG], int s) {
+    if constexpr (NSEG == 1) return v[0];
+    else if constexpr (NSEG == 2) return s == 0 ? v[0] : v[1];
+    else return s == 0 ? v[0] : (s == 1 ? v[1] : v[2]);
+}
+
+template <int BM, int BN, int WM, int WN, int LAYOUT, int NSEG>
+__global__ __launch_bounds__(256) void gemm_async_kernel(AsyncBatch g) {
     static_assert(LAYOUT == 0 || LAYOUT == 1, "a is k-contiguous on this path");
-    static_assert(NST == 3 || NST == 4, "3 or 4 stages");
+    static_assert(NSEG == 1 || NSEG == kAsyncMaxSeg, "one segment, or the general case");
+    constexpr int NST = 3;
     constexpr int FM = WM / 32, FN = WN / 32;
     constexpr int WAVES_N = BN / WN;
     static_assert((BM / WM) * (BN / WN) == 4, "4 waves per workgroup");
@@ -566,11 +603,15 @@ __global__ __launch_bounds__(256) void gemm_async_kernel(GemmArgs p) {
     __shared__ __attribute__((aligned(16))) float St0[STAGE];
     __shared__ __attribute__((aligned(16))) float St1[STAGE];
     __shared__ __attribute__((aligned(16))) float St2[STAGE];
-    __shared__ __attribute__((aligned(16))) float St3[NST == 4 ? STAGE : 4];
     __shared__ __attribute__((aligned(16))) float ExAs[ExA::LDS_FLOATS];
     __shared__ __attribute__((aligned(16))) float ExBs[ExB::LDS_FLOATS];
 
-    const int tile = blockIdx.x;
+    int pi = 0;
+    if (g.count > 1 && (int)blockIdx.x >= g.p[1].tile_begin) pi = 1;
+    if (g.count > 2 && (int)blockIdx.x >= g.p[2].tile_begin) pi = 2;
+    const AsyncProb& p = g.p[pi];
+    const int M = g.M;
+    const int tile = (int)blockIdx.x - p.tile_begin;
     const int m0 = (tile / p.tiles_n) * BM;
     const int n0 = (tile % p.tiles_n) * BN;
     const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
@@ -585,29 +626,50 @@ __global__ __launch_bounds__(256) void gemm_async_kernel(GemmArgs p) {
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
 
-    const int nt = p.K / 32;
-    const bool has_ext = p.a2 != nullptr;
+    // Uniform description of the segments (a missing one repeats the last: never reached).
+    const char* abase[NSEG];
+    const char* bbase[NSEG];
+    int lda_b[NSEG], ldb_b[NSEG], tend[NSEG];
+    bool has_ext[NSEG];
+#pragma unroll
+    for (int s = 0; s < NSEG; s++) {
+        const AsyncSeg& sg = p.seg[s < p.nseg ? s : 0];
+        abase[s] = reinterpret_cast<const char*>(sg.a);
+        bbase[s] = reinterpret_cast<const char*>(sg.b);
+        lda_b[s] = sg.lda * 4;
+        ldb_b[s] = sg.ldb * 2;
+        tend[s] = (s > 0 ? tend[s - 1] : 0) + (s < p.nseg ? sg.nt : 0);
+        has_ext[s] = s < p.nseg && sg.a2 != nullptr;
+    }
+    const int nt = tend[NSEG - 1];
 
-    // The rank-r product's operands: ordinary loads, issued first, consumed last.
-    ExA xa;
-    ExB xb;
-    if (has_ext) {
-        xa.set_offsets(p.lda2, m0, p.M, 4);
-        xb.set_offsets(p.ldb2, n0, p.N, 4);
-        xa.template load<float, true>(reinterpret_cast<const char*>(p.a2), 0, p.K2);
-        xb.template load<float, true>(reinterpret_cast<const char*>(p.b2), 0, p.K2);
+    // The rank-r products' operands: ordinary loads, issued first, consumed last.
+    ExA xa[NSEG];
+    ExB xb[NSEG];
+#pragma unroll
+    for (int s = 0; s < NSEG; s++) {
+        if (has_ext[s]) {
+            const AsyncSeg& sg = p.seg[s];
+            xa[s].set_offsets(sg.lda2, m0, M, 4);
+            xb[s].set_offsets(sg.ldb2, n0, p.N, 4);
+            xa[s].template load<float, true>(reinterpret_cast<const char*>(sg.a2), 0, sg.K2);
+            xb[s].template load<float, true>(reinterpret_cast<const char*>(sg.b2), 0, sg.K2);
+        }
     }
 
-    // Per-lane source offsets (bytes), constant over the K loop.
-    unsigned offA[A_CH], offB[B_CH];
+    // Per-lane source coordinates, constant over the K loop: byte offset =
+    // row * (leading dimension in bytes) + col. With one segment the product is
+    // formed once, here.
+    unsigned rowA[A_CH], colA[A_CH], rowB[B_CH], colB[B_CH];
 #pragma unroll
     for (int j = 0; j < A_CH; j++) {
         const int c = wave + 4 * j, r = lane / 8, cs = lane % 8;
         int row = m0 + 8 * c + r;
-        row = row < p.M ? row : p.M - 1;
-        offA[j] = (unsigned)(((long)row * p.lda + ((cs ^ r) * 4)) * 4);
+        row = row < M ? row : M - 1;
+        rowA[j] = (unsigned)row;
+        colA[j] = (unsigned)((cs ^ r) * 16);
+        if constexpr (NSEG == 1) colA[j] += rowA[j] * (unsigned)lda_b[0];
     }
-    long b_step;
 #pragma unroll
     for (int j = 0; j < B_CH; j++) {
         const int c = wave + 4 * j;
@@ -615,27 +677,39 @@ __global__ __launch_bounds__(256) void gemm_async_kernel(GemmArgs p) {
             const int r = lane / 4, cs = lane % 4;
             int n = n0 + 16 * c + r;
             n = n < p.N ? n : p.N - 1;
-            offB[j] = (unsigned)(((long)n * p.ldb + ((cs ^ ((r >> 1) & 3)) * 8)) * 2);
+            rowB[j] = (unsigned)n;
+            colB[j] = (unsigned)((cs ^ ((r >> 1) & 3)) * 16);
         } else {
             constexpr int LPR = BN / 8, RPC = 64 / LPR;
             const int kr = lane / LPR, cs = lane % LPR;
             int col = n0 + cs * 8;
             col = col + 8 <= p.N ? col : p.N - 8;
-            offB[j] = (unsigned)(((long)(c * RPC + kr) * p.ldb + col) * 2);
+            rowB[j] = (unsigned)(c * RPC + kr);
+            colB[j] = (unsigned)(col * 2);
         }
+        if constexpr (NSEG == 1) colB[j] += rowB[j] * (unsigned)ldb_b[0];
     }
-    b_step = LAYOUT == 1 ? 64 : 64 * p.ldb;  // bytes per K tile
-    const char* abase = reinterpret_cast<const char*>(p.a);
-    const char* bbase = reinterpret_cast<const char*>(p.b);
 
     auto issue = [&](int t, float* st) {
         t = t < nt ? t : nt - 1;  // past the end: re-read the last tile into a stage nobody reads
-        const char* at = abase + (long)t * 128;
-        const char* bt = bbase + (long)t * b_step;
+        int s = 0, tl = t;
+        if constexpr (NSEG > 1) {
+            if (t >= tend[0]) s = 1, tl = t - tend[0];
+            if (t >= tend[1]) s = 2, tl = t - tend[1];
+        }
+        const int la = seg_pick<NSEG>(lda_b, s), lb = seg_pick<NSEG>(ldb_b, s);
+        const char* at = seg_pick<NSEG>(abase, s) + (long)tl * 128;
+        const char* bt = seg_pick<NSEG>(bbase, s) + (long)tl * (LAYOUT == 1 ? 64L : 32L * lb);
 #pragma unroll
-        for (int j = 0; j < A_CH; j++) glds16(at, offA[j], st + (wave + 4 * j) * 256);
+        for (int j = 0; j < A_CH; j++) {
+            const unsigned off = NSEG == 1 ? colA[j] : rowA[j] * (unsigned)la + colA[j];
+            glds16(at, off, st + (wave + 4 * j) * 256);
+        }
 #pragma unroll
-        for (int j = 0; j < B_CH; j++) glds16(bt, offB[j], st + A_FLOATS + (wave + 4 * j) * 256);
+        for (int j = 0; j < B_CH; j++) {
+            const unsigned off = NSEG == 1 ? colB[j] : rowB[j] * (unsigned)lb + colB[j];
+            glds16(bt, off, st + A_FLOATS + (wave + 4 * j) * 256);
+        }
     };
     auto a_frag = [&](const float* st, int s, int row) -> float4 {
         const int kq = 2 * s + half;
@@ -695,32 +769,30 @@ __global__ __launch_bounds__(256) void gemm_async_kernel(GemmArgs p) {
     // Prologue: tiles 0 .. NST-2 in flight.
     issue(0, St0);
     issue(1, St1);
-    if constexpr (NST == 4) issue(2, St2);
     for (int t = 0; t < nt; t += NST) {
-        if constexpr (NST == 3) {
-            iter(t, St0, St2);
-            if (t + 1 < nt) iter(t + 1, St1, St0);
-            if (t + 2 < nt) iter(t + 2, St2, St1);
-        } else {
-            iter(t, St0, St3);
-            if (t + 1 < nt) iter(t + 1, St1, St0);
-            if (t + 2 < nt) iter(t + 2, St2, St1);
-            if (t + 3 < nt) iter(t + 3, St3, St2);
-        }
+        iter(t, St0, St2);
+        if (t + 1 < nt) iter(t + 1, St1, St0);
+        if (t + 2 < nt) iter(t + 2, St2, St1);
     }
 
-    if (has_ext) {
-        xa.template store<float>(ExAs);
-        xb.template store<float>(ExBs);
-        __syncthreads();
+    bool ext_used = false;
 #pragma unroll
-        for (int s = 0; s < 2; s++) {
-            float4 af[FM], bf[FN];
+    for (int s = 0; s < NSEG; s++) {
+        if (has_ext[s]) {
+            if (ext_used) __syncthreads();  // the previous segment's tile is still being read
+            ext_used = true;
+            xa[s].template store<float>(ExAs);
+            xb[s].template store<float>(ExBs);
+            __syncthreads();
 #pragma unroll
-            for (int i = 0; i < FM; i++) af[i] = ExA::frag(ExAs, s, half, wm0 + i * 32 + l32);
+            for (int st = 0; st < 2; st++) {
+                float4 af[FM], bf[FN];
 #pragma unroll
-            for (int j = 0; j < FN; j++) bf[j] = ExB::frag(ExBs, s, half, wn0 + j * 32 + l32);
-            mfma_step(af, bf);
+                for (int i = 0; i < FM; i++) af[i] = ExA::frag(ExAs, st, half, wm0 + i * 32 + l32);
+#pragma unroll
+                for (int j = 0; j < FN; j++) bf[j] = ExB::frag(ExBs, st, half, wn0 + j * 32 + l32);
+                mfma_step(af, bf);
+            }
         }
     }
     // Nothing may still be landing in LDS when the workgroup retires.
@@ -735,7 +807,7 @@ __global__ __launch_bounds__(256) void gemm_async_kernel(GemmArgs p) {
 #pragma unroll
             for (int r = 0; r < 16; r++) {
                 const int row = m0 + wm0 + i * 32 + (r / 4) * 8 + half * 4 + (r % 4);
-                if (row < p.M) {
+                if (row < M) {
                     const long o = (long)row * p.ldc + col;
                     p.out[o] = p.add ? acc[i][j][r] + p.add[o] : acc[i][j][r];
                 }
@@ -851,22 +923,88 @@ __global__ __launch_bounds__(256) void skinny_kernel(const float* __restrict__ x
 // Host side
 // ---------------------------------------------------------------------------
 
-template <int BM, int BN, int WM, int WN, int NST>
-int launch_async(ft_context* ctx, GemmArgs p, int layout) {
-    const int tiles_m = (p.M + BM - 1) / BM;
-    p.tiles_n = (p.N + BN - 1) / BN;
-    const dim3 grid((unsigned)(tiles_m * p.tiles_n));
+template <int BM, int BN, int WM, int WN>
+int launch_async(ft_context* ctx, AsyncBatch g, int layout) {
+    const int tiles_m = (g.M + BM - 1) / BM;
+    int tiles = 0, max_seg = 1;
+    double flops = 0.0, bytes = 0.0;
+    for (int i = 0; i < g.count; i++) {
+        AsyncProb& p = g.p[i];
+        p.tiles_n = (p.N + BN - 1) / BN;
+        p.tile_begin = tiles;
+        tiles += tiles_m * p.tiles_n;
+        if (p.nseg > max_seg) max_seg = p.nseg;
+        for (int s = 0; s < p.nseg; s++) {
+            const double k = 32.0 * p.seg[s].nt, k2 = p.seg[s].a2 ? (double)p.seg[s].K2 : 0.0;
+            flops += 2.0 * g.M * (double)p.N * (k + k2);
+            bytes += 4.0 * g.M * (k + k2) + 2.0 * p.N * k + 4.0 * p.N * k2;
+        }
+        bytes += (p.add ? 8.0 : 4.0) * g.M * (double)p.N;
+    }
+    const dim3 grid((unsigned)tiles);
     char name[96];
-    snprintf(name, sizeof(name), "gemm_async_kernel<%d, %d, %d, %d, %d, %d>", BM, BN, WM, WN, layout, NST);
-    const double kk = (double)p.K + (p.a2 ? (double)p.K2 : 0.0);
-    ft_prof_scope prof(ctx, name, 2.0 * p.M * (double)p.N * kk,
-                       4.0 * p.M * kk + 2.0 * p.N * (double)p.K + 4.0 * p.N * (p.a2 ? p.K2 : 0) + 4.0 * p.M * (double)p.N);
-    if (layout == 0)
-        hipLaunchKernelGGL((gemm_async_kernel<BM, BN, WM, WN, 0, NST>), grid, dim3(256), 0, ctx->stream, p);
-    else
-        hipLaunchKernelGGL((gemm_async_kernel<BM, BN, WM, WN, 1, NST>), grid, dim3(256), 0, ctx->stream, p);
+    snprintf(name, sizeof(name), "gemm_async_kernel<%d, %d, %d, %d, %d, %d>", BM, BN, WM, WN, layout,
+             max_seg > 1 ? kAsyncMaxSeg : 1);
+    ft_prof_scope prof(ctx, name, flops, bytes);
+    if (max_seg == 1) {
+        if (layout == 0)
+            hipLaunchKernelGGL((gemm_async_kernel<BM, BN, WM, WN, 0, 1>), grid, dim3(256), 0, ctx->stream, g);
+        else
+            hipLaunchKernelGGL((gemm_async_kernel<BM, BN, WM, WN, 1, 1>), grid, dim3(256), 0, ctx->stream, g);
+    } else {
+        if (layout == 0)
+            hipLaunchKernelGGL((gemm_async_kernel<BM, BN, WM, WN, 0, kAsyncMaxSeg>), grid, dim3(256), 0,
+                               ctx->stream, g);
+        else
+            hipLaunchKernelGGL((gemm_async_kernel<BM, BN, WM, WN, 1, kAsyncMaxSeg>), grid, dim3(256), 0,
+                               ctx->stream, g);
+    }
     FT_LAUNCH_CHECK();
     return FT_OK;
+}
+
+// 128x128 tiles (64x64 per wave) reach the highest MFMA occupancy but only pay
+// off when there are many of them per CU (the vocabulary head); everything
+// smaller runs best as 64x64 tiles, which keep several workgroups resident per CU.
+int launch_async_auto(ft_context* ctx, const AsyncBatch& g, int layout) {
+    size_t tiles128 = 0;
+    for (int i = 0; i < g.count; i++) tiles128 += (size_t)((g.M + 127) / 128) * (size_t)((g.p[i].N + 127) / 128);
+    if (tiles128 >= 8 * (size_t)ctx->num_cus) return launch_async<128, 128, 64, 64>(ctx, g, layout);
+    return launch_async<64, 64, 32, 32>(ctx, g, layout);
+}
+
+bool aligned16p(const void* q) { return (((uintptr_t)q) & 15) == 0; }
+
+// Can out[M,N] (+)= a[M,K] @ b (f16, `layout`) + a2[M,K2] @ b2 run on the asynchronous path?
+bool async_eligible(int layout, const float* a, const void* b, const float* out, const float* add, size_t M, size_t K,
+                    size_t N, const float* a2, const float* b2, size_t K2) {
+    if (layout != 0 && layout != 1) return false;
+    if (M == 0 || N == 0 || K < 32 || K % 32 != 0) return false;
+    if (!aligned16p(a) || !aligned16p(b) || !aligned16p(out) || !out || !a || !b) return false;
+    (void)add;
+    if (layout == 0 && (N % 8 != 0 || N < 8)) return false;
+    if (K2 > 0 && (K2 > 16 || K2 % 4 != 0 || !aligned16p(a2) || !aligned16p(b2))) return false;
+    // Per-lane operand offsets are 32-bit byte offsets from a uniform base.
+    const double lim = 4294967296.0;
+    const double ldb = layout == 1 ? (double)K : (double)N;
+    return 4.0 * (double)M * (double)K + 4.0 * 64 * (double)K < lim &&
+           2.0 * ldb * (double)(layout == 1 ? N : K) + 2.0 * 64 * ldb < lim;
+}
+
+AsyncSeg make_seg(int layout, const float* a, const void* b, size_t K, size_t N, const float* a2, const float* b2,
+                  size_t K2) {
+    AsyncSeg sg{};
+    sg.a = a;
+    sg.b = b;
+    sg.a2 = K2 > 0 ? a2 : nullptr;
+    sg.b2 = K2 > 0 ? b2 : nullptr;
+    sg.lda = (int)K;
+    sg.ldb = layout == 1 ? (int)K : (int)N;
+    sg.lda2 = (int)K2;
+    sg.ldb2 = layout == 1 ? (int)K2 : (int)N;
+    sg.nt = (int)(K / 32);
+    sg.K2 = (int)K2;
+    return sg;
 }
 
 template <int BM, int BN, int WM, int WN, int BKF = 32>
@@ -929,11 +1067,21 @@ int gemm_dispatch(ft_context* ctx, const char* who, int layout, bool half_b, con
     p.ldc = (long)N;
     p.lda2 = (long)K2;
     p.ldb2 = layout == 1 ? (long)K2 : (long)N;
-    // Tile choice, from measurements on MI355X at M = 2048: 128x128 tiles (64x64
-    // per wave) reach the highest MFMA occupancy but only pay off when there are
-    // many of them per CU (the vocabulary head); everything smaller runs best as
-    // 64x64 tiles, which keep several workgroups resident per CU. A deep K loop
-    // on few tiles prefers BK = 64 (half the barriers per MFMA).
+    if (half_b && K > 0 && async_eligible(layout, a, b, out, add, M, K, N, p.a2, p.b2, p.a2 ? K2 : 0)) {
+        AsyncBatch g{};
+        g.count = 1;
+        g.M = (int)M;
+        g.p[0].seg[0] = make_seg(layout, a, b, K, N, p.a2, p.b2, p.a2 ? K2 : 0);
+        g.p[0].nseg = 1;
+        g.p[0].out = out;
+        g.p[0].add = add;
+        g.p[0].N = (int)N;
+        g.p[0].ldc = (int)N;
+        return launch_async_auto(ctx, g, layout);
+    }
+    // Tile choice for the register-staged kernels, from measurements on MI355X at
+    // M = 2048: 128x128 tiles when there are many per CU, else 64x64; a deep K
+    // loop on few tiles prefers BK = 64 (half the barriers per MFMA).
     const size_t tiles128 = ((M + 127) / 128) * ((N + 127) / 128);
     const size_t tiles64 = ((M + 63) / 64) * ((N + 63) / 64);
     int best = tiles128 >= 8 * (size_t)ctx->num_cus ? 0 : 2;
@@ -949,17 +1097,6 @@ int gemm_dispatch(ft_context* ctx, const char* who, int layout, bool half_b, con
     const double lim = 4294967296.0;
     fast = fast && 4.0 * (double)M * (double)(layout == 2 ? 1 : K) + 4.0 * 64 * (double)p.lda < lim &&
            4.0 * (double)N * (double)(layout == 1 ? K : 1) + 4.0 * 64 * (double)p.ldb < lim;
-    // Asynchronous global->LDS path: f16 b, K in whole tiles, rank-r term at most 16 wide.
-    const bool async_ok = fast && half_b && layout != 2 && K % 32 == 0 && K >= 32 && (!p.a2 || K2 <= 16) &&
-                          (layout == 1 || (N % 8 == 0 && N >= 8)) && p.ldb % 8 == 0 &&
-                          2.0 * (double)p.ldb * (double)(layout == 1 ? N : K) < lim;
-    if (async_ok && !getenv("FT_GEMM_NO_ASYNC")) {
-        const char* st = getenv("FT_GEMM_STAGES");
-        const int nst = st ? atoi(st) : 3;
-        if (best == 0) return launch_async<128, 128, 64, 64, 3>(ctx, p, layout);
-        if (nst == 4) return launch_async<64, 64, 32, 32, 4>(ctx, p, layout);
-        return launch_async<64, 64, 32, 32, 3>(ctx, p, layout);
-    }
     if (best == 0) return launch_cfg<128, 128, 64, 64>(ctx, p, layout, half_b, fast);
     if (best == 3) return launch_cfg<64, 64, 32, 32, 64>(ctx, p, layout, half_b, fast);
     return launch_cfg<64, 64, 32, 32>(ctx, p, layout, half_b, fast);
@@ -1029,6 +1166,80 @@ int ft_lora_linear_dx(ft_context* ctx, const float* dy, const void* w, int w_dty
     FT_CHECK_ARG(w_dtype == FT_DTYPE_F32 || w_dtype == FT_DTYPE_F16, "ft_lora_linear_dx: dtype %d", w_dtype);
     // dx[M,K] = dy[M,N] @ w[K,N]^T + dt[M,r] @ a[K,r]^T: layout 1 with output width K, reduction N.
     return gemm_dispatch(ctx, "ft_lora_linear_dx", 1, w_dtype == FT_DTYPE_F16, dy, w, dx, M, N, K, dt, a, r, residual);
+}
+
+int ft_lora_linear_group(ft_context* ctx, const float* x, const ft_lora_linear_desc* linears, size_t count,
+                         size_t M, size_t K) {
+    FT_CHECK_ARG(ctx && linears && count >= 1 && count <= (size_t)kAsyncMaxProb,
+                 "ft_lora_linear_group: 1..%d linears per call", kAsyncMaxProb);
+    bool batch = M < (1u << 30) && K < (1u << 30) && M > 0;
+    for (size_t i = 0; i < count; i++) {
+        const ft_lora_linear_desc& d = linears[i];
+        FT_CHECK_ARG(d.w_dtype == FT_DTYPE_F32 || d.w_dtype == FT_DTYPE_F16, "ft_lora_linear_group: dtype %d",
+                     d.w_dtype);
+        FT_CHECK_ARG(d.r == 0 || (d.t && d.b), "ft_lora_linear_group: linear %zu has a rank but no factors", i);
+        batch = batch && d.w_dtype == FT_DTYPE_F16 && d.N < (1u << 30) &&
+                async_eligible(0, x, d.w, d.y, d.residual, M, K, d.N, d.t, d.b, d.r);
+    }
+    if (batch && count > 1) {
+        AsyncBatch g{};
+        g.count = (int)count;
+        g.M = (int)M;
+        for (size_t i = 0; i < count; i++) {
+            const ft_lora_linear_desc& d = linears[i];
+            g.p[i].seg[0] = make_seg(0, x, d.w, K, d.N, d.t, d.b, d.r);
+            g.p[i].nseg = 1;
+            g.p[i].out = d.y;
+            g.p[i].add = d.residual;
+            g.p[i].N = (int)d.N;
+            g.p[i].ldc = (int)d.N;
+        }
+        return launch_async_auto(ctx, g, 0);
+    }
+    for (size_t i = 0; i < count; i++) {
+        const ft_lora_linear_desc& d = linears[i];
+        FT_TRY(ft_lora_linear(ctx, x, d.w, d.w_dtype, d.r ? d.t : nullptr, d.r ? d.b : nullptr, d.residual, d.y, M, K,
+                              d.N, d.r));
+    }
+    return FT_OK;
+}
+
+int ft_lora_linear_dx_group(ft_context* ctx, const ft_lora_dx_desc* linears, size_t count, const float* residual,
+                            float* dx, size_t M, size_t K) {
+    FT_CHECK_ARG(ctx && linears && dx && count >= 1 && count <= (size_t)kAsyncMaxSeg,
+                 "ft_lora_linear_dx_group: 1..%d linears per call", kAsyncMaxSeg);
+    bool batch = M < (1u << 30) && K < (1u << 30) && M > 0 && K > 0;
+    size_t tiles = 0;
+    for (size_t i = 0; i < count; i++) {
+        const ft_lora_dx_desc& d = linears[i];
+        FT_CHECK_ARG(d.w_dtype == FT_DTYPE_F32 || d.w_dtype == FT_DTYPE_F16, "ft_lora_linear_dx_group: dtype %d",
+                     d.w_dtype);
+        FT_CHECK_ARG(d.r == 0 || (d.dt && d.a), "ft_lora_linear_dx_group: linear %zu has a rank but no factors", i);
+        batch = batch && d.w_dtype == FT_DTYPE_F16 && d.N < (1u << 30) &&
+                async_eligible(1, d.dy, d.w, dx, residual, M, d.N, K, d.dt, d.a, d.r);
+        tiles += d.N / 32;
+    }
+    if (batch && count > 1 && tiles < (1u << 30)) {
+        AsyncBatch g{};
+        g.count = 1;
+        g.M = (int)M;
+        for (size_t i = 0; i < count; i++) {
+            const ft_lora_dx_desc& d = linears[i];
+            g.p[0].seg[i] = make_seg(1, d.dy, d.w, d.N, K, d.dt, d.a, d.r);
+        }
+        g.p[0].nseg = (int)count;
+        g.p[0].out = dx;
+        g.p[0].add = residual;
+        g.p[0].N = (int)K;
+        g.p[0].ldc = (int)K;
+        return launch_async_auto(ctx, g, 1);
+    }
+    for (size_t i = 0; i < count; i++) {
+        const ft_lora_dx_desc& d = linears[i];
+        FT_TRY(ft_lora_linear_dx(ctx, d.dy, d.w, d.w_dtype, d.r ? d.dt : nullptr, d.r ? d.a : nullptr,
+                                 i == 0 ? residual : dx, dx, M, K, d.N, d.r));
+    }
+    return FT_OK;
 }
 
 int ft_lora_grad_b(ft_context* ctx, const float* t, const float* dy, float* db, size_t M, size_t N, size_t r) {

@@ -255,6 +255,20 @@ int linear_gemm(ft_context* ctx, const LinearW& l, const float* x, const float* 
     return ft_lora_linear(ctx, x, l.w, l.dtype, nullptr, nullptr, residual, y, T, l.in, l.out, 0);
 }
 
+// y_i = x @ W_i (+ t_i @ B_i) for linears that share x, in one launch when they can be batched.
+int linear_gemm_group(ft_context* ctx, LinearW* const* ls, const float* const* ts, float* const* ys, int n,
+                      const float* x, size_t T) {
+    ft_lora_linear_desc d[3];
+    for (int i = 0; i < n; i++) {
+        const LinearW& l = *ls[i];
+        FT_CHECK_ARG(l.w, "linear %s has no weight", l.prefix.c_str());
+        FT_CHECK_ARG(l.in == ls[0]->in, "grouped linears must share their input width");
+        d[i] = ft_lora_linear_desc{l.w, l.dtype, l.has_lora() ? ts[i] : nullptr, l.has_lora() ? l.b : nullptr,
+                                   nullptr, ys[i], l.out, l.has_lora() ? l.r : 0};
+    }
+    return ft_lora_linear_group(ctx, x, d, (size_t)n, T, ls[0]->in);
+}
+
 // y = x @ W (+ (scale * x @ A) @ B) (+ residual), keeping t = scale * x @ A for backward.
 int linear_forward(ft_context* ctx, LinearW& l, const float* x, float* t, float* y, size_t T,
                    const float* residual = nullptr) {
@@ -300,8 +314,8 @@ int linear_backward(ft_model* m, LinearW& l, const float* x, const float* t, con
 
 // The same for up to 3 linears that share their input x (q/k/v, gate/up): the
 // dT, dA and dB products of all of them go into two batched launches. The input
-// gradients are summed into dx (NULL: not wanted): the first GEMM writes it, the
-// others add to it in their epilogue. Falls back to one linear at a time when the
+// gradients are summed into dx (NULL: not wanted) by one GEMM whose K loop runs
+// over all the output gradients. Falls back to one linear at a time when the
 // adapters cannot be batched or gradients are being accumulated.
 int linear_backward_group(ft_model* m, LinearW* const* ls, const float* const* ts, const float* const* dys,
                           float* dx, int n, const float* x, size_t T, bool accumulate) {
@@ -324,14 +338,27 @@ int linear_backward_group(ft_model* m, LinearW* const* ls, const float* const* t
         batch = ft_thin_rowwise_ok(rows[i]) && ft_thin_colwise_ok(cols[2 * i]) && ft_thin_colwise_ok(cols[2 * i + 1]);
     }
     if (!batch) {
-        for (int i = 0; i < n; i++) FT_TRY(linear_backward(m, *ls[i], x, ts[i], dys[i], dx, T, accumulate, i > 0));
-        return FT_OK;
+        bool any_lora = false;
+        for (int i = 0; i < n; i++) any_lora = any_lora || ls[i]->has_lora();
+        if (any_lora || n > 3) {
+            for (int i = 0; i < n; i++)
+                FT_TRY(linear_backward(m, *ls[i], x, ts[i], dys[i], dx, T, accumulate, i > 0));
+            return FT_OK;
+        }
+        // frozen linears: only the summed input gradient is wanted
+        if (!dx) return FT_OK;
+        ft_lora_dx_desc d[3];
+        for (int i = 0; i < n; i++) d[i] = ft_lora_dx_desc{dys[i], ls[i]->w, ls[i]->dtype, nullptr, nullptr, ls[i]->out, 0};
+        return ft_lora_linear_dx_group(ctx, d, (size_t)n, nullptr, dx, T, ls[0]->in);
     }
     FT_TRY(ft_thin_rowwise(ctx, rows, n));
     FT_TRY(ft_thin_colwise(ctx, cols, 2 * n));
-    for (int i = 0; i < n && dx; i++)
-        FT_TRY(ft_lora_linear_dx(ctx, dys[i], ls[i]->w, ls[i]->dtype, dts[i], ls[i]->a, i > 0 ? dx : nullptr, dx, T,
-                                 ls[i]->in, ls[i]->out, ls[i]->r));
+    if (dx) {
+        ft_lora_dx_desc d[3];
+        for (int i = 0; i < n; i++)
+            d[i] = ft_lora_dx_desc{dys[i], ls[i]->w, ls[i]->dtype, dts[i], ls[i]->a, ls[i]->out, ls[i]->r};
+        FT_TRY(ft_lora_linear_dx_group(ctx, d, (size_t)n, nullptr, dx, T, ls[0]->in));
+    }
     return FT_OK;
 }
 
@@ -364,9 +391,12 @@ int model_forward(ft_model* m, const uint32_t* rows_host, size_t B, size_t S) {
             float* ts[3] = {a.tq, a.tk, a.tv};
             FT_TRY(lora_down_group(ctx, ls, ts, 3, a.h1, T));
         }
-        FT_TRY(linear_gemm(ctx, L.q, a.h1, a.tq, a.q, T));
-        FT_TRY(linear_gemm(ctx, L.k, a.h1, a.tk, a.k, T));
-        FT_TRY(linear_gemm(ctx, L.v, a.h1, a.tv, a.v, T));
+        {
+            LinearW* ls[3] = {&L.q, &L.k, &L.v};
+            const float* ts[3] = {a.tq, a.tk, a.tv};
+            float* ys[3] = {a.q, a.k, a.v};
+            FT_TRY(linear_gemm_group(ctx, ls, ts, ys, 3, a.h1, T));
+        }
         if (m->rope_table) {
             FT_TRY(ft_internal_rope_pair(ctx, a.q, a.q, nh, a.k, a.k, nkv, m->rope_table, B, S, D, 0));
         } else {
@@ -382,8 +412,12 @@ int model_forward(ft_model* m, const uint32_t* rows_host, size_t B, size_t S) {
             float* ts[2] = {a.tup, a.tgate};
             FT_TRY(lora_down_group(ctx, ls, ts, 2, a.h2, T));
         }
-        FT_TRY(linear_gemm(ctx, L.up, a.h2, a.tup, a.up, T));
-        FT_TRY(linear_gemm(ctx, L.gate, a.h2, a.tgate, a.gate, T));
+        {
+            LinearW* ls[2] = {&L.up, &L.gate};
+            const float* ts[2] = {a.tup, a.tgate};
+            float* ys[2] = {a.up, a.gate};
+            FT_TRY(linear_gemm_group(ctx, ls, ts, ys, 2, a.h2, T));
+        }
         FT_TRY(ft_silu_gate_fused(ctx, a.gate, a.up, a.act, T * F));
         FT_TRY(linear_forward(ctx, L.down, a.act, a.tdown, x_next, T, a.h));
     }

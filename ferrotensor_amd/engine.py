@@ -239,6 +239,10 @@ def _p(t):
     return C.c_void_p(t.ptr) if t is not None else C.c_void_p(0)
 
 
+def _v(t):
+    return t.ptr if t is not None else None
+
+
 class ComputeEngine:
     """`ComputeEngine` (engine/mod.rs:215-274): the hot subset of its methods."""
 
@@ -294,6 +298,31 @@ class ComputeEngine:
         r = b.shape[0] if b is not None else 0
         assert K == K2 and y.numel() == M * N
         check(self._lib.ft_lora_linear(ctx.handle, _p(x), _p(w), w.dtype, _p(t), _p(b), _p(residual), _p(y), M, K, N, r))
+
+    def lora_linear_group(self, ctx, x, linears):
+        """linears: [(w, t, b, y, residual)] sharing the input x; one launch when all can be batched."""
+        from ._lib import LoraLinearDescC
+        M, K = x.shape
+        descs = (LoraLinearDescC * len(linears))()
+        for d, (w, t, b, y, residual) in zip(descs, linears):
+            assert w.shape[0] == K and y.numel() == M * w.shape[1]
+            d.w, d.w_dtype, d.t, d.b, d.residual, d.y = _v(w), w.dtype, _v(t), _v(b), _v(residual), _v(y)
+            d.N, d.r = w.shape[1], (b.shape[0] if b is not None else 0)
+        check(self._lib.ft_lora_linear_group(ctx.handle, _p(x), descs, len(linears), M, K))
+
+    def lora_linear_dx_group(self, ctx, linears, dx, residual=None):
+        """linears: [(dy, w, dt, a)] of linears that shared their input; dx = (residual +) sum of their dx."""
+        from ._lib import LoraDxDescC
+        M = linears[0][0].shape[0]
+        K = linears[0][1].shape[0]
+        descs = (LoraDxDescC * len(linears))()
+        for d, (dy, w, dt, a) in zip(descs, linears):
+            assert list(dy.shape) == [M, w.shape[1]]
+            assert w.shape[0] == K
+            d.dy, d.w, d.w_dtype, d.dt, d.a = _v(dy), _v(w), w.dtype, _v(dt), _v(a)
+            d.N, d.r = w.shape[1], (a.shape[1] if a is not None else 0)
+        assert dx.numel() == M * K
+        check(self._lib.ft_lora_linear_dx_group(ctx.handle, descs, len(linears), _p(residual), _p(dx), M, K))
 
     def lora_grad_down(self, ctx, dy, b, dt, scale):
         M, N = dy.shape

@@ -131,6 +131,42 @@ int ft_matmul_bt_f16b(ft_context* ctx, const float* a, const uint16_t* b, float*
  *      ferrotensor-graph/src/lib.rs:112-126, and of its backward,
  *      ferrotensor-autograd/src/lib.rs:262-290, 340-357) ---------------------- */
 
+/* Up to 3 linears that read the same input in ONE launch (q/k/v, gate/up of
+ * Lfm2Model::forward, ferrotensor-graph/src/lib.rs:255-330): linear i computes
+ * y_i[M,N_i] = x[M,K] @ w_i[K,N_i] (+ t_i[M,r_i] @ b_i[r_i,N_i]) (+ residual_i),
+ * exactly as ft_lora_linear does. The tiles of all of them share one grid, so a
+ * narrow projection no longer leaves most of the chip idle. Linears that cannot
+ * take the batched path (f32 weights, unaligned operands) run one by one. */
+typedef struct ft_lora_linear_desc {
+    const void* w;
+    int32_t w_dtype;       /* FT_DTYPE_F32 or FT_DTYPE_F16 */
+    const float* t;        /* NULL when r == 0 */
+    const float* b;
+    const float* residual; /* NULL = none; may alias y */
+    float* y;
+    size_t N;
+    size_t r;
+} ft_lora_linear_desc;
+int ft_lora_linear_group(ft_context* ctx, const float* x, const ft_lora_linear_desc* linears, size_t count,
+                         size_t M, size_t K);
+
+/* The input gradient shared by up to 3 linears that read the same input
+ * (MatMulNode::backward for each of them followed by the AddNode accumulation,
+ * ferrotensor-autograd/src/lib.rs:262-357), in ONE launch:
+ * dx[M,K] = (residual) + sum_i ( dy_i[M,N_i] @ w_i[K,N_i]^T + dt_i[M,r_i] @ a_i[K,r_i]^T ).
+ * The sum runs inside the accumulators: one K loop over the concatenated N_i. */
+typedef struct ft_lora_dx_desc {
+    const float* dy;
+    const void* w;
+    int32_t w_dtype;
+    const float* dt;       /* NULL when r == 0 */
+    const float* a;
+    size_t N;
+    size_t r;
+} ft_lora_dx_desc;
+int ft_lora_linear_dx_group(ft_context* ctx, const ft_lora_dx_desc* linears, size_t count, const float* residual,
+                            float* dx, size_t M, size_t K);
+
 /* t[M,r] = scale * (x[M,K] @ a[K,r]): the `x @ A` product with the alpha/rank
  * scale applied where the reference applies it (graph/src/lib.rs:116-122).
  * r <= 32. */

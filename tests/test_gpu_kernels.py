@@ -149,6 +149,48 @@ def test_fused_lora_linear_forward_and_backward(g, M, K, N, r, f16):
     assert_close("dA", da.to_numpy(), grads["l.lora_a"], atol=2e-3, rtol=1e-4)
 
 
+@pytest.mark.parametrize("M,K,Ns,r,f16", [(256, 960, (960, 320, 320), 8, True), (100, 64, (64, 32, 96), 4, True),
+                                          (192, 128, (320, 256), 0, True), (64, 32, (48, 40), 8, False),
+                                          (130, 96, (40, 72, 8), 16, True)])
+def test_grouped_linears_match_single_calls(g, M, K, Ns, r, f16):
+    """q/k/v (gate/up) of one input in one launch, and their summed input gradient in one launch."""
+    from ferrotensor_amd import UnifiedTensor
+    ctx, eng = g
+    x = rnd(1, M, K)
+    xt = up(ctx, x)
+    fwd, bwd, want_dx = [], [], np.zeros((M, K), np.float32)
+    res = rnd(50, M, K)
+    for i, N in enumerate(Ns):
+        w = rnd(10 + i, K, N, scale=0.05)
+        wr = cpu.round_f16(w) if f16 else w
+        wt = UnifiedTensor.from_f32_as_f16(ctx, w, [K, N]) if f16 else up(ctx, w)
+        dy = rnd(20 + i, M, N)
+        if r:
+            A, B = rnd(30 + i, K, r, scale=0.1), rnd(40 + i, r, N, scale=0.1)
+            t, dt = rnd(60 + i, M, r), rnd(70 + i, M, r)
+            want_y = cpu.matmul(x, wr) + cpu.matmul(t, B)
+            want_dx += cpu.matmul(dy, np.ascontiguousarray(wr.T)) + cpu.matmul(dt, np.ascontiguousarray(A.T))
+            y = empty(ctx, M, N)
+            fwd.append((wt, up(ctx, t), up(ctx, B), y, None))
+            bwd.append((up(ctx, dy), wt, up(ctx, dt), up(ctx, A)))
+        else:
+            want_y = cpu.matmul(x, wr)
+            want_dx += cpu.matmul(dy, np.ascontiguousarray(wr.T))
+            y = empty(ctx, M, N)
+            fwd.append((wt, None, None, y, None))
+            bwd.append((up(ctx, dy), wt, None, None))
+        fwd[-1] = fwd[-1] + (want_y,)
+    eng.lora_linear_group(ctx, xt, [f[:5] for f in fwd])
+    for i, f in enumerate(fwd):
+        assert_close("group y%d" % i, f[3].to_numpy(), f[5], atol=1e-3, rtol=1e-4)
+    dx = empty(ctx, M, K)
+    eng.lora_linear_dx_group(ctx, bwd, dx)
+    assert_close("group dx", dx.to_numpy(), want_dx, atol=3e-3, rtol=1e-4)
+    dx2 = up(ctx, res)
+    eng.lora_linear_dx_group(ctx, bwd, dx2, residual=dx2)
+    assert_close("group dx + residual", dx2.to_numpy(), want_dx + res, atol=3e-3, rtol=1e-4)
+
+
 @pytest.mark.parametrize("rows,size", [(1, 1), (3, 7), (37, 96), (16, 576), (64, 960), (5, 2048), (3, 2100)])
 def test_rms_norm_forward_backward(g, rows, size):
     ctx, eng = g
