@@ -519,6 +519,195 @@ __global__ __launch_bounds__(dkdv_waves(DP) * 64) void attn_bwd_dkdv_kernel(Attn
     }
 }
 
+// ---------------------------------------------------------------------------
+// dK/dV for whole, aligned head dims (D == DP): the same decomposition, with the
+// operand traffic arranged for latency. Every tile is read from global memory
+// once, as coalesced 16-byte quads: the key block's K and V go to a tile in LDS
+// that all waves share; an item's Q and dO quads go to registers (they are the
+// A operands of S and dP), and from there into a wave-private LDS tile from
+// which the same data is read back transposed (lane = head-dim index) as the A
+// operands of dV^T and dK^T. The next item's quads are fetched into the same
+// registers while the current item's second half multiplies, so a wave sees one
+// global latency per launch, not two per item.
+// LDS rows are 16-byte-chunk swizzled (chunk c of row r sits at c ^ (r & 15)):
+// quad reads/writes of 16 consecutive rows and transposed reads of 32
+// consecutive columns are both conflict-free.
+// Grid (B*Hkv, ceil(Sk/32)): key block 0 (the most items under the causal mask)
+// is dispatched first.
+// ---------------------------------------------------------------------------
+template <int DP>
+__device__ __forceinline__ int sw_off(int row, int chunk) {
+    constexpr int CH = DP / 4;
+    return row * DP + ((chunk ^ (row & (CH < 16 ? CH - 1 : 15))) * 4);
+}
+
+template <int DP>
+__global__ __launch_bounds__(512) void attn_bwd_dkdv_lds_kernel(AttnArgs p) {
+    constexpr int NF = DP / 32;
+    constexpr int NS = DP / 8;
+    constexpr int NWV = 8;
+    constexpr int TILE = 32 * DP;
+    constexpr int REGION = 2 * DP * 33;                                  // reduction layout: dK^T, dV^T as [d][33]
+    constexpr int PRIV = (2 * TILE + 64) > REGION ? (2 * TILE + 64) : REGION;  // Q tile, dO tile, 32 (Delta, LSE)
+    extern __shared__ __attribute__((aligned(16))) float smem[];
+    float* ks = smem;            // K * scale
+    float* vs = smem + TILE;
+    float* priv = smem + 2 * TILE + (threadIdx.x / 64) * PRIV;
+    float* qs = priv;
+    float* dos = priv + TILE;
+    float* sts = priv + 2 * TILE;
+
+    const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
+    const int l32 = lane % 32, half = lane / 32;
+    const int b = blockIdx.x / p.Hkv, kvh = blockIdx.x % p.Hkv;
+    const int G = p.H / p.Hkv;
+    const int kb0 = blockIdx.y * 32;
+    const int key = kb0 + l32;
+    const bool k_ok = key < p.Sk;
+    const long qst = (long)p.H * DP;
+
+    // K and V of the key block -> shared LDS tile (rows past Sk are clamped: masked below).
+    for (int e = tid; e < 32 * (DP / 4); e += NWV * 64) {
+        const int r = e / (DP / 4), c = e % (DP / 4);
+        int kr = kb0 + r;
+        kr = kr < p.Sk ? kr : p.Sk - 1;
+        const long o = (((long)b * p.Sk + kr) * p.Hkv + kvh) * DP + 4 * c;
+        const float4 kq = *reinterpret_cast<const float4*>(p.k + o);
+        *reinterpret_cast<float4*>(ks + sw_off<DP>(r, c)) =
+            make_float4(kq.x * p.scale, kq.y * p.scale, kq.z * p.scale, kq.w * p.scale);
+        *reinterpret_cast<float4*>(vs + sw_off<DP>(r, c)) = *reinterpret_cast<const float4*>(p.v + o);
+    }
+
+    floatx16 dk[NF], dv[NF];
+#pragma unroll
+    for (int f = 0; f < NF; f++) {
+        dk[f] = zero16();
+        dv[f] = zero16();
+    }
+
+    // Query blocks that can see key block kb0.
+    const int nqb = (p.Sq + 31) / 32;
+    int qb_start = 0;
+    if (p.causal) {
+        const int first_q = kb0 - p.causal_offset;  // smallest i with i + offset >= kb0
+        qb_start = first_q > 0 ? first_q / 32 : 0;
+    }
+    const int per_head = nqb > qb_start ? nqb - qb_start : 0;
+    const int items = per_head * G;
+
+    float4 qa[NS], qc[NS];
+    float2 st_mine = make_float2(0.0f, kLseEmpty);
+    auto fetch = [&](int item) {
+        const int g = item / per_head;
+        const int q0 = (qb_start + item % per_head) * 32;
+        const int h = kvh * G + g;
+        int qr = q0 + l32;
+        const bool ok = qr < p.Sq;
+        qr = ok ? qr : p.Sq - 1;
+        const float* qrow = p.q + ((long)b * p.Sq * p.H + h) * DP + qr * qst;
+        const float* dorow = p.d_out + ((long)b * p.Sq * p.H + h) * DP + qr * qst;
+#pragma unroll
+        for (int s = 0; s < NS; s++) {
+            qa[s] = *reinterpret_cast<const float4*>(qrow + 8 * s + 4 * half);
+            qc[s] = *reinterpret_cast<const float4*>(dorow + 8 * s + 4 * half);
+        }
+        const float2 t = *reinterpret_cast<const float2*>(p.stats + 2 * (((long)b * p.H + h) * p.Sq + qr));
+        st_mine = ok ? t : make_float2(0.0f, kLseEmpty);
+    };
+    if (wave < items) fetch(wave);
+    __syncthreads();  // K/V tile complete
+
+    for (int item = wave; item < items; item += NWV) {
+        const int q0 = (qb_start + item % per_head) * 32;
+        // this item's tiles -> private LDS (for the transposed reads), S and dP from the registers
+#pragma unroll
+        for (int s = 0; s < NS; s++) {
+            *reinterpret_cast<float4*>(qs + sw_off<DP>(l32, 2 * s + half)) = qa[s];
+            *reinterpret_cast<float4*>(dos + sw_off<DP>(l32, 2 * s + half)) = qc[s];
+        }
+        if (half == 0) *reinterpret_cast<float2*>(sts + 2 * l32) = st_mine;
+        floatx16 s = zero16(), dp = zero16();
+#pragma unroll
+        for (int st = 0; st < NS; st++) {
+            const float4 kq = *reinterpret_cast<const float4*>(ks + sw_off<DP>(l32, 2 * st + half));
+            const float4 vq = *reinterpret_cast<const float4*>(vs + sw_off<DP>(l32, 2 * st + half));
+            s = MFMA(qa[st].x, kq.x, s);
+            s = MFMA(qa[st].y, kq.y, s);
+            s = MFMA(qa[st].z, kq.z, s);
+            s = MFMA(qa[st].w, kq.w, s);
+            dp = MFMA(qc[st].x, vq.x, dp);
+            dp = MFMA(qc[st].y, vq.y, dp);
+            dp = MFMA(qc[st].z, vq.z, dp);
+            dp = MFMA(qc[st].w, vq.w, dp);
+            if (st % 2 == 1) __builtin_amdgcn_sched_barrier(0);  // bounds how many LDS quads are live
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        // the next item's quads travel while the rest of this item is computed
+        if (item + NWV < items) fetch(item + NWV);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int t = 0; t < 16; t++) {
+            const int r = row_of(t, half);
+            const int qi = q0 + r;
+            const float2 st2 = *reinterpret_cast<const float2*>(sts + 2 * r);
+            const bool vis = k_ok && qi < p.Sq && (!p.causal || key <= qi + p.causal_offset);
+            const float pij = vis ? __expf(s[t] - st2.y) : 0.0f;
+            s[t] = pij;                     // P
+            dp[t] = pij * (dp[t] - st2.x);  // dS
+        }
+        // transposed operands in groups of 4 rows: 4 * 2 * NF LDS reads, then their MFMAs
+#pragma unroll
+        for (int t4 = 0; t4 < 16; t4 += 4) {
+            float ao[4][NF], aq[4][NF];
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const int r = row_of(t4 + u, half);
+#pragma unroll
+                for (int f = 0; f < NF; f++) {
+                    const int d = f * 32 + l32;
+                    ao[u][f] = dos[sw_off<DP>(r, d / 4) + (d & 3)];
+                    aq[u][f] = qs[sw_off<DP>(r, d / 4) + (d & 3)];
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < 4; u++)
+#pragma unroll
+                for (int f = 0; f < NF; f++) {
+                    dv[f] = MFMA(ao[u][f], s[t4 + u], dv[f]);
+                    dk[f] = MFMA(aq[u][f], dp[t4 + u], dk[f]);
+                }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+
+    // Cross-wave sum in wave order: red[wave][which][d][33] over the private regions.
+#pragma unroll
+    for (int f = 0; f < NF; f++)
+#pragma unroll
+        for (int t = 0; t < 16; t++) {
+            const int d = f * 32 + row_of(t, half);
+            priv[d * 33 + l32] = dk[f][t];
+            priv[DP * 33 + d * 33 + l32] = dv[f][t];
+        }
+    __syncthreads();
+    const float* red = smem + 2 * TILE;
+    for (int e = tid; e < 32 * DP; e += NWV * 64) {
+        const int kk = e / DP, d = e % DP;
+        const int krow = kb0 + kk;
+        if (krow < p.Sk) {
+            float sk = 0.0f, sv = 0.0f;
+#pragma unroll
+            for (int w = 0; w < NWV; w++) {
+                sk += red[w * PRIV + d * 33 + kk];
+                sv += red[w * PRIV + DP * 33 + d * 33 + kk];
+            }
+            const long o = (((long)b * p.Sk + krow) * p.Hkv + kvh) * DP + d;
+            p.dk[o] = sk * p.scale;  // dK = scale * sum dS Q (Q is read unscaled)
+            p.dv[o] = sv;
+        }
+    }
+}
+
 // The unguarded vector loads need whole, aligned quads in every row.
 bool attn_full(const AttnArgs& a, int DP) {
     auto al = [](const void* q) { return q == nullptr || (((uintptr_t)q) & 15) == 0; };
@@ -555,6 +744,24 @@ int launch_bwd(ft_context* ctx, const AttnArgs& a) {
             hipLaunchKernelGGL((attn_bwd_dq_kernel<DP, false>), grid, dim3(kKeySplit * 64), 0, ctx->stream, a);
     }
     FT_LAUNCH_CHECK();
+    if constexpr (DP <= 64) {
+        if (full && a.Sk < 32 * 65535) {
+            constexpr int TILE = 32 * DP, REGION = 2 * DP * 33;
+            constexpr int PRIV = (2 * TILE + 64) > REGION ? (2 * TILE + 64) : REGION;
+            constexpr size_t smem_lds = (size_t)(2 * TILE + 8 * PRIV) * sizeof(float);
+            static bool attr_lds = false;
+            if (!attr_lds) {
+                FT_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_bwd_dkdv_lds_kernel<DP>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem_lds));
+                attr_lds = true;
+            }
+            const dim3 grid3((unsigned)(a.B * a.Hkv), ft_div_up(a.Sk, 32));
+            ft_prof_scope prof(ctx, "attn_bwd_dkdv_kernel", 1.5 * fl, by * 0.5);
+            hipLaunchKernelGGL((attn_bwd_dkdv_lds_kernel<DP>), grid3, dim3(512), smem_lds, ctx->stream, a);
+            FT_LAUNCH_CHECK();
+            return FT_OK;
+        }
+    }
     constexpr size_t smem = (size_t)dkdv_waves(DP) * 2 * DP * 33 * sizeof(float);
     static bool attr_set = false;
     if (!attr_set) {

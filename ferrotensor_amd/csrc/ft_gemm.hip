@@ -657,10 +657,10 @@ __global__ __launch_bounds__(256) void gemm_async_kernel(AsyncBatch g) {
         }
     }
 
-    // Per-lane source coordinates, constant over the K loop: byte offset =
-    // row * (leading dimension in bytes) + col. With one segment the product is
-    // formed once, here.
-    unsigned rowA[A_CH], colA[A_CH], rowB[B_CH], colB[B_CH];
+    // Per-lane source coordinates: byte offset = row * (leading dimension in
+    // bytes) + col. The products are formed once per segment (offA / offB), so
+    // the K loop itself carries no per-lane address arithmetic.
+    unsigned rowA[A_CH], colA[A_CH], rowB[B_CH], colB[B_CH], offA[A_CH], offB[B_CH];
 #pragma unroll
     for (int j = 0; j < A_CH; j++) {
         const int c = wave + 4 * j, r = lane / 8, cs = lane % 8;
@@ -668,7 +668,7 @@ __global__ __launch_bounds__(256) void gemm_async_kernel(AsyncBatch g) {
         row = row < M ? row : M - 1;
         rowA[j] = (unsigned)row;
         colA[j] = (unsigned)((cs ^ r) * 16);
-        if constexpr (NSEG == 1) colA[j] += rowA[j] * (unsigned)lda_b[0];
+        offA[j] = rowA[j] * (unsigned)lda_b[0] + colA[j];
     }
 #pragma unroll
     for (int j = 0; j < B_CH; j++) {
@@ -687,29 +687,40 @@ __global__ __launch_bounds__(256) void gemm_async_kernel(AsyncBatch g) {
             rowB[j] = (unsigned)(c * RPC + kr);
             colB[j] = (unsigned)(col * 2);
         }
-        if constexpr (NSEG == 1) colB[j] += rowB[j] * (unsigned)ldb_b[0];
+        offB[j] = rowB[j] * (unsigned)ldb_b[0] + colB[j];
     }
+    int seg_cur = 0;           // segment the offsets are formed for
+    int seg_first = 0;         // its first tile
+    const char* aseg = abase[0];
+    const char* bseg = bbase[0];
+    long b_step = LAYOUT == 1 ? 64L : 32L * ldb_b[0];  // bytes per K tile
 
     auto issue = [&](int t, float* st) {
         t = t < nt ? t : nt - 1;  // past the end: re-read the last tile into a stage nobody reads
-        int s = 0, tl = t;
         if constexpr (NSEG > 1) {
-            if (t >= tend[0]) s = 1, tl = t - tend[0];
-            if (t >= tend[1]) s = 2, tl = t - tend[1];
-        }
-        const int la = seg_pick<NSEG>(lda_b, s), lb = seg_pick<NSEG>(ldb_b, s);
-        const char* at = seg_pick<NSEG>(abase, s) + (long)tl * 128;
-        const char* bt = seg_pick<NSEG>(bbase, s) + (long)tl * (LAYOUT == 1 ? 64L : 32L * lb);
+            int s = 0;
+            if (t >= tend[0]) s = 1;
+            if (t >= tend[1]) s = 2;
+            if (s != seg_cur) {  // uniform, taken once per segment
+                seg_cur = s;
+                seg_first = s == 1 ? tend[0] : tend[1];
+                const int la = seg_pick<NSEG>(lda_b, s), lb = seg_pick<NSEG>(ldb_b, s);
+                aseg = seg_pick<NSEG>(abase, s);
+                bseg = seg_pick<NSEG>(bbase, s);
+                b_step = LAYOUT == 1 ? 64L : 32L * lb;
 #pragma unroll
-        for (int j = 0; j < A_CH; j++) {
-            const unsigned off = NSEG == 1 ? colA[j] : rowA[j] * (unsigned)la + colA[j];
-            glds16(at, off, st + (wave + 4 * j) * 256);
-        }
+                for (int j = 0; j < A_CH; j++) offA[j] = rowA[j] * (unsigned)la + colA[j];
 #pragma unroll
-        for (int j = 0; j < B_CH; j++) {
-            const unsigned off = NSEG == 1 ? colB[j] : rowB[j] * (unsigned)lb + colB[j];
-            glds16(bt, off, st + A_FLOATS + (wave + 4 * j) * 256);
+                for (int j = 0; j < B_CH; j++) offB[j] = rowB[j] * (unsigned)lb + colB[j];
+            }
         }
+        const int tl = t - seg_first;
+        const char* at = aseg + (long)tl * 128;
+        const char* bt = bseg + (long)tl * b_step;
+#pragma unroll
+        for (int j = 0; j < A_CH; j++) glds16(at, offA[j], st + (wave + 4 * j) * 256);
+#pragma unroll
+        for (int j = 0; j < B_CH; j++) glds16(bt, offB[j], st + A_FLOATS + (wave + 4 * j) * 256);
     };
     auto a_frag = [&](const float* st, int s, int row) -> float4 {
         const int kq = 2 * s + half;
