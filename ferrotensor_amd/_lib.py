@@ -88,6 +88,8 @@ SIGNATURES = {
     "ft_lora_down": [_P, _P, _P, _P, _SZ, _SZ, _SZ, _F],
     "ft_lora_linear_group": [_P, _P, C.POINTER(LoraLinearDescC), _SZ, _SZ, _SZ],
     "ft_lora_linear_dx_group": [_P, C.POINTER(LoraDxDescC), _SZ, _P, _P, _SZ, _SZ],
+    "ft_mlp_gate_up": [_P, _P, _P, _P, _I, _P, _P, _P, _SZ, _SZ, _SZ],
+    "ft_mlp_down_backward": [_P, _P, _P, _I, _P, _P, _P, _P, _P, _SZ, _SZ, _SZ],
     "ft_lora_linear": [_P, _P, _P, _I, _P, _P, _P, _P, _SZ, _SZ, _SZ, _SZ],
     "ft_lora_grad_down": [_P, _P, _P, _P, _SZ, _SZ, _SZ, _F],
     "ft_lora_linear_dx": [_P, _P, _P, _I, _P, _P, _P, _P, _SZ, _SZ, _SZ, _SZ],

@@ -81,15 +81,32 @@ __device__ __forceinline__ float ld_one(const float* row, int d, int D) {
     return d < D ? row[d] : 0.0f;
 }
 
+// Work distribution. Under the causal mask a block's cost grows (or shrinks)
+// with its index. The items of a launch are ordered block-major, most expensive
+// block index first, over a 1-D grid: the long items start first (the tail of
+// the launch is made of short ones), and because consecutive workgroups go
+// round-robin to the 8 XCDs, every XCD receives the same mix of block indices
+// (a (block, batch*head) grid with 8 blocks would hand XCD c all the blocks
+// of index c). `j` counts the block indices in dispatch order.
+__device__ __forceinline__ bool attn_work_item(int nblk, int nbh, int& j, int& bh) {
+    const int t = (int)blockIdx.x;
+    if (t >= nblk * nbh) return false;
+    j = t / nbh;
+    bh = t % nbh;
+    return true;
+}
+inline unsigned attn_grid(size_t nblk, size_t nbh) { return (unsigned)(nblk * nbh); }
+
 // ---------------------------------------------------------------------------
 // Forward. A workgroup owns 32 queries of one (batch, head); its NSPL waves take
 // every NSPL-th block of 32 keys and merge their partial softmax states through
 // LDS at the end (shorter critical path under the causal mask, and two waves
 // per SIMD to overlap one wave's softmax arithmetic with the other's MFMAs).
-// Grid (ceil(Sq/32), B*H); query blocks are issued last-first: the last block
-// has the longest key loop, so the long ones start first.
+// One workgroup per (query block, batch*head) item (attn_work_item); within a
+// head the last query block, which has the longest key loop, starts first.
 // ---------------------------------------------------------------------------
-constexpr int kKeySplit = 2;
+constexpr int kKeySplit = 4;    // forward
+constexpr int kKeySplitDq = 2;  // dQ: two waves per SIMD need <= 256 registers per lane
 
 template <int DP, bool FULL>
 __global__ __launch_bounds__(kKeySplit * 64) void attn_fwd_kernel(AttnArgs p) {
@@ -98,9 +115,12 @@ __global__ __launch_bounds__(kKeySplit * 64) void attn_fwd_kernel(AttnArgs p) {
     constexpr int NSPL = kKeySplit;
     __shared__ float merge[(NSPL - 1) * 64 * (NF * 16 + 2)];
     const int lane = threadIdx.x % 64, wave = threadIdx.x / 64, l32 = lane % 32, half = lane / 32;
-    const int b = blockIdx.y / p.H, h = blockIdx.y % p.H;
+    int blk_j, bh_i;
+    const int nqb_grid = (p.Sq + 31) / 32;
+    if (!attn_work_item(nqb_grid, p.B * p.H, blk_j, bh_i)) return;
+    const int b = bh_i / p.H, h = bh_i % p.H;
     const int kvh = h / (p.H / p.Hkv);
-    const int q0 = ((int)gridDim.x - 1 - (int)blockIdx.x) * 32;
+    const int q0 = (nqb_grid - 1 - blk_j) * 32;  // the last query block has the longest key loop: first
     const int qi = q0 + l32;
     const bool q_ok = qi < p.Sq;
     const int qc = q_ok ? qi : p.Sq - 1;
@@ -249,15 +269,18 @@ __global__ __launch_bounds__(kKeySplit * 64) void attn_fwd_kernel(AttnArgs p) {
 // Same decomposition as the forward.
 // ---------------------------------------------------------------------------
 template <int DP, bool FULL>
-__global__ __launch_bounds__(kKeySplit * 64) void attn_bwd_dq_kernel(AttnArgs p) {
+__global__ __launch_bounds__(kKeySplitDq * 64) void attn_bwd_dq_kernel(AttnArgs p) {
     constexpr int NF = DP / 32;
     constexpr int NS = DP / 8;
-    constexpr int NSPL = kKeySplit;
+    constexpr int NSPL = kKeySplitDq;
     __shared__ float merge[(NSPL - 1) * 64 * NF * 16];
     const int lane = threadIdx.x % 64, wave = threadIdx.x / 64, l32 = lane % 32, half = lane / 32;
-    const int b = blockIdx.y / p.H, h = blockIdx.y % p.H;
+    int blk_j, bh_i;
+    const int nqb_grid = (p.Sq + 31) / 32;
+    if (!attn_work_item(nqb_grid, p.B * p.H, blk_j, bh_i)) return;
+    const int b = bh_i / p.H, h = bh_i % p.H;
     const int kvh = h / (p.H / p.Hkv);
-    const int q0 = ((int)gridDim.x - 1 - (int)blockIdx.x) * 32;
+    const int q0 = (nqb_grid - 1 - blk_j) * 32;  // the last query block has the longest key loop: first
     const int qi = q0 + l32;
     const bool q_ok = qi < p.Sq;
     const int qc = q_ok ? qi : p.Sq - 1;
@@ -393,8 +416,8 @@ __global__ __launch_bounds__(kKeySplit * 64) void attn_bwd_dq_kernel(AttnArgs p)
 // the query heads of the group and over the query blocks that can see them.
 // The (head, query block) items are dealt round-robin to the NWV waves of the
 // workgroup; the partial results are added in wave order through LDS (no
-// atomics: the result is deterministic). Grid (ceil(Sk/32), B*Hkv), key blocks
-// issued first-first (under the causal mask key block 0 has the most items).
+// atomics: the result is deterministic). One workgroup per (key block, batch*kv
+// head) item, key block 0 first (under the causal mask it has the most items).
 // ---------------------------------------------------------------------------
 // 8 waves for head dims up to 64; 4 for 128 (the reduction buffer must fit LDS).
 constexpr int dkdv_waves(int dp) { return dp <= 64 ? 8 : 4; }
@@ -409,9 +432,11 @@ __global__ __launch_bounds__(dkdv_waves(DP) * 64) void attn_bwd_dkdv_kernel(Attn
 
     const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
     const int l32 = lane % 32, half = lane / 32;
-    const int b = blockIdx.y / p.Hkv, kvh = blockIdx.y % p.Hkv;
+    int blk_j, bh_i;
+    if (!attn_work_item((p.Sk + 31) / 32, p.B * p.Hkv, blk_j, bh_i)) return;
+    const int b = bh_i / p.Hkv, kvh = bh_i % p.Hkv;
     const int G = p.H / p.Hkv;
-    const int kb0 = blockIdx.x * 32;
+    const int kb0 = blk_j * 32;  // key block 0 has the most items under the causal mask: first
     const int key = kb0 + l32;
     const bool k_ok = key < p.Sk;
     const long koff = (((long)b * p.Sk + (k_ok ? key : p.Sk - 1)) * p.Hkv + kvh) * p.D;
@@ -532,8 +557,8 @@ __global__ __launch_bounds__(dkdv_waves(DP) * 64) void attn_bwd_dkdv_kernel(Attn
 // LDS rows are 16-byte-chunk swizzled (chunk c of row r sits at c ^ (r & 15)):
 // quad reads/writes of 16 consecutive rows and transposed reads of 32
 // consecutive columns are both conflict-free.
-// Grid (B*Hkv, ceil(Sk/32)): key block 0 (the most items under the causal mask)
-// is dispatched first.
+// One workgroup per (key block, batch*kv head) item, key block 0 (the most
+// items under the causal mask) first within a head.
 // ---------------------------------------------------------------------------
 template <int DP>
 __device__ __forceinline__ int sw_off(int row, int chunk) {
@@ -559,9 +584,11 @@ __global__ __launch_bounds__(512) void attn_bwd_dkdv_lds_kernel(AttnArgs p) {
 
     const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
     const int l32 = lane % 32, half = lane / 32;
-    const int b = blockIdx.x / p.Hkv, kvh = blockIdx.x % p.Hkv;
+    int blk_j, bh_i;
+    if (!attn_work_item((p.Sk + 31) / 32, p.B * p.Hkv, blk_j, bh_i)) return;
+    const int b = bh_i / p.Hkv, kvh = bh_i % p.Hkv;
     const int G = p.H / p.Hkv;
-    const int kb0 = blockIdx.y * 32;
+    const int kb0 = blk_j * 32;  // key block 0 has the most items under the causal mask: first
     const int key = kb0 + l32;
     const bool k_ok = key < p.Sk;
     const long qst = (long)p.H * DP;
@@ -708,6 +735,306 @@ __global__ __launch_bounds__(512) void attn_bwd_dkdv_lds_kernel(AttnArgs p) {
     }
 }
 
+// ---------------------------------------------------------------------------
+// Forward and dQ for whole, aligned head dims (D == DP), same operand scheme as
+// the dK/dV kernel above: a key block's K and V are read from global memory once
+// as coalesced quads into registers (the next block's while the current one
+// multiplies); the operand that is needed with the head dim as the MFMA row
+// (V^T in the forward, K^T for dQ) is written to a wave-private swizzled LDS
+// tile and read back transposed.
+// ---------------------------------------------------------------------------
+template <int DP>
+__global__ __launch_bounds__(kKeySplit * 64) void attn_fwd_lds_kernel(AttnArgs p) {
+    constexpr int NF = DP / 32;
+    constexpr int NS = DP / 8;
+    constexpr int NSPL = kKeySplit;
+    constexpr int TILE = 32 * DP;
+    constexpr int MERGE = 64 * (NF * 16 + 2);
+    constexpr int PRIV = TILE > MERGE ? TILE : MERGE;
+    __shared__ __attribute__((aligned(16))) float lds[NSPL * PRIV];
+    const int lane = threadIdx.x % 64, wave = threadIdx.x / 64, l32 = lane % 32, half = lane / 32;
+    float* vt = lds + wave * PRIV;
+    int blk_j, bh_i;
+    const int nqb_grid = (p.Sq + 31) / 32;
+    if (!attn_work_item(nqb_grid, p.B * p.H, blk_j, bh_i)) return;
+    const int b = bh_i / p.H, h = bh_i % p.H;
+    const int kvh = h / (p.H / p.Hkv);
+    const int q0 = (nqb_grid - 1 - blk_j) * 32;  // the last query block has the longest key loop: first
+    const int qi = q0 + l32;
+    const bool q_ok = qi < p.Sq;
+    const int qc = q_ok ? qi : p.Sq - 1;
+    const float* qrow = p.q + (((long)b * p.Sq + qc) * p.H + h) * DP;
+    const long kst = (long)p.Hkv * DP;
+    const float* kbase = p.k + ((long)b * p.Sk * p.Hkv + kvh) * DP;
+    const float* vbase = p.v + ((long)b * p.Sk * p.Hkv + kvh) * DP;
+
+    float4 qreg[NS];
+#pragma unroll
+    for (int s = 0; s < NS; s++) {
+        const float4 t = *reinterpret_cast<const float4*>(qrow + 8 * s + 4 * half);
+        qreg[s] = make_float4(t.x * p.scale, t.y * p.scale, t.z * p.scale, t.w * p.scale);
+    }
+    floatx16 o[NF];
+#pragma unroll
+    for (int f = 0; f < NF; f++) o[f] = zero16();
+    float m_run = kMasked, l_run = 0.0f;
+
+    int k_end = p.Sk;
+    if (p.causal && q0 + 31 + p.causal_offset + 1 < k_end) k_end = q0 + 31 + p.causal_offset + 1;
+    const int q_pos = qi + p.causal_offset;
+
+    float4 kc[NS], vc[NS];
+    auto fetch = [&](int kb) {
+        int key = kb + l32;
+        key = key < p.Sk ? key : p.Sk - 1;
+#pragma unroll
+        for (int s = 0; s < NS; s++) {
+            kc[s] = *reinterpret_cast<const float4*>(kbase + key * kst + 8 * s + 4 * half);
+            vc[s] = *reinterpret_cast<const float4*>(vbase + key * kst + 8 * s + 4 * half);
+        }
+    };
+    const int kb_first = wave * 32;
+    if (kb_first < k_end) fetch(kb_first);
+    for (int kb = kb_first; kb < k_end; kb += 32 * NSPL) {
+#pragma unroll
+        for (int s = 0; s < NS; s++)
+            *reinterpret_cast<float4*>(vt + sw_off<DP>(l32, 2 * s + half)) =
+                make_float4(vc[s].x, vc[s].y, vc[s].z, vc[s].w);
+        floatx16 s = zero16();
+#pragma unroll
+        for (int st = 0; st < NS; st++) {
+            s = MFMA(kc[st].x, qreg[st].x, s);
+            s = MFMA(kc[st].y, qreg[st].y, s);
+            s = MFMA(kc[st].z, qreg[st].z, s);
+            s = MFMA(kc[st].w, qreg[st].w, s);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        if (kb + 32 * NSPL < k_end) fetch(kb + 32 * NSPL);
+        __builtin_amdgcn_sched_barrier(0);
+        float tile_max = kMasked;
+#pragma unroll
+        for (int t = 0; t < 16; t++) {
+            const int key = kb + row_of(t, half);
+            const bool vis = q_ok && key < p.Sk && (!p.causal || key <= q_pos);
+            s[t] = vis ? s[t] : kMasked;
+            tile_max = fmaxf(tile_max, s[t]);
+        }
+        tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, 64));
+        const float m_new = fmaxf(m_run, tile_max);
+        const float corr = __expf(m_run - m_new);
+        float psum = 0.0f;
+#pragma unroll
+        for (int t = 0; t < 16; t++) {
+            const float pj = s[t] > kMasked ? __expf(s[t] - m_new) : 0.0f;
+            s[t] = pj;
+            psum += pj;
+        }
+        psum += __shfl_xor(psum, 32, 64);
+        l_run = l_run * corr + psum;
+        m_run = m_new;
+#pragma unroll
+        for (int f = 0; f < NF; f++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) o[f][r] *= corr;
+#pragma unroll
+        for (int t4 = 0; t4 < 16; t4 += 4) {
+            float av[4][NF];
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const int r = row_of(t4 + u, half);
+#pragma unroll
+                for (int f = 0; f < NF; f++) {
+                    const int d = f * 32 + l32;
+                    av[u][f] = vt[sw_off<DP>(r, d / 4) + (d & 3)];
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < 4; u++)
+#pragma unroll
+                for (int f = 0; f < NF; f++) o[f] = MFMA(av[u][f], s[t4 + u], o[f]);
+        }
+    }
+
+    // Merge the waves' (m, l, O) into wave 0, in wave order (through the private tiles).
+    constexpr int W = NF * 16 + 2;
+    if (wave > 0) {
+        float* dst = vt + lane * W;
+        dst[0] = m_run;
+        dst[1] = l_run;
+#pragma unroll
+        for (int f = 0; f < NF; f++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) dst[2 + f * 16 + r] = o[f][r];
+    }
+    __syncthreads();
+    if (wave > 0) return;
+#pragma unroll
+    for (int w = 1; w < NSPL; w++) {
+        const float* src = lds + w * PRIV + lane * W;
+        const float m_o = src[0], l_o = src[1];
+        const float m_new = fmaxf(m_run, m_o);
+        const float c0 = __expf(m_run - m_new), c1 = __expf(m_o - m_new);
+        l_run = l_run * c0 + l_o * c1;
+        m_run = m_new;
+#pragma unroll
+        for (int f = 0; f < NF; f++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) o[f][r] = o[f][r] * c0 + src[2 + f * 16 + r] * c1;
+    }
+
+    if (!q_ok) return;
+    const float inv = l_run > 0.0f ? 1.0f / l_run : 0.0f;
+    float* orow = p.o + (((long)b * p.Sq + qi) * p.H + h) * DP;
+#pragma unroll
+    for (int f = 0; f < NF; f++)
+#pragma unroll
+        for (int r4 = 0; r4 < 4; r4++) {
+            const int d = f * 32 + r4 * 8 + half * 4;
+            *reinterpret_cast<float4*>(orow + d) = make_float4(o[f][r4 * 4 + 0] * inv, o[f][r4 * 4 + 1] * inv,
+                                                               o[f][r4 * 4 + 2] * inv, o[f][r4 * 4 + 3] * inv);
+        }
+    if (p.stats && half == 0)
+        p.stats[2 * (((long)b * p.H + h) * p.Sq + qi) + 1] = l_run > 0.0f ? m_run + __logf(l_run) : kLseEmpty;
+}
+
+template <int DP>
+__global__ __launch_bounds__(kKeySplitDq * 64) void attn_bwd_dq_lds_kernel(AttnArgs p) {
+    constexpr int NF = DP / 32;
+    constexpr int NS = DP / 8;
+    constexpr int NSPL = kKeySplitDq;
+    constexpr int TILE = 32 * DP;
+    constexpr int MERGE = 64 * NF * 16;
+    constexpr int PRIV = TILE > MERGE ? TILE : MERGE;
+    __shared__ __attribute__((aligned(16))) float lds[NSPL * PRIV];
+    const int lane = threadIdx.x % 64, wave = threadIdx.x / 64, l32 = lane % 32, half = lane / 32;
+    float* kt = lds + wave * PRIV;
+    int blk_j, bh_i;
+    const int nqb_grid = (p.Sq + 31) / 32;
+    if (!attn_work_item(nqb_grid, p.B * p.H, blk_j, bh_i)) return;
+    const int b = bh_i / p.H, h = bh_i % p.H;
+    const int kvh = h / (p.H / p.Hkv);
+    const int q0 = (nqb_grid - 1 - blk_j) * 32;  // the last query block has the longest key loop: first
+    const int qi = q0 + l32;
+    const bool q_ok = qi < p.Sq;
+    const int qc = q_ok ? qi : p.Sq - 1;
+    const long qoff = (((long)b * p.Sq + qc) * p.H + h) * DP;
+    const long srow = ((long)b * p.H + h) * p.Sq + qc;
+    const long kst = (long)p.Hkv * DP;
+    const float* kbase = p.k + ((long)b * p.Sk * p.Hkv + kvh) * DP;
+    const float* vbase = p.v + ((long)b * p.Sk * p.Hkv + kvh) * DP;
+
+    float4 qreg[NS], doreg[NS];
+    float delta = 0.0f;
+#pragma unroll
+    for (int s = 0; s < NS; s++) {
+        const int d = 8 * s + 4 * half;
+        const float4 t = *reinterpret_cast<const float4*>(p.q + qoff + d);
+        qreg[s] = make_float4(t.x * p.scale, t.y * p.scale, t.z * p.scale, t.w * p.scale);
+        doreg[s] = *reinterpret_cast<const float4*>(p.d_out + qoff + d);
+        const float4 ov = *reinterpret_cast<const float4*>(p.out + qoff + d);
+        delta += doreg[s].x * ov.x + doreg[s].y * ov.y + doreg[s].z * ov.z + doreg[s].w * ov.w;
+    }
+    delta += __shfl_xor(delta, 32, 64);
+    const float lse = q_ok ? p.stats[2 * srow + 1] : kLseEmpty;
+    if (q_ok && half == 0 && wave == 0) p.stats[2 * srow] = delta;
+
+    floatx16 acc[NF];
+#pragma unroll
+    for (int f = 0; f < NF; f++) acc[f] = zero16();
+
+    int k_end = p.Sk;
+    if (p.causal && q0 + 31 + p.causal_offset + 1 < k_end) k_end = q0 + 31 + p.causal_offset + 1;
+    const int q_pos = qi + p.causal_offset;
+
+    float4 kc[NS], vc[NS];
+    auto fetch = [&](int kb) {
+        int key = kb + l32;
+        key = key < p.Sk ? key : p.Sk - 1;
+#pragma unroll
+        for (int s = 0; s < NS; s++) {
+            kc[s] = *reinterpret_cast<const float4*>(kbase + key * kst + 8 * s + 4 * half);
+            vc[s] = *reinterpret_cast<const float4*>(vbase + key * kst + 8 * s + 4 * half);
+        }
+    };
+    const int kb_first = wave * 32;
+    if (kb_first < k_end) fetch(kb_first);
+    for (int kb = kb_first; kb < k_end; kb += 32 * NSPL) {
+#pragma unroll
+        for (int s = 0; s < NS; s++) *reinterpret_cast<float4*>(kt + sw_off<DP>(l32, 2 * s + half)) = kc[s];
+        floatx16 s = zero16(), dp = zero16();
+#pragma unroll
+        for (int st = 0; st < NS; st++) {
+            s = MFMA(kc[st].x, qreg[st].x, s);
+            s = MFMA(kc[st].y, qreg[st].y, s);
+            s = MFMA(kc[st].z, qreg[st].z, s);
+            s = MFMA(kc[st].w, qreg[st].w, s);
+            dp = MFMA(vc[st].x, doreg[st].x, dp);
+            dp = MFMA(vc[st].y, doreg[st].y, dp);
+            dp = MFMA(vc[st].z, doreg[st].z, dp);
+            dp = MFMA(vc[st].w, doreg[st].w, dp);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        if (kb + 32 * NSPL < k_end) fetch(kb + 32 * NSPL);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int t = 0; t < 16; t++) {
+            const int key = kb + row_of(t, half);
+            const bool vis = q_ok && key < p.Sk && (!p.causal || key <= q_pos);
+            const float pij = vis ? __expf(s[t] - lse) : 0.0f;
+            s[t] = pij * (dp[t] - delta);
+        }
+#pragma unroll
+        for (int t4 = 0; t4 < 16; t4 += 4) {
+            float ak[4][NF];
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const int r = row_of(t4 + u, half);
+#pragma unroll
+                for (int f = 0; f < NF; f++) {
+                    const int d = f * 32 + l32;
+                    ak[u][f] = kt[sw_off<DP>(r, d / 4) + (d & 3)];
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < 4; u++)
+#pragma unroll
+                for (int f = 0; f < NF; f++) acc[f] = MFMA(ak[u][f], s[t4 + u], acc[f]);
+        }
+    }
+
+    // Sum of the waves' partial dQ, in wave order (through the private tiles).
+    constexpr int W = NF * 16;
+    if (wave > 0) {
+        float* dst = kt + lane * W;
+#pragma unroll
+        for (int f = 0; f < NF; f++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) dst[f * 16 + r] = acc[f][r];
+    }
+    __syncthreads();
+    if (wave > 0) return;
+#pragma unroll
+    for (int w = 1; w < NSPL; w++) {
+        const float* src = lds + w * PRIV + lane * W;
+#pragma unroll
+        for (int f = 0; f < NF; f++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[f][r] += src[f * 16 + r];
+    }
+
+    if (!q_ok) return;
+    float* drow = p.dq + qoff;
+#pragma unroll
+    for (int f = 0; f < NF; f++)
+#pragma unroll
+        for (int r4 = 0; r4 < 4; r4++) {
+            const int d = f * 32 + r4 * 8 + half * 4;
+            *reinterpret_cast<float4*>(drow + d) =
+                make_float4(acc[f][r4 * 4 + 0] * p.scale, acc[f][r4 * 4 + 1] * p.scale, acc[f][r4 * 4 + 2] * p.scale,
+                            acc[f][r4 * 4 + 3] * p.scale);
+        }
+}
+
 // The unguarded vector loads need whole, aligned quads in every row.
 bool attn_full(const AttnArgs& a, int DP) {
     auto al = [](const void* q) { return q == nullptr || (((uintptr_t)q) & 15) == 0; };
@@ -716,11 +1043,18 @@ bool attn_full(const AttnArgs& a, int DP) {
 
 template <int DP>
 int launch_fwd(ft_context* ctx, const AttnArgs& a) {
-    const dim3 grid(ft_div_up(a.Sq, 32), (unsigned)(a.B * a.H));
+    const dim3 grid(attn_grid(ft_div_up(a.Sq, 32), (size_t)a.B * a.H));
     // flop convention of the reference's benchmarks: causal forward 2*B*H*Sq*Sk*D, full 4*...
     const double fl = (a.causal ? 2.0 : 4.0) * a.B * a.H * (double)a.Sq * a.Sk * a.D;
     const double by = 4.0 * a.B * ((double)a.Sq * a.H * a.D * 2 + (double)a.Sk * a.Hkv * a.D * 2);
     ft_prof_scope prof(ctx, "attn_fwd_kernel", fl, by);
+    if constexpr (DP <= 64) {
+        if (attn_full(a, DP)) {
+            hipLaunchKernelGGL((attn_fwd_lds_kernel<DP>), grid, dim3(kKeySplit * 64), 0, ctx->stream, a);
+            FT_LAUNCH_CHECK();
+            return FT_OK;
+        }
+    }
     if (attn_full(a, DP))
         hipLaunchKernelGGL((attn_fwd_kernel<DP, true>), grid, dim3(kKeySplit * 64), 0, ctx->stream, a);
     else
@@ -731,21 +1065,29 @@ int launch_fwd(ft_context* ctx, const AttnArgs& a) {
 
 template <int DP>
 int launch_bwd(ft_context* ctx, const AttnArgs& a) {
-    const dim3 grid(ft_div_up(a.Sq, 32), (unsigned)(a.B * a.H));
+    const dim3 grid(attn_grid(ft_div_up(a.Sq, 32), (size_t)a.B * a.H));
     // backward = 2.5x forward by the reference's convention, charged 1.0x to the dQ pass and 1.5x to dK/dV.
     const double fl = (a.causal ? 2.0 : 4.0) * a.B * a.H * (double)a.Sq * a.Sk * a.D;
     const double by = 4.0 * a.B * ((double)a.Sq * a.H * a.D * 4 + (double)a.Sk * a.Hkv * a.D * 4);
     const bool full = attn_full(a, DP);
     {
         ft_prof_scope prof(ctx, "attn_bwd_dq_kernel", 1.0 * fl, by * 0.5);
-        if (full)
-            hipLaunchKernelGGL((attn_bwd_dq_kernel<DP, true>), grid, dim3(kKeySplit * 64), 0, ctx->stream, a);
+        bool done = false;
+        if constexpr (DP <= 64) {
+            if (full) {
+                hipLaunchKernelGGL((attn_bwd_dq_lds_kernel<DP>), grid, dim3(kKeySplitDq * 64), 0, ctx->stream, a);
+                done = true;
+            }
+        }
+        if (done) {
+        } else if (full)
+            hipLaunchKernelGGL((attn_bwd_dq_kernel<DP, true>), grid, dim3(kKeySplitDq * 64), 0, ctx->stream, a);
         else
-            hipLaunchKernelGGL((attn_bwd_dq_kernel<DP, false>), grid, dim3(kKeySplit * 64), 0, ctx->stream, a);
+            hipLaunchKernelGGL((attn_bwd_dq_kernel<DP, false>), grid, dim3(kKeySplitDq * 64), 0, ctx->stream, a);
     }
     FT_LAUNCH_CHECK();
     if constexpr (DP <= 64) {
-        if (full && a.Sk < 32 * 65535) {
+        if (full) {
             constexpr int TILE = 32 * DP, REGION = 2 * DP * 33;
             constexpr int PRIV = (2 * TILE + 64) > REGION ? (2 * TILE + 64) : REGION;
             constexpr size_t smem_lds = (size_t)(2 * TILE + 8 * PRIV) * sizeof(float);
@@ -755,7 +1097,7 @@ int launch_bwd(ft_context* ctx, const AttnArgs& a) {
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem_lds));
                 attr_lds = true;
             }
-            const dim3 grid3((unsigned)(a.B * a.Hkv), ft_div_up(a.Sk, 32));
+            const dim3 grid3(attn_grid(ft_div_up(a.Sk, 32), (size_t)a.B * a.Hkv));
             ft_prof_scope prof(ctx, "attn_bwd_dkdv_kernel", 1.5 * fl, by * 0.5);
             hipLaunchKernelGGL((attn_bwd_dkdv_lds_kernel<DP>), grid3, dim3(512), smem_lds, ctx->stream, a);
             FT_LAUNCH_CHECK();
@@ -771,7 +1113,7 @@ int launch_bwd(ft_context* ctx, const AttnArgs& a) {
                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
         attr_set = true;
     }
-    const dim3 grid2(ft_div_up(a.Sk, 32), (unsigned)(a.B * a.Hkv));
+    const dim3 grid2(attn_grid(ft_div_up(a.Sk, 32), (size_t)a.B * a.Hkv));
     {
         ft_prof_scope prof(ctx, "attn_bwd_dkdv_kernel", 1.5 * fl, by * 0.5);
         if (full)
@@ -790,7 +1132,7 @@ int check_common(const char* who, ft_context* ctx, size_t B, size_t Sq, size_t S
     FT_CHECK_ARG(Hkv > 0 && H % Hkv == 0, "%s: num_heads (%zu) must be a multiple of num_kv_heads (%zu)", who, H, Hkv);
     FT_CHECK_ARG(opts->window == 0, "%s: sliding windows are not supported", who);
     FT_CHECK_ARG(opts->dropout_prob == 0.0f, "%s: attention dropout is not supported", who);
-    FT_CHECK_ARG(B * H < 65536 && B * Hkv < 65536, "%s: batch*heads too large for the launch grid", who);
+    FT_CHECK_ARG(B * H * ((Sq + 31) / 32 + (Sk + 31) / 32) < (1u << 30), "%s: too many blocks for one launch", who);
     FT_CHECK_ARG(Sq < (1u << 24) && Sk < (1u << 24), "%s: sequence too long", who);
     return FT_OK;
 }

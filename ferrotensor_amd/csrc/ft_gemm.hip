@@ -567,8 +567,20 @@ struct AsyncProb {
     AsyncSeg seg[kAsyncMaxSeg];
     float* out;
     const float* add;  // optional [M, N] term added in the epilogue (may be `out` itself)
+    // Fused epilogues (one segment, no rank-r term):
+    //   kEpiGateUp     b_alt is a second b of the same shape; out = a@b, out2 = a@b_alt,
+    //                  out3 = silu(out2) * out            (up, gate, activation)
+    //   kEpiSiluBwd    with d = a@b (never stored), e1 = gate, e2 = up:
+    //                  out = d * e2 * silu'(e1), out2 = d * silu(e1)   (d_gate, d_up)
+    const void* b_alt;
+    float* out2;
+    float* out3;
+    const float* e1;
+    const float* e2;
     int N, ldc, tiles_n, tile_begin, nseg;
 };
+
+constexpr int kEpiPlain = 0, kEpiGateUp = 1, kEpiSiluBwd = 2;
 
 struct AsyncBatch {
     AsyncProb p[kAsyncMaxProb];
@@ -582,20 +594,22 @@ __device__ __forceinline__ T seg_pick(const T (&v)[NSEG], int s) {
     else return s == 0 ? v[0] : (s == 1 ? v[1] : v[2]);
 }
 
-template <int BM, int BN, int WM, int WN, int LAYOUT, int NSEG>
+template <int BM, int BN, int WM, int WN, int LAYOUT, int NSEG, int EPI = kEpiPlain>
 __global__ __launch_bounds__(256) void gemm_async_kernel(AsyncBatch g) {
     static_assert(LAYOUT == 0 || LAYOUT == 1, "a is k-contiguous on this path");
     static_assert(NSEG == 1 || NSEG == kAsyncMaxSeg, "one segment, or the general case");
+    static_assert(EPI == kEpiPlain || NSEG == 1, "fused epilogues take one segment");
     constexpr int NST = 3;
+    constexpr int NB = EPI == kEpiGateUp ? 2 : 1;  // b matrices multiplied against the same a tile
     constexpr int FM = WM / 32, FN = WN / 32;
     constexpr int WAVES_N = BN / WN;
     static_assert((BM / WM) * (BN / WN) == 4, "4 waves per workgroup");
     constexpr int A_FLOATS = BM * 32;             // f32 tile
     constexpr int B_FLOATS = BN * 16;             // f16 tile, in float units
-    constexpr int STAGE = A_FLOATS + B_FLOATS;
+    constexpr int STAGE = A_FLOATS + NB * B_FLOATS;
     constexpr int A_CH = BM / 8 / 4;              // 1 KiB chunks per wave
     constexpr int B_CH = BN / 16 / 4;
-    constexpr int LPT = A_CH + B_CH;              // load instructions per wave per tile
+    constexpr int LPT = A_CH + NB * B_CH;         // load instructions per wave per tile
     constexpr int WAIT = (NST - 2) * LPT;         // loads that may still be in flight when tile t is needed
     using ExA = FastTile<BM, true, 16>;
     using ExB = FastTile<BN, LAYOUT == 1, 16>;
@@ -603,8 +617,8 @@ __global__ __launch_bounds__(256) void gemm_async_kernel(AsyncBatch g) {
     __shared__ __attribute__((aligned(16))) float St0[STAGE];
     __shared__ __attribute__((aligned(16))) float St1[STAGE];
     __shared__ __attribute__((aligned(16))) float St2[STAGE];
-    __shared__ __attribute__((aligned(16))) float ExAs[ExA::LDS_FLOATS];
-    __shared__ __attribute__((aligned(16))) float ExBs[ExB::LDS_FLOATS];
+    __shared__ __attribute__((aligned(16))) float ExAs[NB == 1 ? ExA::LDS_FLOATS : 4];
+    __shared__ __attribute__((aligned(16))) float ExBs[NB == 1 ? ExB::LDS_FLOATS : 4];
 
     int pi = 0;
     if (g.count > 1 && (int)blockIdx.x >= g.p[1].tile_begin) pi = 1;
@@ -618,11 +632,11 @@ __global__ __launch_bounds__(256) void gemm_async_kernel(AsyncBatch g) {
     const int wm0 = (wave / WAVES_N) * WM, wn0 = (wave % WAVES_N) * WN;
     const int l32 = lane % 32, half = lane / 32;
 
-    floatx16 acc[FM][FN];
+    floatx16 acc[FM][FN * NB];
 #pragma unroll
     for (int i = 0; i < FM; i++)
 #pragma unroll
-        for (int j = 0; j < FN; j++)
+        for (int j = 0; j < FN * NB; j++)
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
 
@@ -639,8 +653,9 @@ __global__ __launch_bounds__(256) void gemm_async_kernel(AsyncBatch g) {
         lda_b[s] = sg.lda * 4;
         ldb_b[s] = sg.ldb * 2;
         tend[s] = (s > 0 ? tend[s - 1] : 0) + (s < p.nseg ? sg.nt : 0);
-        has_ext[s] = s < p.nseg && sg.a2 != nullptr;
+        has_ext[s] = NB == 1 && s < p.nseg && sg.a2 != nullptr;
     }
+    const char* balt = reinterpret_cast<const char*>(p.b_alt);
     const int nt = tend[NSEG - 1];
 
     // The rank-r products' operands: ordinary loads, issued first, consumed last.
@@ -721,13 +736,18 @@ __global__ __launch_bounds__(256) void gemm_async_kernel(AsyncBatch g) {
         for (int j = 0; j < A_CH; j++) glds16(at, offA[j], st + (wave + 4 * j) * 256);
 #pragma unroll
         for (int j = 0; j < B_CH; j++) glds16(bt, offB[j], st + A_FLOATS + (wave + 4 * j) * 256);
+        if constexpr (NB == 2) {
+            const char* bt2 = balt + (long)tl * b_step;
+#pragma unroll
+            for (int j = 0; j < B_CH; j++) glds16(bt2, offB[j], st + A_FLOATS + B_FLOATS + (wave + 4 * j) * 256);
+        }
     };
     auto a_frag = [&](const float* st, int s, int row) -> float4 {
         const int kq = 2 * s + half;
         return *reinterpret_cast<const float4*>(st + row * 32 + ((kq ^ (row & 7)) * 4));
     };
-    auto b_frag = [&](const float* st, int s, int n) -> float4 {
-        const char* bs = reinterpret_cast<const char*>(st + A_FLOATS);
+    auto b_frag = [&](const float* st, int s, int n, int jb) -> float4 {
+        const char* bs = reinterpret_cast<const char*>(st + A_FLOATS + jb * B_FLOATS);
         if constexpr (LAYOUT == 1) {
             const int kq = 2 * s + half;
             const int col = (kq >> 1) ^ ((n >> 1) & 3);
@@ -738,11 +758,11 @@ __global__ __launch_bounds__(256) void gemm_async_kernel(AsyncBatch g) {
             return make_float4((float)q[0], (float)q[BN], (float)q[2 * BN], (float)q[3 * BN]);
         }
     };
-    auto mfma_step = [&](const float4 (&af)[FM], const float4 (&bf)[FN]) {
+    auto mfma_step = [&](const float4 (&af)[FM], const float4 (&bf)[FN * NB]) {
 #pragma unroll
         for (int i = 0; i < FM; i++)
 #pragma unroll
-            for (int j = 0; j < FN; j++) {
+            for (int j = 0; j < FN * NB; j++) {
                 acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i].x, bf[j].x, acc[i][j], 0, 0, 0);
                 acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i].y, bf[j].y, acc[i][j], 0, 0, 0);
                 acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i].z, bf[j].z, acc[i][j], 0, 0, 0);
@@ -757,11 +777,11 @@ __global__ __launch_bounds__(256) void gemm_async_kernel(AsyncBatch g) {
         __builtin_amdgcn_sched_barrier(0);
         issue(t + NST - 1, refill);
         __builtin_amdgcn_sched_barrier(0);
-        float4 af[2][FM], bf[2][FN];
+        float4 af[2][FM], bf[2][FN * NB];
 #pragma unroll
         for (int i = 0; i < FM; i++) af[0][i] = a_frag(cur, 0, wm0 + i * 32 + l32);
 #pragma unroll
-        for (int j = 0; j < FN; j++) bf[0][j] = b_frag(cur, 0, wn0 + j * 32 + l32);
+        for (int j = 0; j < FN * NB; j++) bf[0][j] = b_frag(cur, 0, wn0 + (j % FN) * 32 + l32, j / FN);
 #pragma unroll
         for (int s = 0; s < 4; s++) {
             const int c = s & 1, nx = c ^ 1;
@@ -769,7 +789,8 @@ __global__ __launch_bounds__(256) void gemm_async_kernel(AsyncBatch g) {
 #pragma unroll
                 for (int i = 0; i < FM; i++) af[nx][i] = a_frag(cur, s + 1, wm0 + i * 32 + l32);
 #pragma unroll
-                for (int j = 0; j < FN; j++) bf[nx][j] = b_frag(cur, s + 1, wn0 + j * 32 + l32);
+                for (int j = 0; j < FN * NB; j++)
+                    bf[nx][j] = b_frag(cur, s + 1, wn0 + (j % FN) * 32 + l32, j / FN);
             }
             __builtin_amdgcn_sched_barrier(0);
             mfma_step(af[c], bf[c]);
@@ -789,7 +810,7 @@ __global__ __launch_bounds__(256) void gemm_async_kernel(AsyncBatch g) {
     bool ext_used = false;
 #pragma unroll
     for (int s = 0; s < NSEG; s++) {
-        if (has_ext[s]) {
+        if (has_ext[s]) {  // never with two b matrices
             if (ext_used) __syncthreads();  // the previous segment's tile is still being read
             ext_used = true;
             xa[s].template store<float>(ExAs);
@@ -797,11 +818,11 @@ __global__ __launch_bounds__(256) void gemm_async_kernel(AsyncBatch g) {
             __syncthreads();
 #pragma unroll
             for (int st = 0; st < 2; st++) {
-                float4 af[FM], bf[FN];
+                float4 af[FM], bf[FN * NB];
 #pragma unroll
                 for (int i = 0; i < FM; i++) af[i] = ExA::frag(ExAs, st, half, wm0 + i * 32 + l32);
 #pragma unroll
-                for (int j = 0; j < FN; j++) bf[j] = ExB::frag(ExBs, st, half, wn0 + j * 32 + l32);
+                for (int j = 0; j < FN * NB; j++) bf[j] = ExB::frag(ExBs, st, half, wn0 + (j % FN) * 32 + l32);
                 mfma_step(af, bf);
             }
         }
@@ -820,7 +841,19 @@ __global__ __launch_bounds__(256) void gemm_async_kernel(AsyncBatch g) {
                 const int row = m0 + wm0 + i * 32 + (r / 4) * 8 + half * 4 + (r % 4);
                 if (row < M) {
                     const long o = (long)row * p.ldc + col;
-                    p.out[o] = p.add ? acc[i][j][r] + p.add[o] : acc[i][j][r];
+                    if constexpr (EPI == kEpiGateUp) {
+                        const float up = acc[i][j][r], x = acc[i][FN + j][r];
+                        p.out[o] = up;
+                        p.out2[o] = x;
+                        p.out3[o] = x * (1.0f / (1.0f + __expf(-x))) * up;
+                    } else if constexpr (EPI == kEpiSiluBwd) {
+                        const float d = acc[i][j][r], x = p.e1[o], y = p.e2[o];
+                        const float sg = 1.0f / (1.0f + __expf(-x));
+                        p.out2[o] = d * (x * sg);
+                        p.out[o] = d * y * (sg * (1.0f + x * (1.0f - sg)));
+                    } else {
+                        p.out[o] = p.add ? acc[i][j][r] + p.add[o] : acc[i][j][r];
+                    }
                 }
             }
         }
@@ -935,7 +968,7 @@ __global__ __launch_bounds__(256) void skinny_kernel(const float* __restrict__ x
 // ---------------------------------------------------------------------------
 
 template <int BM, int BN, int WM, int WN>
-int launch_async(ft_context* ctx, AsyncBatch g, int layout) {
+int launch_async(ft_context* ctx, AsyncBatch g, int layout, int epi = kEpiPlain) {
     const int tiles_m = (g.M + BM - 1) / BM;
     int tiles = 0, max_seg = 1;
     double flops = 0.0, bytes = 0.0;
@@ -954,6 +987,27 @@ int launch_async(ft_context* ctx, AsyncBatch g, int layout) {
     }
     const dim3 grid((unsigned)tiles);
     char name[96];
+    if (epi != kEpiPlain) {
+        // both fused forms: one product, one segment, 64x64 tiles (the only instantiation)
+        if constexpr (BM == 64) {
+            const bool gu = epi == kEpiGateUp;
+            snprintf(name, sizeof(name), "gemm_async_kernel<64, 64, 32, 32, %d, 1, %s>", layout,
+                     gu ? "gate_up" : "silu_bwd");
+            const double mn = (double)g.M * g.p[0].N;
+            ft_prof_scope prof(ctx, name, gu ? 2.0 * flops : flops,
+                               gu ? bytes + 64.0 * g.p[0].N * g.p[0].seg[0].nt + 8.0 * mn : bytes + 12.0 * mn);
+            if (gu)
+                hipLaunchKernelGGL((gemm_async_kernel<64, 64, 32, 32, 0, 1, kEpiGateUp>), grid, dim3(256), 0,
+                                   ctx->stream, g);
+            else
+                hipLaunchKernelGGL((gemm_async_kernel<64, 64, 32, 32, 1, 1, kEpiSiluBwd>), grid, dim3(256), 0,
+                                   ctx->stream, g);
+            FT_LAUNCH_CHECK();
+            return FT_OK;
+        } else {
+            return ft_set_error(FT_ERR_INVALID, "fused epilogues use 64x64 tiles");
+        }
+    }
     snprintf(name, sizeof(name), "gemm_async_kernel<%d, %d, %d, %d, %d, %d>", BM, BN, WM, WN, layout,
              max_seg > 1 ? kAsyncMaxSeg : 1);
     ft_prof_scope prof(ctx, name, flops, bytes);
@@ -1251,6 +1305,60 @@ int ft_lora_linear_dx_group(ft_context* ctx, const ft_lora_dx_desc* linears, siz
                                  i == 0 ? residual : dx, dx, M, K, d.N, d.r));
     }
     return FT_OK;
+}
+
+int ft_mlp_gate_up(ft_context* ctx, const float* x, const void* w_gate, const void* w_up, int w_dtype, float* gate,
+                   float* up, float* act, size_t M, size_t K, size_t N) {
+    FT_CHECK_ARG(ctx && x && w_gate && w_up && gate && up && act, "ft_mlp_gate_up: NULL argument");
+    FT_CHECK_ARG(w_dtype == FT_DTYPE_F32 || w_dtype == FT_DTYPE_F16, "ft_mlp_gate_up: dtype %d", w_dtype);
+    if (M == 0 || N == 0) return FT_OK;
+    const bool fused = w_dtype == FT_DTYPE_F16 && M < (1u << 30) && K < (1u << 30) && N < (1u << 30) &&
+                       async_eligible(0, x, w_up, up, nullptr, M, K, N, nullptr, nullptr, 0) &&
+                       async_eligible(0, x, w_gate, gate, nullptr, M, K, N, nullptr, nullptr, 0) && aligned16p(act);
+    if (fused) {
+        AsyncBatch g{};
+        g.count = 1;
+        g.M = (int)M;
+        g.p[0].seg[0] = make_seg(0, x, w_up, K, N, nullptr, nullptr, 0);
+        g.p[0].nseg = 1;
+        g.p[0].b_alt = w_gate;
+        g.p[0].out = up;
+        g.p[0].out2 = gate;
+        g.p[0].out3 = act;
+        g.p[0].N = (int)N;
+        g.p[0].ldc = (int)N;
+        return launch_async<64, 64, 32, 32>(ctx, g, 0, kEpiGateUp);
+    }
+    FT_TRY(ft_lora_linear(ctx, x, w_up, w_dtype, nullptr, nullptr, nullptr, up, M, K, N, 0));
+    FT_TRY(ft_lora_linear(ctx, x, w_gate, w_dtype, nullptr, nullptr, nullptr, gate, M, K, N, 0));
+    return ft_silu_gate_fused(ctx, gate, up, act, M * N);
+}
+
+int ft_mlp_down_backward(ft_context* ctx, const float* dy, const void* w_down, int w_dtype, const float* gate,
+                         const float* up, float* d_gate, float* d_up, float* scratch, size_t M, size_t F, size_t H) {
+    FT_CHECK_ARG(ctx && dy && w_down && gate && up && d_gate && d_up, "ft_mlp_down_backward: NULL argument");
+    FT_CHECK_ARG(w_dtype == FT_DTYPE_F32 || w_dtype == FT_DTYPE_F16, "ft_mlp_down_backward: dtype %d", w_dtype);
+    if (M == 0 || F == 0) return FT_OK;
+    // d_act[M,F] = dy[M,H] @ w_down[F,H]^T: layout 1 with output width F, reduction H.
+    const bool fused = w_dtype == FT_DTYPE_F16 && M < (1u << 30) && F < (1u << 30) && H < (1u << 30) &&
+                       async_eligible(1, dy, w_down, d_gate, nullptr, M, H, F, nullptr, nullptr, 0);
+    if (fused) {
+        AsyncBatch g{};
+        g.count = 1;
+        g.M = (int)M;
+        g.p[0].seg[0] = make_seg(1, dy, w_down, H, F, nullptr, nullptr, 0);
+        g.p[0].nseg = 1;
+        g.p[0].out = d_gate;
+        g.p[0].out2 = d_up;
+        g.p[0].e1 = gate;
+        g.p[0].e2 = up;
+        g.p[0].N = (int)F;
+        g.p[0].ldc = (int)F;
+        return launch_async<64, 64, 32, 32>(ctx, g, 1, kEpiSiluBwd);
+    }
+    FT_CHECK_ARG(scratch, "ft_mlp_down_backward: this operand combination needs the [M,F] scratch buffer");
+    FT_TRY(ft_lora_linear_dx(ctx, dy, w_down, w_dtype, nullptr, nullptr, nullptr, scratch, M, F, H, 0));
+    return ft_silu_gate_backward(ctx, gate, up, scratch, d_gate, d_up, M * F);
 }
 
 int ft_lora_grad_b(ft_context* ctx, const float* t, const float* dy, float* db, size_t M, size_t N, size_t r) {

@@ -412,13 +412,15 @@ int model_forward(ft_model* m, const uint32_t* rows_host, size_t B, size_t S) {
             float* ts[2] = {a.tup, a.tgate};
             FT_TRY(lora_down_group(ctx, ls, ts, 2, a.h2, T));
         }
-        {
+        if (!L.up.has_lora() && !L.gate.has_lora() && L.up.dtype == L.gate.dtype) {
+            FT_TRY(ft_mlp_gate_up(ctx, a.h2, L.gate.w, L.up.w, L.up.dtype, a.gate, a.up, a.act, T, H, F));
+        } else {
             LinearW* ls[2] = {&L.up, &L.gate};
             const float* ts[2] = {a.tup, a.tgate};
             float* ys[2] = {a.up, a.gate};
             FT_TRY(linear_gemm_group(ctx, ls, ts, ys, 2, a.h2, T));
+            FT_TRY(ft_silu_gate_fused(ctx, a.gate, a.up, a.act, T * F));
         }
-        FT_TRY(ft_silu_gate_fused(ctx, a.gate, a.up, a.act, T * F));
         FT_TRY(linear_forward(ctx, L.down, a.act, a.tdown, x_next, T, a.h));
     }
     FT_TRY(ft_rms_norm_eps(ctx, m->x_final, m->norm_f, m->hf, T, H, c.rms_norm_eps));
@@ -443,8 +445,13 @@ int model_backward(ft_model* m, size_t B, size_t S, bool accumulate) {
         Layer& L = m->layers[li];
         LayerActs& a = m->acts[li];
         // x_next = h + down(silu(gate) * up)
-        FT_TRY(linear_backward(m, L.down, a.act, a.tdown, g, m->d_act, T, accumulate));
-        FT_TRY(ft_silu_gate_backward(ctx, a.gate, a.up, m->d_act, m->d_gate, m->d_up, T * F));
+        if (!L.down.has_lora()) {
+            FT_TRY(ft_mlp_down_backward(ctx, g, L.down.w, L.down.dtype, a.gate, a.up, m->d_gate, m->d_up, m->d_act, T,
+                                        F, H));
+        } else {
+            FT_TRY(linear_backward(m, L.down, a.act, a.tdown, g, m->d_act, T, accumulate));
+            FT_TRY(ft_silu_gate_backward(ctx, a.gate, a.up, m->d_act, m->d_gate, m->d_up, T * F));
+        }
         {
             LinearW* ls[2] = {&L.up, &L.gate};
             const float* ts[2] = {a.tup, a.tgate};

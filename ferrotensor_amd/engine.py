@@ -324,6 +324,23 @@ class ComputeEngine:
         assert dx.numel() == M * K
         check(self._lib.ft_lora_linear_dx_group(ctx.handle, descs, len(linears), _p(residual), _p(dx), M, K))
 
+    def mlp_gate_up(self, ctx, x, w_gate, w_up, gate, up, act):
+        """gate = x@w_gate, up = x@w_up, act = silu(gate) * up in one launch."""
+        M, K = x.shape
+        K2, N = w_up.shape
+        assert K == K2 and list(w_gate.shape) == [K, N] and w_gate.dtype == w_up.dtype
+        assert gate.numel() == up.numel() == act.numel() == M * N
+        check(self._lib.ft_mlp_gate_up(ctx.handle, _p(x), _p(w_gate), _p(w_up), w_up.dtype, _p(gate), _p(up), _p(act),
+                                       M, K, N))
+
+    def mlp_down_backward(self, ctx, dy, w_down, gate, up, d_gate, d_up, scratch=None):
+        """d_gate, d_up from dy through the down projection and the gated activation, in one launch."""
+        M, H = dy.shape
+        F, H2 = w_down.shape
+        assert H == H2 and gate.numel() == up.numel() == d_gate.numel() == d_up.numel() == M * F
+        check(self._lib.ft_mlp_down_backward(ctx.handle, _p(dy), _p(w_down), w_down.dtype, _p(gate), _p(up),
+                                             _p(d_gate), _p(d_up), _p(scratch), M, F, H))
+
     def lora_grad_down(self, ctx, dy, b, dt, scale):
         M, N = dy.shape
         r, N2 = b.shape

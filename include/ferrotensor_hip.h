@@ -167,6 +167,24 @@ typedef struct ft_lora_dx_desc {
 int ft_lora_linear_dx_group(ft_context* ctx, const ft_lora_dx_desc* linears, size_t count, const float* residual,
                             float* dx, size_t M, size_t K);
 
+/* The gated-MLP front half in ONE launch (Lfm2Model's feed-forward,
+ * ferrotensor-graph/src/lib.rs:312-330: two project_2d calls and silu_gate_fused):
+ * gate[M,N] = x @ w_gate, up[M,N] = x @ w_up, act = silu(gate) * up. Each
+ * workgroup multiplies one x tile against the matching tiles of both weights
+ * and applies the activation in the epilogue; gate and up are still written
+ * (the backward pass reads them). Frozen weights only (no rank-r term). */
+int ft_mlp_gate_up(ft_context* ctx, const float* x, const void* w_gate, const void* w_up, int w_dtype,
+                   float* gate, float* up, float* act, size_t M, size_t K, size_t N);
+/* The gated-MLP back half in ONE launch: with d_act[M,F] = dy[M,H] @ w_down[F,H]^T
+ * (MatMulNode::backward of the down projection) never stored, the epilogue applies
+ * SiluGateNode::backward (engine/elementwise.rs:194-216):
+ * d_gate = d_act * up * silu'(gate), d_up = d_act * silu(gate). `scratch` ([M,F]
+ * floats, may be NULL) is only used when the operands rule out the fused kernel
+ * (f32 weights, unaligned buffers). */
+int ft_mlp_down_backward(ft_context* ctx, const float* dy, const void* w_down, int w_dtype,
+                         const float* gate, const float* up, float* d_gate, float* d_up, float* scratch,
+                         size_t M, size_t F, size_t H);
+
 /* t[M,r] = scale * (x[M,K] @ a[K,r]): the `x @ A` product with the alpha/rank
  * scale applied where the reference applies it (graph/src/lib.rs:116-122).
  * r <= 32. */

@@ -191,6 +191,34 @@ def test_grouped_linears_match_single_calls(g, M, K, Ns, r, f16):
     assert_close("group dx + residual", dx2.to_numpy(), want_dx + res, atol=3e-3, rtol=1e-4)
 
 
+@pytest.mark.parametrize("M,H,F,f16", [(256, 960, 2560, True), (100, 64, 96, True), (70, 32, 40, True),
+                                       (64, 32, 48, False)])
+def test_fused_gated_mlp_halves(g, M, H, F, f16):
+    """gate/up projections + silu_gate in one launch; down-projection backward + silu_gate backward in one."""
+    from ferrotensor_amd import UnifiedTensor
+    ctx, eng = g
+    x = rnd(1, M, H)
+    wg, wu, wd = rnd(2, H, F, scale=0.1), rnd(3, H, F, scale=0.1), rnd(4, F, H, scale=0.1)
+    rd = (lambda w: cpu.round_f16(w)) if f16 else (lambda w: w)
+    mk = (lambda w: UnifiedTensor.from_f32_as_f16(ctx, w, list(w.shape))) if f16 else (lambda w: up(ctx, w))
+    want_gate, want_up = cpu.matmul(x, rd(wg)), cpu.matmul(x, rd(wu))
+    want_act = cpu.silu_gate(want_gate, want_up)
+    gate, upt, act = empty(ctx, M, F), empty(ctx, M, F), empty(ctx, M, F)
+    eng.mlp_gate_up(ctx, up(ctx, x), mk(wg), mk(wu), gate, upt, act)
+    assert_close("gate", gate.to_numpy(), want_gate, atol=1e-3, rtol=1e-4)
+    assert_close("up", upt.to_numpy(), want_up, atol=1e-3, rtol=1e-4)
+    assert_close("act", act.to_numpy(), want_act, atol=1e-3, rtol=1e-3)
+
+    dy = rnd(5, M, H)
+    gate_in, up_in = rnd(6, M, F), rnd(7, M, F)
+    d_act = cpu.matmul(dy, np.ascontiguousarray(rd(wd).T))
+    want_dg, want_du = cpu.silu_gate_backward(gate_in, up_in, d_act)
+    d_gate, d_up, scratch = empty(ctx, M, F), empty(ctx, M, F), empty(ctx, M, F)
+    eng.mlp_down_backward(ctx, up(ctx, dy), mk(wd), up(ctx, gate_in), up(ctx, up_in), d_gate, d_up, scratch)
+    assert_close("d_gate", d_gate.to_numpy(), want_dg, atol=2e-3, rtol=1e-3)
+    assert_close("d_up", d_up.to_numpy(), want_du, atol=2e-3, rtol=1e-3)
+
+
 @pytest.mark.parametrize("rows,size", [(1, 1), (3, 7), (37, 96), (16, 576), (64, 960), (5, 2048), (3, 2100)])
 def test_rms_norm_forward_backward(g, rows, size):
     ctx, eng = g
