@@ -28,6 +28,15 @@ struct ft_context {
     // Partial sums of the sliced thin products (LoRA dA, dB); allocated on first use.
     float* thin_scratch = nullptr;
 
+    // A second stream for work that is off the critical path of a training step
+    // (the LoRA factor gradients, which only the optimizer reads): ft_side_begin
+    // makes it wait for everything enqueued so far and redirects launches to it,
+    // ft_side_end switches back, ft_side_join makes the main stream wait for it.
+    hipStream_t side_stream = nullptr;
+    hipStream_t main_stream = nullptr;  // saved while launches are redirected
+    hipEvent_t fork_event = nullptr, join_event = nullptr;
+    bool side_active = false, side_pending = false;
+
     // Per-kernel timing with HIP events on the context's stream (off by default).
     struct ProfRecord {
         int key;
@@ -56,6 +65,10 @@ struct ft_prof_scope {
 };
 
 int ft_set_error(int code, const char* fmt, ...);
+
+int ft_side_begin(ft_context* ctx);
+int ft_side_end(ft_context* ctx);
+int ft_side_join(ft_context* ctx);
 
 #define FT_CHECK_ARG(cond, ...)                                  \
     do {                                                         \

@@ -47,8 +47,43 @@ ft_prof_scope::~ft_prof_scope() {
     if (index >= 0) (void)hipEventRecord(ctx->prof_records[index].e1, ctx->stream);
 }
 
+int ft_side_begin(ft_context* ctx) {
+    FT_CHECK_ARG(ctx && !ctx->side_active, "ft_side_begin: already redirected");
+    if (!ctx->side_stream) {
+        FT_HIP(hipSetDevice(ctx->device));
+        FT_HIP(hipStreamCreateWithFlags(&ctx->side_stream, hipStreamNonBlocking));
+        FT_HIP(hipEventCreateWithFlags(&ctx->fork_event, hipEventDisableTiming));
+        FT_HIP(hipEventCreateWithFlags(&ctx->join_event, hipEventDisableTiming));
+    }
+    FT_HIP(hipEventRecord(ctx->fork_event, ctx->stream));
+    FT_HIP(hipStreamWaitEvent(ctx->side_stream, ctx->fork_event, 0));
+    ctx->main_stream = ctx->stream;
+    ctx->stream = ctx->side_stream;
+    ctx->side_active = true;
+    return FT_OK;
+}
+
+int ft_side_end(ft_context* ctx) {
+    FT_CHECK_ARG(ctx && ctx->side_active, "ft_side_end: not redirected");
+    const hipError_t e = hipEventRecord(ctx->join_event, ctx->side_stream);
+    ctx->stream = ctx->main_stream;
+    ctx->side_active = false;
+    ctx->side_pending = true;
+    FT_HIP(e);
+    return FT_OK;
+}
+
+int ft_side_join(ft_context* ctx) {
+    FT_CHECK_ARG(ctx && !ctx->side_active, "ft_side_join: still redirected");
+    if (!ctx->side_pending) return FT_OK;
+    ctx->side_pending = false;
+    FT_HIP(hipStreamWaitEvent(ctx->stream, ctx->join_event, 0));
+    return FT_OK;
+}
+
 // Waits for the stream and folds the finished records into the totals.
 static int prof_collect(ft_context* ctx) {
+    FT_TRY(ft_side_join(ctx));
     FT_HIP(hipStreamSynchronize(ctx->stream));
     for (auto& r : ctx->prof_records) {
         float ms = 0.0f;
@@ -156,6 +191,12 @@ int ft_context_destroy(ft_context* ctx) {
         (void)hipEventDestroy(r.e1);
     }
     for (hipEvent_t e : ctx->prof_event_pool) (void)hipEventDestroy(e);
+    if (ctx->side_stream) {
+        (void)hipStreamSynchronize(ctx->side_stream);
+        (void)hipEventDestroy(ctx->fork_event);
+        (void)hipEventDestroy(ctx->join_event);
+        (void)hipStreamDestroy(ctx->side_stream);
+    }
     if (ctx->thin_scratch) (void)hipFree(ctx->thin_scratch);
     if (ctx->owns_stream) (void)hipStreamDestroy(ctx->stream);
     delete ctx;
@@ -164,6 +205,7 @@ int ft_context_destroy(ft_context* ctx) {
 
 int ft_synchronize(ft_context* ctx) {
     FT_CHECK_ARG(ctx, "ft_synchronize: ctx is NULL");
+    FT_TRY(ft_side_join(ctx));
     FT_HIP(hipStreamSynchronize(ctx->stream));
     return FT_OK;
 }
@@ -240,6 +282,7 @@ int ft_upload(ft_context* ctx, void* dst_dev, const void* src_host, size_t bytes
 int ft_download(ft_context* ctx, void* dst_host, const void* src_dev, size_t bytes) {
     FT_CHECK_ARG(ctx && (bytes == 0 || (dst_host && src_dev)), "ft_download: NULL argument");
     if (bytes == 0) return FT_OK;
+    FT_TRY(ft_side_join(ctx));
     FT_HIP(hipMemcpyAsync(dst_host, src_dev, bytes, hipMemcpyDeviceToHost, ctx->stream));
     FT_HIP(hipStreamSynchronize(ctx->stream));
     return FT_OK;

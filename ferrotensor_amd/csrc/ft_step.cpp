@@ -284,6 +284,7 @@ int linear_backward(ft_model* m, LinearW& l, const float* x, const float* t, con
                     bool accumulate, bool dx_add = false) {
     ft_context* ctx = m->ctx;
     if (l.has_lora()) {
+        FT_TRY(ft_side_join(ctx));  // factor gradients still in flight read m->dt
         FT_TRY(ft_lora_grad_down(ctx, dy, l.b, m->dt, T, l.out, l.r, l.scale()));
         if (accumulate) {
             FT_TRY(ft_lora_grad_b(ctx, t, dy, m->gtmp, T, l.out, l.r));
@@ -296,7 +297,11 @@ int linear_backward(ft_model* m, LinearW& l, const float* x, const float* t, con
                 {dy, t, l.gb, (int)T, 0, (int)l.out, (int)l.r, (long)l.out, (long)l.r, (long)l.out, 1.0f, 0, 1, 0},
                 {x, m->dt, l.ga, (int)T, 0, (int)l.in, (int)l.r, (long)l.in, (long)l.r, (long)l.r, 1.0f, 0, 0, 0}};
             if (ft_thin_colwise_ok(pb[0]) && ft_thin_colwise_ok(pb[1])) {
-                FT_TRY(ft_thin_colwise(ctx, pb, 2));
+                // Only the optimizer reads dA and dB: they run beside the input-gradient GEMM.
+                FT_TRY(ft_side_begin(ctx));
+                const int rc = ft_thin_colwise(ctx, pb, 2);
+                FT_TRY(ft_side_end(ctx));
+                FT_TRY(rc);
             } else {
                 FT_TRY(ft_lora_grad_b(ctx, t, dy, l.gb, T, l.out, l.r));
                 FT_TRY(ft_lora_grad_a(ctx, x, m->dt, l.ga, T, l.in, l.r));
@@ -351,8 +356,14 @@ int linear_backward_group(ft_model* m, LinearW* const* ls, const float* const* t
         for (int i = 0; i < n; i++) d[i] = ft_lora_dx_desc{dys[i], ls[i]->w, ls[i]->dtype, nullptr, nullptr, ls[i]->out, 0};
         return ft_lora_linear_dx_group(ctx, d, (size_t)n, nullptr, dx, T, ls[0]->in);
     }
+    FT_TRY(ft_side_join(ctx));  // factor gradients still in flight read the dt buffers
     FT_TRY(ft_thin_rowwise(ctx, rows, n));
-    FT_TRY(ft_thin_colwise(ctx, cols, 2 * n));
+    {
+        FT_TRY(ft_side_begin(ctx));
+        const int rc = ft_thin_colwise(ctx, cols, 2 * n);
+        FT_TRY(ft_side_end(ctx));
+        FT_TRY(rc);
+    }
     if (dx) {
         ft_lora_dx_desc d[3];
         for (int i = 0; i < n; i++)
@@ -485,7 +496,7 @@ int model_backward(ft_model* m, size_t B, size_t S, bool accumulate) {
         // g = g_h + norm1_backward(d_h1)
         FT_TRY(ft_internal_rms_norm_backward_add(ctx, a.x, L.norm1, m->d_h1, g_other, g, T, H, c.rms_norm_eps));
     }
-    return FT_OK;
+    return ft_side_join(ctx);
 }
 
 LinearW* find_linear(ft_model* m, const std::string& prefix) {

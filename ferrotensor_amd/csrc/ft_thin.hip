@@ -230,6 +230,8 @@ int ft_thin_rowwise(ft_context* ctx, const ft_thin_problem* probs, int count) {
 int ft_thin_colwise(ft_context* ctx, const ft_thin_problem* probs, int count) {
     FT_CHECK_ARG(ctx && probs && count >= 1 && count <= FT_THIN_MAX_BATCH, "thin colwise: bad batch");
     FT_TRY(ensure_scratch(ctx));
+    // The partial-sum buffer is shared: a call on the main stream must not overtake one on the side stream.
+    if (!ctx->side_active) FT_TRY(ft_side_join(ctx));
     ThinBatch b{};
     b.count = count;
     int rmax = 0, mmax = 0;
