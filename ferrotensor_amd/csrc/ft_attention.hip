@@ -646,18 +646,21 @@ __global__ __launch_bounds__(512) void attn_bwd_dkdv_lds_kernel(AttnArgs p) {
 
     for (int item = wave; item < items; item += NWV) {
         const int q0 = (qb_start + item % per_head) * 32;
+        // LDS addresses are formed from this per item (not kept in registers across the loop)
+        int lq = l32;
+        asm volatile("" : "+v"(lq));
         // this item's tiles -> private LDS (for the transposed reads), S and dP from the registers
 #pragma unroll
         for (int s = 0; s < NS; s++) {
-            *reinterpret_cast<float4*>(qs + sw_off<DP>(l32, 2 * s + half)) = qa[s];
-            *reinterpret_cast<float4*>(dos + sw_off<DP>(l32, 2 * s + half)) = qc[s];
+            *reinterpret_cast<float4*>(qs + sw_off<DP>(lq, 2 * s + half)) = qa[s];
+            *reinterpret_cast<float4*>(dos + sw_off<DP>(lq, 2 * s + half)) = qc[s];
         }
-        if (half == 0) *reinterpret_cast<float2*>(sts + 2 * l32) = st_mine;
+        if (half == 0) *reinterpret_cast<float2*>(sts + 2 * lq) = st_mine;
         floatx16 s = zero16(), dp = zero16();
 #pragma unroll
         for (int st = 0; st < NS; st++) {
-            const float4 kq = *reinterpret_cast<const float4*>(ks + sw_off<DP>(l32, 2 * st + half));
-            const float4 vq = *reinterpret_cast<const float4*>(vs + sw_off<DP>(l32, 2 * st + half));
+            const float4 kq = *reinterpret_cast<const float4*>(ks + sw_off<DP>(lq, 2 * st + half));
+            const float4 vq = *reinterpret_cast<const float4*>(vs + sw_off<DP>(lq, 2 * st + half));
             s = MFMA(qa[st].x, kq.x, s);
             s = MFMA(qa[st].y, kq.y, s);
             s = MFMA(qa[st].z, kq.z, s);
@@ -691,7 +694,7 @@ __global__ __launch_bounds__(512) void attn_bwd_dkdv_lds_kernel(AttnArgs p) {
                 const int r = row_of(t4 + u, half);
 #pragma unroll
                 for (int f = 0; f < NF; f++) {
-                    const int d = f * 32 + l32;
+                    const int d = f * 32 + lq;
                     ao[u][f] = dos[sw_off<DP>(r, d / 4) + (d & 3)];
                     aq[u][f] = qs[sw_off<DP>(r, d / 4) + (d & 3)];
                 }

@@ -28,14 +28,18 @@ struct ft_context {
     // Partial sums of the sliced thin products (LoRA dA, dB); allocated on first use.
     float* thin_scratch = nullptr;
 
-    // A second stream for work that is off the critical path of a training step
-    // (the LoRA factor gradients, which only the optimizer reads): ft_side_begin
-    // makes it wait for everything enqueued so far and redirects launches to it,
-    // ft_side_end switches back, ft_side_join makes the main stream wait for it.
-    hipStream_t side_stream = nullptr;
+    // Extra streams ("lanes") for work that can run beside the main stream:
+    // lane 0 carries the LoRA factor gradients of a training step (only the
+    // optimizer reads them), lane 1 one of the two attention backward kernels.
+    // ft_side_begin makes a lane wait for everything enqueued on the main stream
+    // so far and redirects launches to it, ft_side_end switches back,
+    // ft_side_join makes the main stream wait for one lane or for all of them.
+    static constexpr int kLanes = 2;
+    hipStream_t side_stream[kLanes] = {nullptr, nullptr};
+    hipEvent_t fork_event[kLanes] = {nullptr, nullptr}, join_event[kLanes] = {nullptr, nullptr};
+    bool side_pending[kLanes] = {false, false};
     hipStream_t main_stream = nullptr;  // saved while launches are redirected
-    hipEvent_t fork_event = nullptr, join_event = nullptr;
-    bool side_active = false, side_pending = false;
+    int side_active = -1;               // lane that launches are redirected to, or -1
 
     // Per-kernel timing with HIP events on the context's stream (off by default).
     struct ProfRecord {
@@ -66,9 +70,9 @@ struct ft_prof_scope {
 
 int ft_set_error(int code, const char* fmt, ...);
 
-int ft_side_begin(ft_context* ctx);
+int ft_side_begin(ft_context* ctx, int lane = 0);
 int ft_side_end(ft_context* ctx);
-int ft_side_join(ft_context* ctx);
+int ft_side_join(ft_context* ctx, int lane = -1);  // -1: every lane
 
 #define FT_CHECK_ARG(cond, ...)                                  \
     do {                                                         \

@@ -284,7 +284,7 @@ int linear_backward(ft_model* m, LinearW& l, const float* x, const float* t, con
                     bool accumulate, bool dx_add = false) {
     ft_context* ctx = m->ctx;
     if (l.has_lora()) {
-        FT_TRY(ft_side_join(ctx));  // factor gradients still in flight read m->dt
+        FT_TRY(ft_side_join(ctx, 0));  // factor gradients still in flight read m->dt
         FT_TRY(ft_lora_grad_down(ctx, dy, l.b, m->dt, T, l.out, l.r, l.scale()));
         if (accumulate) {
             FT_TRY(ft_lora_grad_b(ctx, t, dy, m->gtmp, T, l.out, l.r));
@@ -356,7 +356,7 @@ int linear_backward_group(ft_model* m, LinearW* const* ls, const float* const* t
         for (int i = 0; i < n; i++) d[i] = ft_lora_dx_desc{dys[i], ls[i]->w, ls[i]->dtype, nullptr, nullptr, ls[i]->out, 0};
         return ft_lora_linear_dx_group(ctx, d, (size_t)n, nullptr, dx, T, ls[0]->in);
     }
-    FT_TRY(ft_side_join(ctx));  // factor gradients still in flight read the dt buffers
+    FT_TRY(ft_side_join(ctx, 0));  // factor gradients still in flight read the dt buffers
     FT_TRY(ft_thin_rowwise(ctx, rows, n));
     {
         FT_TRY(ft_side_begin(ctx));

@@ -22,31 +22,35 @@ struct ThinBatch {
 };
 
 // ---- row-wise ---------------------------------------------------------------
-// grid (ceil(M / 16), count); 256 threads = 4 waves. A workgroup owns 16 rows;
-// each wave takes a quarter of K through v_mfma_f32_16x16x4_f32 (X rows are the
-// A operand, Y columns the B operand, columns >= C fed with zeros), and the four
-// partial 16x16 tiles are added in wave order through LDS. Every lane reads X in
+// grid (ceil(M / 16), count); 512 threads = 8 waves. A workgroup owns 16 rows;
+// each wave takes an eighth of K through v_mfma_f32_16x16x4_f32 (X rows are the
+// A operand, Y columns the B operand, columns >= C fed with zeros), and the eight
+// partial 16x16 tiles are added in wave order through LDS. A wave issues the
+// loads of 8 iterations (128 k) together: at K around 1000 that is all of them,
+// so the launch costs one memory round trip. Every lane reads X in
 // 16-byte pieces: lane (row = l % 16, q = l / 16) takes k = 16*it + 4*q .. +3,
 // so MFMA e of an iteration contracts k = 16*it + 4*q + e.
 typedef float thin_f4 __attribute__((ext_vector_type(4)));
 
+constexpr int kRowWaves = 8;
+
 template <int C, bool YT>
-__global__ __launch_bounds__(256) void thin_rowwise_kernel(ThinBatch b) {
+__global__ __launch_bounds__(kRowWaves * 64) void thin_rowwise_kernel(ThinBatch b) {
     const ft_thin_problem& p = b.p[blockIdx.y];
     const int row0 = blockIdx.x * 16;
     if (row0 >= p.M) return;
-    __shared__ float red[4][16][17];
+    __shared__ float red[kRowWaves][16][17];
     const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
     const int li = lane % 16, q = lane / 16;
     const int row = row0 + li < p.M ? row0 + li : p.M - 1;  // clamped rows are computed and dropped
     const float* xr = p.x + (long)row * p.ldx + 4 * q;
     const bool col_live = li < C;
-    // K is a multiple of 4; the quarters are multiples of 16, so a 4-run of k is all in or all out.
-    const int part = ((p.K + 63) / 64) * 16;
+    // K is a multiple of 4; the parts are multiples of 16, so a 4-run of k is all in or all out.
+    const int part = ((p.K + 16 * kRowWaves - 1) / (16 * kRowWaves)) * 16;
     const int k_begin = wave * part;
     const int k_end = k_begin + part < p.K ? k_begin + part : p.K;
     thin_f4 acc = {0.f, 0.f, 0.f, 0.f};
-    constexpr int U = 4;  // iterations whose loads are issued together
+    constexpr int U = 8;  // iterations whose loads are issued together
     for (int k0 = k_begin; k0 < k_end; k0 += 16 * U) {
         float4 xa[U];
         float yb[U][4];
@@ -77,8 +81,10 @@ __global__ __launch_bounds__(256) void thin_rowwise_kernel(ThinBatch b) {
     for (int r = 0; r < 4; r++) red[wave][4 * q + r][li] = acc[r];
     __syncthreads();
     const int orow = threadIdx.x / 16, ocol = threadIdx.x % 16;
-    if (ocol < C && row0 + orow < p.M) {
-        const float v = ((red[0][orow][ocol] + red[1][orow][ocol]) + red[2][orow][ocol]) + red[3][orow][ocol];
+    if (threadIdx.x < 256 && ocol < C && row0 + orow < p.M) {
+        float v = red[0][orow][ocol];
+#pragma unroll
+        for (int w = 1; w < kRowWaves; w++) v += red[w][orow][ocol];
         p.out[(long)(row0 + orow) * p.ldo + ocol] = v * p.scale;
     }
 }
@@ -215,9 +221,9 @@ int ft_thin_rowwise(ft_context* ctx, const ft_thin_problem* probs, int count) {
 #define FT_ROW(CC)                                                                                              \
     do {                                                                                                        \
         if (probs[0].y_transposed)                                                                              \
-            hipLaunchKernelGGL((thin_rowwise_kernel<CC, true>), grid, dim3(256), 0, ctx->stream, b);           \
+            hipLaunchKernelGGL((thin_rowwise_kernel<CC, true>), grid, dim3(kRowWaves * 64), 0, ctx->stream, b); \
         else                                                                                                    \
-            hipLaunchKernelGGL((thin_rowwise_kernel<CC, false>), grid, dim3(256), 0, ctx->stream, b);          \
+            hipLaunchKernelGGL((thin_rowwise_kernel<CC, false>), grid, dim3(kRowWaves * 64), 0, ctx->stream, b); \
     } while (0)
     if (probs[0].C == 4) FT_ROW(4);
     else if (probs[0].C == 8) FT_ROW(8);
@@ -231,7 +237,7 @@ int ft_thin_colwise(ft_context* ctx, const ft_thin_problem* probs, int count) {
     FT_CHECK_ARG(ctx && probs && count >= 1 && count <= FT_THIN_MAX_BATCH, "thin colwise: bad batch");
     FT_TRY(ensure_scratch(ctx));
     // The partial-sum buffer is shared: a call on the main stream must not overtake one on the side stream.
-    if (!ctx->side_active) FT_TRY(ft_side_join(ctx));
+    if (ctx->side_active < 0) FT_TRY(ft_side_join(ctx, 0));
     ThinBatch b{};
     b.count = count;
     int rmax = 0, mmax = 0;
