@@ -18,6 +18,7 @@
 // operand registers, the reduction dimension split across the 4 waves.
 #include "ft_common.h"
 #include "ft_thin.h"
+#include <cstring>
 
 namespace {
 
@@ -1035,6 +1036,10 @@ int launch_async_auto(ft_context* ctx, const AsyncBatch& g, int layout) {
     size_t tiles128 = 0;
     for (int i = 0; i < g.count; i++) tiles128 += (size_t)((g.M + 127) / 128) * (size_t)((g.p[i].N + 127) / 128);
     if (tiles128 >= 8 * (size_t)ctx->num_cus) return launch_async<128, 128, 64, 64>(ctx, g, layout);
+    if (const char* t = getenv("FT_GEMM_TILE")) {
+        if (!strcmp(t, "64x128")) return launch_async<64, 128, 32, 64>(ctx, g, layout);
+        if (!strcmp(t, "128x64")) return launch_async<128, 64, 64, 32>(ctx, g, layout);
+    }
     return launch_async<64, 64, 32, 32>(ctx, g, layout);
 }
 

@@ -104,7 +104,8 @@ def test_f16_upload_is_bit_exact(g):
     np.testing.assert_array_equal(tf.to_numpy(), m.T)
 
 
-@pytest.mark.parametrize("M,K,N,r", [(64, 32, 48, 4), (256, 576, 1536, 8), (100, 960, 320, 8), (96, 64, 40, 16)])
+@pytest.mark.parametrize("M,K,N,r", [(64, 32, 48, 4), (256, 576, 1536, 8), (100, 960, 320, 8), (96, 64, 40, 16),
+                                     (2048, 576, 1536, 8)])  # the last: the kernel-microbench GEMM, full size
 @pytest.mark.parametrize("f16", [False, True])
 def test_fused_lora_linear_forward_and_backward(g, M, K, N, r, f16):
     """Linear::project_2d and its backward (graph/src/lib.rs:112-126; autograd MatMulNode/ScaleNode)."""
@@ -219,7 +220,8 @@ def test_fused_gated_mlp_halves(g, M, H, F, f16):
     assert_close("d_up", d_up.to_numpy(), want_du, atol=2e-3, rtol=1e-3)
 
 
-@pytest.mark.parametrize("rows,size", [(1, 1), (3, 7), (37, 96), (16, 576), (64, 960), (5, 2048), (3, 2100)])
+@pytest.mark.parametrize("rows,size", [(1, 1), (3, 7), (37, 96), (16, 576), (64, 960), (5, 2048), (3, 2100),
+                                       (2048, 576)])
 def test_rms_norm_forward_backward(g, rows, size):
     ctx, eng = g
     x, w, gy = rnd(1, rows, size), rnd(2, size), rnd(3, rows, size)
@@ -339,6 +341,23 @@ def test_sum_squares_and_adamw(g):
         np.testing.assert_array_equal(got, tw.to_numpy())
 
 
+def test_adamw_four_million_parameters(g):
+    """The kernel-microbench AdamW case: one fused update over 4M f32 parameters."""
+    ctx, eng = g
+    from ferrotensor_amd import AdamParams
+    n = 4 * 1024 * 1024
+    w0, gr = rnd(1, n), rnd(2, n)
+    m0, v0 = rnd(3, n, scale=0.1), np.abs(rnd(4, n, scale=0.1))
+    p = AdamParams(lr=2e-4, weight_decay=0.01, t=3.0)
+    w, m, v = w0.copy(), m0.copy(), v0.copy()
+    cpu.adamw_update(w, gr, m, v, p.lr, p.beta1, p.beta2, p.eps, p.weight_decay, p.t)
+    tw, tm, tv = up(ctx, w0), up(ctx, m0), up(ctx, v0)
+    eng.adamw_update(ctx, tw, up(ctx, gr), tm, tv, p)
+    assert_close("adamw w", tw.to_numpy(), w, atol=1e-6, rtol=1e-5)
+    assert_close("adamw m", tm.to_numpy(), m, atol=1e-7, rtol=1e-5)
+    assert_close("adamw v", tv.to_numpy(), v, atol=1e-7, rtol=1e-5)
+
+
 def test_errors_are_reported_not_fatal(g):
     from ferrotensor_amd import FtError
     ctx, eng = g
@@ -360,6 +379,8 @@ ATTN_CASES = [
     (2, 17, 17, 3, 1, 64, False, 0),
     (1, 100, 100, 2, 2, 64, True, 0),
     (2, 256, 256, 9, 3, 64, True, 0),       # SmolLM2-135M heads at seq 256
+    (8, 256, 256, 9, 3, 64, True, 0),       # the kernel-microbench attention case, full size
+    (2, 256, 256, 15, 5, 64, True, 0),      # SmolLM2-360M heads
     (1, 70, 70, 2, 1, 128, True, 0),
     (1, 33, 65, 2, 1, 32, True, 32),        # queries at positions 32.. against a longer key run
     (1, 5, 37, 4, 4, 24, False, 0),
