@@ -158,6 +158,27 @@ def cpu_baseline(w, seconds_budget=30.0):
                                                           cpu.num_threads())}
 
 
+def measured_traffic(kernel, workload):
+    """HBM-side bytes per launch of `kernel` (FETCH_SIZE + WRITE_SIZE, KiB per dispatch) as recorded by the
+    rocprofv3 --pmc runs summarised under profiles/; None when there is no record for this kernel."""
+    if workload != "360m":
+        return None
+    path = os.path.join(ROOT, "profiles", "lora_step_360m_hbm_traffic.md")
+    name = kernel
+    for tag, code in (("gate_up", "1"), ("silu_bwd", "2")):
+        name = name.replace(", %s>" % tag, ", %s>" % code)
+    if name == kernel:
+        name = kernel[:-1] + ", 0>"
+    try:
+        for line in open(path):
+            cells = [c.strip() for c in line.split("|")]
+            if len(cells) >= 5 and cells[1] == "`%s`" % name:
+                return (float(cells[3]) + float(cells[4])) * 1024.0
+    except (OSError, ValueError):
+        pass
+    return None
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -236,7 +257,8 @@ def main():
         "step_tflops": step_flops(w) / (elapsed / args.steps) / 1e12,
         "step_mfma_frac": step_flops(w) / (elapsed / args.steps) / 1e12 / FP32_MFMA_PEAK_TFLOPS,
         "roofline": {"bound": "mfma", "kernel": dom["name"], "achieved": achieved, "peak": FP32_MFMA_PEAK_TFLOPS,
-                     "unit": "TFLOP/s", "frac": achieved / FP32_MFMA_PEAK_TFLOPS, "traffic": None,
+                     "unit": "TFLOP/s", "frac": achieved / FP32_MFMA_PEAK_TFLOPS,
+                     "traffic": measured_traffic(dom["name"], args.workload),
                      "launches_per_step": dom["launches"] // args.steps,
                      "avg_launch_us": dom["ms"] * 1e3 / dom["launches"],
                      "all_gemm_kernels_tflops": all_gemm_tf,

@@ -18,7 +18,6 @@
 // operand registers, the reduction dimension split across the 4 waves.
 #include "ft_common.h"
 #include "ft_thin.h"
-#include <cstring>
 
 namespace {
 
@@ -1029,17 +1028,15 @@ int launch_async(ft_context* ctx, AsyncBatch g, int layout, int epi = kEpiPlain)
     return FT_OK;
 }
 
-// 128x128 tiles (64x64 per wave) reach the highest MFMA occupancy but only pay
-// off when there are many of them per CU (the vocabulary head); everything
-// smaller runs best as 64x64 tiles, which keep several workgroups resident per CU.
+// Tile choice, from measurements of the whole step on MI355X at M = 2048: 128x128
+// tiles (64x64 per wave) reach the highest MFMA rate but only pay off when there
+// are many of them per CU (the vocabulary head); everything else runs best as
+// 64x64 tiles, three workgroups resident per CU (128x64 and 64x128 tiles were
+// measured too: no gain inside the step).
 int launch_async_auto(ft_context* ctx, const AsyncBatch& g, int layout) {
     size_t tiles128 = 0;
     for (int i = 0; i < g.count; i++) tiles128 += (size_t)((g.M + 127) / 128) * (size_t)((g.p[i].N + 127) / 128);
     if (tiles128 >= 8 * (size_t)ctx->num_cus) return launch_async<128, 128, 64, 64>(ctx, g, layout);
-    if (const char* t = getenv("FT_GEMM_TILE")) {
-        if (!strcmp(t, "64x128")) return launch_async<64, 128, 32, 64>(ctx, g, layout);
-        if (!strcmp(t, "128x64")) return launch_async<128, 64, 64, 32>(ctx, g, layout);
-    }
     return launch_async<64, 64, 32, 32>(ctx, g, layout);
 }
 
