@@ -44,12 +44,14 @@ class ModelConfigC(C.Structure):
 
 class TrainerConfigC(C.Structure):
     _fields_ = [("lr", C.c_float), ("beta1", C.c_float), ("beta2", C.c_float), ("eps", C.c_float),
-                ("weight_decay", C.c_float), ("clip_grad_norm", C.c_float), ("grad_accum_steps", C.c_uint32)]
+                ("weight_decay", C.c_float), ("clip_grad_norm", C.c_float), ("grad_accum_steps", C.c_uint32),
+                ("lr_schedule", C.c_uint32), ("warmup_steps", C.c_uint32), ("total_steps", C.c_uint32),
+                ("min_lr", C.c_float)]
 
 
 class StepStatsC(C.Structure):
     _fields_ = [("loss", C.c_float), ("grad_norm", C.c_float), ("clip_scale", C.c_float),
-                ("supervised_tokens", C.c_uint32), ("optimizer_step", C.c_int32)]
+                ("supervised_tokens", C.c_uint32), ("optimizer_step", C.c_int32), ("lr", C.c_float)]
 
 
 _P = C.c_void_p
@@ -128,9 +130,12 @@ SIGNATURES = {
     "ft_model_forward_logits": [_P, _P, _SZ, _SZ, _P],
     "ft_trainer_create": [_P, C.POINTER(TrainerConfigC), C.POINTER(_P)],
     "ft_trainer_destroy": [_P],
+    "ft_trainer_optimizer_steps": [_P, C.POINTER(_SZ)],
+    "ft_trainer_set_optimizer_steps": [_P, _SZ],
+    "ft_lr_schedule": [C.c_uint32, _F, _F, C.c_uint32, C.c_uint32, C.c_uint32],
     "ft_trainer_train_chunk": [_P, _P, _P, _P, _SZ, _SZ, _I, C.POINTER(StepStatsC), _P],
 }
-_RESTYPES = {"ft_last_error": C.c_char_p, "ft_context_stream": _P}
+_RESTYPES = {"ft_last_error": C.c_char_p, "ft_context_stream": _P, "ft_lr_schedule": C.c_float}
 
 _lib = None
 

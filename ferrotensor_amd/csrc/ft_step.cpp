@@ -119,6 +119,7 @@ struct ft_trainer {
     ft_model* model = nullptr;
     ft_trainer_config cfg{};
     float t = 0.0f;                 // AdamW step counter (f32, as in the reference)
+    size_t optimizer_steps = 0;     // steps taken = position of the LR schedule
     size_t step_in_accum = 0;
     std::vector<float*> m, v;       // per parameter
     ft_segment* segs_dev = nullptr;
@@ -769,6 +770,37 @@ int ft_trainer_destroy(ft_trainer* t) {
     return FT_OK;
 }
 
+float ft_lr_schedule(uint32_t kind, float peak_lr, float min_lr, uint32_t warmup_steps, uint32_t total_steps,
+                     uint32_t step) {
+    const float pi = 3.14159265358979323846f;
+    if (kind == FT_LR_COSINE) {
+        if (step >= total_steps) return min_lr;
+        const float progress = (float)step / (float)total_steps;
+        const float cosine = (1.0f + cosf(pi * progress)) / 2.0f;
+        return min_lr + (peak_lr - min_lr) * cosine;
+    }
+    if (kind == FT_LR_WARMUP_COSINE) {
+        if (step < warmup_steps) return peak_lr * ((float)step / (float)warmup_steps);
+        if (step >= total_steps) return min_lr;
+        const float progress = (float)(step - warmup_steps) / (float)(total_steps - warmup_steps);
+        const float cosine = (1.0f + cosf(pi * progress)) / 2.0f;
+        return min_lr + (peak_lr - min_lr) * cosine;
+    }
+    return peak_lr;
+}
+
+int ft_trainer_optimizer_steps(ft_trainer* t, size_t* steps) {
+    FT_CHECK_ARG(t && steps, "ft_trainer_optimizer_steps: NULL argument");
+    *steps = t->optimizer_steps;
+    return FT_OK;
+}
+
+int ft_trainer_set_optimizer_steps(ft_trainer* t, size_t steps) {
+    FT_CHECK_ARG(t, "ft_trainer_set_optimizer_steps: NULL argument");
+    t->optimizer_steps = steps;
+    return FT_OK;
+}
+
 int ft_trainer_train_chunk(ft_trainer* t, const uint32_t* rows, const uint32_t* targets, const uint8_t* loss_mask,
                            size_t B, size_t S, int apply, ft_step_stats* stats, float* per_sequence_loss) {
     return guarded([&]() -> int {
@@ -823,7 +855,10 @@ int ft_trainer_train_chunk(ft_trainer* t, const uint32_t* rows, const uint32_t* 
 
         const bool window_full = t->step_in_accum >= accum;
         bool launched_update = false;
-        ft_adam_params ap{t->cfg.lr, t->cfg.beta1, t->cfg.beta2, t->cfg.eps, t->cfg.weight_decay, t->t + 1.0f};
+        // Step k (1-based) uses the schedule's value at k (trainer/src/lib.rs:345-352).
+        const float lr = ft_lr_schedule(t->cfg.lr_schedule, t->cfg.lr, t->cfg.min_lr, t->cfg.warmup_steps,
+                                        t->cfg.total_steps, (uint32_t)(t->optimizer_steps + 1));
+        ft_adam_params ap{lr, t->cfg.beta1, t->cfg.beta2, t->cfg.eps, t->cfg.weight_decay, t->t + 1.0f};
         if (window_full) {
             t->step_in_accum = 0;
             if (total_tokens > 0 || true) {
@@ -858,8 +893,11 @@ int ft_trainer_train_chunk(ft_trainer* t, const uint32_t* rows, const uint32_t* 
             stats->grad_norm = control[0];
             stats->clip_scale = control[1];
             if (launched_update && applied) {
+                // A skipped step leaves both counters alone, so the schedule does not advance either.
                 t->t += 1.0f;
+                t->optimizer_steps += 1;
                 stats->optimizer_step = 1;
+                stats->lr = lr;
             }
         }
         return FT_OK;

@@ -55,6 +55,7 @@ class StepStats:
     grad_norm: Optional[float]
     clip_scale: float
     per_sequence: List[float]
+    lr: Optional[float] = None
 
 
 class Lfm2Model:
@@ -160,6 +161,14 @@ class Lfm2Model:
             pass
 
 
+LR_SCHEDULES = {"constant": 0, "cosine": 1, "warmup_cosine": 2}
+
+
+def lr_schedule(kind: str, peak_lr: float, min_lr: float, warmup_steps: int, total_steps: int, step: int) -> float:
+    """`LRScheduler::get_lr` after `step` calls of `step()` (autograd/src/lib.rs:1705-1814)."""
+    return float(_lib.load().ft_lr_schedule(LR_SCHEDULES[kind], peak_lr, min_lr, warmup_steps, total_steps, step))
+
+
 def pad_chunk(seqs, length_bucket=32):
     """`Trainer::train_chunk` padding (trainer/src/lib.rs:431-450): right-pad to a
     multiple of `length_bucket` with each row's last token, loss mask 0."""
@@ -179,12 +188,18 @@ class Trainer:
     """`Trainer::new(..).with_grad_accum_steps(..).with_clip_grad_norm(..)` with an AdamW optimizer."""
 
     def __init__(self, model: Lfm2Model, lr: float, beta1=0.9, beta2=0.999, eps=1e-8, weight_decay=0.01,
-                 clip_grad_norm: Optional[float] = None, grad_accum_steps: int = 0, length_bucket: int = 32):
+                 clip_grad_norm: Optional[float] = None, grad_accum_steps: int = 0, length_bucket: int = 32,
+                 lr_schedule: str = "constant", warmup_steps: int = 0, total_steps: int = 0, min_lr: float = 0.0):
+        """`lr_schedule`: "constant", "cosine" (`CosineAnnealingLR`) or "warmup_cosine"
+        (`WarmupCosineScheduler`, what the CLI's train command installs with min_lr = lr / 10,
+        ferrotensor-cli/src/main.rs:1686-1695); `lr` is the peak rate."""
         self.model = model
         self.length_bucket = length_bucket
         self._lib = model._lib
+        kind = LR_SCHEDULES[lr_schedule]
         cfg = _lib.TrainerConfigC(lr, beta1, beta2, eps, weight_decay,
-                                  clip_grad_norm if clip_grad_norm else 0.0, grad_accum_steps)
+                                  clip_grad_norm if clip_grad_norm else 0.0, grad_accum_steps,
+                                  kind, warmup_steps, total_steps, min_lr)
         h = C.c_void_p()
         check(self._lib.ft_trainer_create(model.handle, C.byref(cfg), C.byref(h)))
         self.handle = h
@@ -202,7 +217,18 @@ class Trainer:
                                                targets.ctypes.data_as(C.c_void_p), masks.ctypes.data_as(C.c_void_p),
                                                B, S, 1 if apply else 0, C.byref(st), per.ctypes.data_as(C.c_void_p)))
         return StepStats(loss=st.loss, tokens=st.supervised_tokens, optimizer_step=bool(st.optimizer_step),
-                         grad_norm=st.grad_norm, clip_scale=st.clip_scale, per_sequence=per.tolist())
+                         grad_norm=st.grad_norm, clip_scale=st.clip_scale, per_sequence=per.tolist(),
+                         lr=st.lr if st.optimizer_step else None)
+
+    @property
+    def optimizer_steps(self) -> int:
+        n = C.c_size_t()
+        check(self._lib.ft_trainer_optimizer_steps(self.handle, C.byref(n)))
+        return n.value
+
+    def set_optimizer_steps(self, steps: int):
+        """Resume: restores the step counter, which is also the position of the LR schedule."""
+        check(self._lib.ft_trainer_set_optimizer_steps(self.handle, steps))
 
     def train_batch(self, seqs, apply: bool = True) -> StepStats:
         """Ragged sequences [(input_ids, target_ids, loss_mask)]: dropped when

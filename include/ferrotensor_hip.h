@@ -366,7 +366,26 @@ typedef struct ft_trainer_config {
     float lr, beta1, beta2, eps, weight_decay;
     float clip_grad_norm;
     uint32_t grad_accum_steps;   /* 0 = the chunk's number of sequences */
+    /* Trainer::with_lr_scheduler (trainer/src/lib.rs:172-176): FT_LR_CONSTANT keeps `lr`;
+     * otherwise optimizer step k (1-based) uses ft_lr_schedule(.., k) with peak `lr`
+     * (apply_gradients, trainer/src/lib.rs:345-352). A skipped step (non-finite
+     * gradient norm) does not advance the schedule. */
+    uint32_t lr_schedule;
+    uint32_t warmup_steps;
+    uint32_t total_steps;
+    float min_lr;
 } ft_trainer_config;
+
+#define FT_LR_CONSTANT 0u
+#define FT_LR_COSINE 1u         /* CosineAnnealingLR (autograd/src/lib.rs:1717-1758) */
+#define FT_LR_WARMUP_COSINE 2u  /* WarmupCosineScheduler (autograd/src/lib.rs:1761-1814) */
+
+/* LRScheduler::get_lr after `step` calls of step() (f32 arithmetic as in the
+ * reference): cosine from peak to min over total_steps, or linear warm-up from 0
+ * to peak over warmup_steps followed by the cosine to min at total_steps. Host
+ * only; never touches the GPU. */
+float ft_lr_schedule(uint32_t kind, float peak_lr, float min_lr, uint32_t warmup_steps, uint32_t total_steps,
+                     uint32_t step);
 
 /* StepStats of a chunk (trainer/src/lib.rs:36-58). */
 typedef struct ft_step_stats {
@@ -375,10 +394,15 @@ typedef struct ft_step_stats {
     float clip_scale;      /* 1.0 when not clipped */
     uint32_t supervised_tokens;
     int32_t optimizer_step;
+    float lr;              /* the rate the optimizer step used (0 when no step was taken) */
 } ft_step_stats;
 
 int ft_trainer_create(ft_model* m, const ft_trainer_config* cfg, ft_trainer** out);
 int ft_trainer_destroy(ft_trainer* t);
+/* Trainer::optimizer_steps / set_optimizer_steps (trainer/src/lib.rs:199-213): the
+ * number of optimizer steps taken; setting it (resume) also advances the schedule. */
+int ft_trainer_optimizer_steps(ft_trainer* t, size_t* steps);
+int ft_trainer_set_optimizer_steps(ft_trainer* t, size_t steps);
 /* Trainer::train_chunk (trainer/src/lib.rs:426-502) for B equally long rows
  * (already padded; see ft_pad_chunk): forward, masked cross-entropy, backward
  * with seed 1/grad_accum_steps, gradient norm, clip, AdamW. rows/targets are

@@ -374,12 +374,55 @@ class AdamW:
 
 
 @dataclass
+class CosineAnnealingLR:
+    """`CosineAnnealingLR` (autograd/src/lib.rs:1717-1758), f32 arithmetic."""
+    initial_lr: float
+    min_lr: float
+    total_steps: int
+    current: int = 0
+
+    def get_lr(self) -> float:
+        if self.current >= self.total_steps:
+            return float(np.float32(self.min_lr))
+        progress = np.float32(self.current) / np.float32(self.total_steps)
+        cosine = (np.float32(1.0) + np.cos(np.float32(np.pi) * progress, dtype=np.float32)) / np.float32(2.0)
+        return float(np.float32(self.min_lr) + (np.float32(self.initial_lr) - np.float32(self.min_lr)) * cosine)
+
+    def step(self):
+        self.current += 1
+
+
+@dataclass
+class WarmupCosineScheduler:
+    """`WarmupCosineScheduler` (autograd/src/lib.rs:1761-1814), f32 arithmetic."""
+    peak_lr: float
+    min_lr: float
+    warmup_steps: int
+    total_steps: int
+    current: int = 0
+
+    def get_lr(self) -> float:
+        peak, low = np.float32(self.peak_lr), np.float32(self.min_lr)
+        if self.current < self.warmup_steps:
+            return float(peak * (np.float32(self.current) / np.float32(self.warmup_steps)))
+        if self.current >= self.total_steps:
+            return float(low)
+        progress = np.float32(self.current - self.warmup_steps) / np.float32(self.total_steps - self.warmup_steps)
+        cosine = (np.float32(1.0) + np.cos(np.float32(np.pi) * progress, dtype=np.float32)) / np.float32(2.0)
+        return float(low + (peak - low) * cosine)
+
+    def step(self):
+        self.current += 1
+
+
+@dataclass
 class StepStats:
     loss: float
     per_sequence: List[Tuple[float, int]]
     grad_norm: Optional[float]
     optimizer_step: bool
     clip_scale: Optional[float] = None
+    lr: Optional[float] = None
 
 
 def pad_chunk(seqs, length_bucket=32):
@@ -398,7 +441,7 @@ def pad_chunk(seqs, length_bucket=32):
 
 
 def train_chunk(model: Model, opt: AdamW, rows, targets, masks, grad_accum_steps=None,
-                clip_grad_norm: Optional[float] = None, trainable_base=False, return_grads=False):
+                clip_grad_norm: Optional[float] = None, trainable_base=False, return_grads=False, scheduler=None):
     """One forward + backward over equally long rows and one optimizer step
     (`Trainer::train_chunk` with the chunk filling the accumulation window:
     the CLI sets grad_accum_steps = batch * accum, main.rs:1687-1695)."""
@@ -426,6 +469,10 @@ def train_chunk(model: Model, opt: AdamW, rows, targets, masks, grad_accum_steps
             for n, _ in params:
                 if n in grads:
                     grads[n] = cpu.scale(grads[n], float(s))
+        if scheduler is not None:   # apply_gradients, trainer/src/lib.rs:345-352: step k uses the value at k
+            scheduler.step()
+            opt.lr = scheduler.get_lr()
+            stats.lr = opt.lr
         opt.step(params, grads)
         stats.optimizer_step = True
     if return_grads:

@@ -51,3 +51,21 @@ def test_product_does_not_import_the_oracle():
             if f.endswith((".py", ".cpp", ".hip", ".h")):
                 text = open(os.path.join(dirpath, f)).read()
                 assert "oracle" not in text.replace("the oracle", ""), os.path.join(dirpath, f)
+
+
+def test_lr_schedule_entry_point_matches_the_oracle():
+    """ft_lr_schedule is host arithmetic (no GPU): compared with the restated schedulers step by step."""
+    from ferrotensor_amd.trainer import lr_schedule
+    from oracle import reference_step as rs
+    import numpy as np
+    for peak, low, warm, total in [(1.0, 0.1, 4, 14), (2e-4, 2e-5, 100, 1000), (3e-4, 0.0, 0, 50), (1e-3, 1e-4, 7, 7)]:
+        w = rs.WarmupCosineScheduler(peak, low, warm, total)
+        c = rs.CosineAnnealingLR(peak, low, total)
+        for k in range(total + 3):
+            got = lr_schedule("warmup_cosine", peak, low, warm, total, k)
+            assert abs(got - w.get_lr()) <= 2e-7 * peak, (peak, low, warm, total, k, got, w.get_lr())
+            got = lr_schedule("cosine", peak, low, warm, total, k)
+            assert abs(got - c.get_lr()) <= 2e-7 * peak
+            assert lr_schedule("constant", peak, low, warm, total, k) == np.float32(peak)
+            w.step()
+            c.step()

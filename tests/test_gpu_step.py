@@ -176,6 +176,36 @@ def test_tiny_llama_full_step_matches_oracle(ctx, f16, tied):
             assert_close(f"step {step} weight {n}", params[n], w, atol=1e-6, rtol=1e-4)
 
 
+def test_warmup_cosine_schedule_drives_the_step(ctx):
+    """Optimizer step k uses the schedule's value at k (trainer/src/lib.rs:345-352); a resumed
+    trainer continues the curve where the counter says."""
+    from ferrotensor_amd.trainer import Trainer
+    cfg = tiny_config()
+    hip, orc = build_pair(ctx, cfg, ["q_proj", "k_proj", "v_proj", "o_proj"], rank=4, alpha=8.0, seed=21)
+    rng = np.random.default_rng(6)
+    rows = rng.integers(0, 256, (2, 16)).astype(np.uint32)
+    targets = np.concatenate([rows[:, 1:], rows[:, :1]], axis=1)
+    masks = np.ones((2, 16), np.uint8)
+    peak, low, warm, total = 2e-3, 2e-4, 2, 6
+    tr = Trainer(hip, lr=peak, weight_decay=0.0, lr_schedule="warmup_cosine", warmup_steps=warm, total_steps=total,
+                 min_lr=low)
+    opt = rs.AdamW(lr=peak, weight_decay=0.0)
+    sched = rs.WarmupCosineScheduler(peak, low, warm, total)
+    for step in range(4):
+        want = rs.train_chunk(orc, opt, rows, targets, masks, scheduler=sched)
+        st = tr.train_chunk(rows, targets, masks)
+        assert st.optimizer_step and tr.optimizer_steps == step + 1
+        assert abs(st.lr - want.lr) <= 2e-7 * peak, (step, st.lr, want.lr)
+        assert_close("loss", [st.loss], [want.loss])
+        params = hip.params()
+        for n, w in orc.lora_params():
+            assert_close(f"step {step} weight {n}", params[n], w, atol=1e-6, rtol=1e-4)
+    # resume at step 5 of 6: the next step is the last of the curve and lands on min_lr
+    tr.set_optimizer_steps(5)
+    st = tr.train_chunk(rows, targets, masks)
+    assert st.lr == np.float32(low) and tr.optimizer_steps == 6
+
+
 def test_targets_masking_is_bit_exact_against_oracle(ctx):
     """Skipped rows (mask 0 or target >= vocab) contribute exactly nothing:
     the loss equals the oracle's and flipping masked targets changes no bit."""

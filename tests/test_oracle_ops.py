@@ -240,3 +240,27 @@ def test_embedding_out_of_range_row_is_zero():
     np.testing.assert_array_equal(out[0, 0], table[0])
     np.testing.assert_array_equal(out[0, 1], table[4])
     assert (out[0, 2:] == 0).all()
+
+
+def test_lr_schedulers_follow_the_reference_curves():
+    """The vectors of `schedulers_follow_their_curves` (autograd/src/lib.rs:1914-1941)."""
+    cosine = rs.CosineAnnealingLR(1.0, 0.0, 10)
+    assert cosine.get_lr() == 1.0
+    for _ in range(5):
+        cosine.step()
+    assert abs(cosine.get_lr() - 0.5) < 1e-6
+    for _ in range(5):
+        cosine.step()
+    assert cosine.get_lr() == 0.0 and cosine.current == 10
+
+    warm = rs.WarmupCosineScheduler(1.0, 0.1, 4, 14)
+    lrs = []
+    for _ in range(15):
+        lrs.append(warm.get_lr())
+        warm.step()
+    assert lrs[:5] == [0.0, 0.25, 0.5, 0.75, 1.0]
+    assert abs(lrs[9] - 0.55) < 1e-6
+    assert lrs[14] == np.float32(0.1)
+    # monotone: up through the warm-up, down afterwards, never below min_lr
+    assert all(a < b for a, b in zip(lrs[:4], lrs[1:5]))
+    assert all(a > b for a, b in zip(lrs[4:14], lrs[5:15]))
