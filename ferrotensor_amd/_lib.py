@@ -132,10 +132,13 @@ SIGNATURES = {
     "ft_trainer_destroy": [_P],
     "ft_trainer_optimizer_steps": [_P, C.POINTER(_SZ)],
     "ft_trainer_set_optimizer_steps": [_P, _SZ],
+    "ft_lora_seed": [C.c_uint64, C.c_char_p],
+    "ft_lora_init_a": [_P, _SZ, _SZ, _SZ, C.c_uint64],
+    "ft_model_add_lora": [_P, C.c_char_p, _SZ, _F],
     "ft_lr_schedule": [C.c_uint32, _F, _F, C.c_uint32, C.c_uint32, C.c_uint32],
     "ft_trainer_train_chunk": [_P, _P, _P, _P, _SZ, _SZ, _I, C.POINTER(StepStatsC), _P],
 }
-_RESTYPES = {"ft_last_error": C.c_char_p, "ft_context_stream": _P, "ft_lr_schedule": C.c_float}
+_RESTYPES = {"ft_last_error": C.c_char_p, "ft_context_stream": _P, "ft_lr_schedule": C.c_float, "ft_lora_seed": C.c_uint64}
 
 _lib = None
 

@@ -678,6 +678,57 @@ int ft_model_set_lora(ft_model* m, const char* prefix, const float* a, const flo
     });
 }
 
+uint64_t ft_lora_seed(uint64_t layer_seed, const char* module_name) {
+    // FNV-1a over the name bytes, then the seed's little-endian bytes, then the splitmix64 finalizer.
+    uint64_t h = 0xcbf29ce484222325ull;
+    auto mix = [&](uint8_t byte) {
+        h ^= (uint64_t)byte;
+        h *= 0x00000100000001b3ull;
+    };
+    for (const char* c = module_name ? module_name : ""; *c; c++) mix((uint8_t)*c);
+    for (int i = 0; i < 8; i++) mix((uint8_t)(layer_seed >> (8 * i)));
+    h ^= h >> 30;
+    h *= 0xbf58476d1ce4e5b9ull;
+    h ^= h >> 27;
+    h *= 0x94d049bb133111ebull;
+    return h ^ (h >> 31);
+}
+
+int ft_lora_init_a(float* a_host, size_t in_dim, size_t out_dim, size_t rank, uint64_t seed) {
+    FT_CHECK_ARG(a_host || in_dim * rank == 0, "ft_lora_init_a: NULL argument");
+    const float bound = 1.0f / std::sqrt((float)(in_dim > 0 ? in_dim : 1));
+    uint64_t state =
+        (seed * 0x9E3779B97F4A7C15ull + (((uint64_t)in_dim << 32) | ((uint64_t)out_dim << 8) | (uint64_t)rank)) | 1ull;
+    for (size_t i = 0; i < in_dim * rank; i++) {
+        // xorshift64*
+        state ^= state >> 12;
+        state ^= state << 25;
+        state ^= state >> 27;
+        const uint64_t bits = (state * 0x2545F4914F6CDD1Dull) >> 40;
+        const float unit = (float)bits / (float)(1ull << 24);
+        a_host[i] = (unit * 2.0f - 1.0f) * bound;
+    }
+    return FT_OK;
+}
+
+int ft_model_add_lora(ft_model* m, const char* prefix, size_t rank, float alpha) {
+    return guarded([&]() -> int {
+        FT_CHECK_ARG(m && prefix, "ft_model_add_lora: NULL argument");
+        LinearW* l = find_linear(m, prefix);
+        FT_CHECK_ARG(l, "ft_model_add_lora: no linear named %s", prefix);
+        // layer seed = layer index + 1, 0 for lm_head; module name = last component of the prefix
+        const std::string pre(prefix);
+        uint64_t layer_seed = 0;
+        const size_t at = pre.find("layers.");
+        if (at != std::string::npos) layer_seed = (uint64_t)std::strtoull(pre.c_str() + at + 7, nullptr, 10) + 1;
+        const size_t dot = pre.rfind('.');
+        const std::string module = dot == std::string::npos ? pre : pre.substr(dot + 1);
+        std::vector<float> a(l->in * rank), b(rank * l->out, 0.0f);
+        FT_TRY(ft_lora_init_a(a.data(), l->in, l->out, rank, ft_lora_seed(layer_seed, module.c_str())));
+        return ft_model_set_lora(m, prefix, a.data(), b.data(), rank, alpha);
+    });
+}
+
 int ft_model_param_count(ft_model* m, size_t* count) {
     return guarded([&]() -> int {
         FT_CHECK_ARG(m && count, "ft_model_param_count: NULL argument");

@@ -88,6 +88,10 @@ class Lfm2Model:
         check(self._lib.ft_model_set_lora(self.handle, prefix.encode(), a.ctypes.data_as(C.c_void_p),
                                           b.ctypes.data_as(C.c_void_p), a.shape[1], alpha))
 
+    def add_lora(self, prefix: str, rank: int, alpha: float):
+        """`ModelBuilder::maybe_add_lora`: a fresh adapter, A seeded from (layer, module name), B zero."""
+        check(self._lib.ft_model_add_lora(self.handle, prefix.encode(), rank, alpha))
+
     def linear_prefixes(self, targets: Sequence[str]) -> List[str]:
         out = []
         for l in range(self.config.num_hidden_layers):
@@ -167,6 +171,18 @@ LR_SCHEDULES = {"constant": 0, "cosine": 1, "warmup_cosine": 2}
 def lr_schedule(kind: str, peak_lr: float, min_lr: float, warmup_steps: int, total_steps: int, step: int) -> float:
     """`LRScheduler::get_lr` after `step` calls of `step()` (autograd/src/lib.rs:1705-1814)."""
     return float(_lib.load().ft_lr_schedule(LR_SCHEDULES[kind], peak_lr, min_lr, warmup_steps, total_steps, step))
+
+
+def lora_seed(layer_seed: int, module_name: str) -> int:
+    """`lora_seed` (model_builder.rs:739-759)."""
+    return int(_lib.load().ft_lora_seed(layer_seed, module_name.encode()))
+
+
+def lora_init_a(in_dim: int, out_dim: int, rank: int, seed: int) -> np.ndarray:
+    """`LoRAAdapter::new_seeded`'s A matrix [in_dim, rank] (graph/src/lib.rs:59-92)."""
+    a = np.empty((in_dim, rank), np.float32)
+    check(_lib.load().ft_lora_init_a(a.ctypes.data_as(C.c_void_p), in_dim, out_dim, rank, seed))
+    return a
 
 
 def pad_chunk(seqs, length_bucket=32):

@@ -348,6 +348,16 @@ int ft_model_set_tensor(ft_model* m, const char* hf_name, const float* data, con
  * named `prefix` (`model.layers.N.self_attn.q_proj`, `lm_head`, ...):
  * a [in, rank], b [rank, out], both copied. */
 int ft_model_set_lora(ft_model* m, const char* prefix, const float* a, const float* b, size_t rank, float alpha);
+/* lora_seed (model_builder.rs:739-759): the seed of the adapter of `module_name`
+ * ("q_proj", ...) in the layer with seed `layer_seed` (layer index + 1; 0 for
+ * lm_head). Pure integer arithmetic, bit-exact with the reference's pinned values. */
+uint64_t ft_lora_seed(uint64_t layer_seed, const char* module_name);
+/* LoRAAdapter::new_seeded (graph/src/lib.rs:59-92): fills a[in_dim*rank] (host
+ * memory) with xorshift64* draws, uniform in +-1/sqrt(in_dim). */
+int ft_lora_init_a(float* a_host, size_t in_dim, size_t out_dim, size_t rank, uint64_t seed);
+/* ModelBuilder::maybe_add_lora (model_builder.rs:425-446): attaches a freshly
+ * initialised adapter (seeded A, zero B) to the linear named `prefix`. */
+int ft_model_add_lora(ft_model* m, const char* prefix, size_t rank, float alpha);
 /* Number of trainable tensors and their fixture names / sizes, in the order
  * gradients and parameters are reported (`<prefix>.lora_a`, `<prefix>.lora_b`). */
 int ft_model_param_count(ft_model* m, size_t* count);

@@ -373,6 +373,39 @@ class AdamW:
                              self.eps, self.weight_decay, self.t)
 
 
+_M64 = (1 << 64) - 1
+
+
+def lora_seed(layer_seed: int, module_name: str) -> int:
+    """`lora_seed` (model_builder.rs:739-759): FNV-1a over the name bytes and the seed's
+    little-endian bytes, then the splitmix64 finalizer. Pinned values at model_builder.rs:870-876."""
+    h = 0xcbf29ce484222325
+    for byte in module_name.encode() + int(layer_seed).to_bytes(8, "little"):
+        h ^= byte
+        h = (h * 0x00000100000001b3) & _M64
+    h ^= h >> 30
+    h = (h * 0xbf58476d1ce4e5b9) & _M64
+    h ^= h >> 27
+    h = (h * 0x94d049bb133111eb) & _M64
+    return h ^ (h >> 31)
+
+
+def lora_init_a(in_dim: int, out_dim: int, rank: int, seed: int) -> np.ndarray:
+    """`LoRAAdapter::new_seeded` (graph/src/lib.rs:59-92): A [in, rank] uniform in +-1/sqrt(in)
+    from xorshift64* (shifts 12, 25, 27; multiplier 0x2545F4914F6CDD1D; top 24 bits)."""
+    bound = np.float32(1.0) / np.sqrt(np.float32(max(in_dim, 1)))
+    state = ((seed * 0x9E3779B97F4A7C15 + ((in_dim << 32) | (out_dim << 8) | rank)) & _M64) | 1
+    out = np.empty(in_dim * rank, np.float32)
+    for i in range(in_dim * rank):
+        state ^= state >> 12
+        state = (state ^ (state << 25)) & _M64
+        state ^= state >> 27
+        bits = ((state * 0x2545F4914F6CDD1D) & _M64) >> 40
+        unit = np.float32(bits) / np.float32(1 << 24)
+        out[i] = (unit * np.float32(2.0) - np.float32(1.0)) * bound
+    return out.reshape(in_dim, rank)
+
+
 @dataclass
 class CosineAnnealingLR:
     """`CosineAnnealingLR` (autograd/src/lib.rs:1717-1758), f32 arithmetic."""

@@ -206,6 +206,32 @@ def test_warmup_cosine_schedule_drives_the_step(ctx):
     assert st.lr == np.float32(low) and tr.optimizer_steps == 6
 
 
+def test_fresh_adapters_are_seeded_like_the_builder(ctx):
+    """`maybe_add_lora`: A from xorshift64* seeded by (layer index + 1, module name), B zero, so the
+    model starts at the base logits; one training step then moves B away from zero."""
+    from ferrotensor_amd.trainer import Trainer
+    cfg = tiny_config()
+    hip, orc = build_pair(ctx, cfg, [], rank=4, alpha=8.0, seed=13)
+    rows = np.random.default_rng(2).integers(0, 256, (2, 16)).astype(np.uint32)
+    base = hip.forward_batch(rows)
+    for prefix in hip.linear_prefixes(["q_proj", "v_proj", "down_proj"]):
+        hip.add_lora(prefix, 4, 8.0)
+    params = hip.params()
+    for layer in range(cfg.num_hidden_layers):
+        for mod, sub in (("q_proj", "self_attn"), ("v_proj", "self_attn"), ("down_proj", "mlp")):
+            prefix = f"model.layers.{layer}.{sub}.{mod}"
+            i, o = hip.linear_dims(prefix)
+            want = rs.lora_init_a(i, o, 4, rs.lora_seed(layer + 1, mod))
+            np.testing.assert_array_equal(params[prefix + ".lora_a"].reshape(want.shape), want)
+            assert not params[prefix + ".lora_b"].any()
+    np.testing.assert_array_equal(hip.forward_batch(rows), base)
+    targets = np.concatenate([rows[:, 1:], rows[:, :1]], axis=1)
+    st = Trainer(hip, lr=1e-2, weight_decay=0.0).train_chunk(rows, targets, np.ones((2, 16), np.uint8))
+    assert st.optimizer_step
+    after = hip.params()
+    assert all(after[n].any() for n in after if n.endswith(".lora_b"))
+
+
 def test_targets_masking_is_bit_exact_against_oracle(ctx):
     """Skipped rows (mask 0 or target >= vocab) contribute exactly nothing:
     the loss equals the oracle's and flipping masked targets changes no bit."""

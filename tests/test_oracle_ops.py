@@ -264,3 +264,38 @@ def test_lr_schedulers_follow_the_reference_curves():
     # monotone: up through the warm-up, down afterwards, never below min_lr
     assert all(a < b for a, b in zip(lrs[:4], lrs[1:5]))
     assert all(a > b for a, b in zip(lrs[4:14], lrs[5:15]))
+
+
+def test_lora_seed_pinned_values():
+    """`lora_seed_is_pinned` (model_builder.rs:869-876)."""
+    assert rs.lora_seed(1, "q_proj") == 0x5f28d61921d3ddb3
+    assert rs.lora_seed(1, "o_proj") == 0xfabfd7977f143d7c
+    assert rs.lora_seed(2, "q_proj") == 0x4bae9242648e2fc1
+    assert rs.lora_seed(0, "lm_head") == 0x6d1a1dffacc30def
+
+
+def test_lora_init_a_is_xorshift64star_uniform():
+    """The generator is the published xorshift64* (Vigna): from state 1 its first output is
+    0x2000001 * 0x2545F4914F6CDD1D mod 2^64 (the three shifts of 1 give 0x2000001). The matrix is
+    uniform in +-1/sqrt(in), differs between seeds and shapes, and is not rank-1."""
+    first_state = 0x2000001
+    first_bits = ((first_state * 0x2545F4914F6CDD1D) & ((1 << 64) - 1)) >> 40
+    # choose seed / dims so that the initial state is exactly 1: seed 0, in = out = rank = 0 is degenerate,
+    # so check through the recurrence instead: state0 = (0 + (in<<32 | out<<8 | rank)) | 1
+    a = rs.lora_init_a(1, 0, 1, 0)             # state0 = (1<<32 | 1) | 1
+    s = (1 << 32) | 1
+    s ^= s >> 12
+    s = (s ^ (s << 25)) & ((1 << 64) - 1)
+    s ^= s >> 27
+    bits = ((s * 0x2545F4914F6CDD1D) & ((1 << 64) - 1)) >> 40
+    assert a[0, 0] == np.float32((np.float32(bits) / np.float32(1 << 24)) * 2 - 1)   # bound = 1 for in_dim 1
+    assert first_bits == 0x47E4CE        # top 24 bits of the textbook first output 0x47E4CE4B896CDD1D
+    a = rs.lora_init_a(960, 320, 8, rs.lora_seed(3, "k_proj"))
+    bound = 1.0 / math.sqrt(960)
+    assert a.shape == (960, 8) and np.all(np.abs(a) <= bound) and abs(float(a.mean())) < 0.05 * bound
+    assert abs(float(a.std()) - bound / math.sqrt(3)) < 0.03 * bound          # uniform: sigma = bound / sqrt 3
+    assert np.linalg.matrix_rank(a.astype(np.float64)) == 8
+    b = rs.lora_init_a(960, 320, 8, rs.lora_seed(4, "k_proj"))
+    c = rs.lora_init_a(960, 960, 8, rs.lora_seed(3, "k_proj"))
+    assert not np.array_equal(a, b) and not np.array_equal(a, c)
+    np.testing.assert_array_equal(a, rs.lora_init_a(960, 320, 8, rs.lora_seed(3, "k_proj")))
