@@ -43,7 +43,9 @@ WORKLOADS = {
                  label="SmolLM2-135M-shaped LoRA step, 8x256 (BASELINE.json configs[2])"),
     "1.7b": dict(layers=24, hidden=2048, heads=32, kv=32, ffn=8192, vocab=49152, B=8, S=1024, rank=16, alpha=32.0,
                  targets=("q_proj", "k_proj", "v_proj", "o_proj", "gate_proj", "up_proj", "down_proj"),
-                 prompt=(64, 512), label="SmolLM2-1.7B-shaped LoRA step, 8x1024 (BASELINE.json configs[4])"),
+                 prompt=(64, 512), checkpoint=True,
+                 label="SmolLM2-1.7B-shaped LoRA step, 8x1024, per-layer activation checkpointing "
+                       "(BASELINE.json configs[4])"),
     "tiny": dict(layers=2, hidden=64, heads=4, kv=2, ffn=128, vocab=256, B=2, S=32, rank=4, alpha=8.0,
                  targets=("q_proj", "k_proj", "v_proj", "o_proj"), prompt=(4, 8), label="tiny Llama (plumbing check)"),
 }
@@ -200,7 +202,8 @@ def main():
     ctx = HipContext(0)
     cfg = ModelConfig(vocab_size=w["vocab"], hidden_size=w["hidden"], intermediate_size=w["ffn"],
                       num_hidden_layers=w["layers"], num_attention_heads=w["heads"], num_key_value_heads=w["kv"],
-                      rms_norm_eps=1e-5, rope_theta=100000.0, tie_word_embeddings=True, f16_linears=True)
+                      rms_norm_eps=1e-5, rope_theta=100000.0, tie_word_embeddings=True, f16_linears=True,
+                      checkpoint_blocks=bool(w.get("checkpoint", False)))
     model = Lfm2Model(ctx, cfg)
     for name, value in synthetic_tensors(w):
         model.set_tensor(name, value)
@@ -246,7 +249,8 @@ def main():
         print("sum of kernel event time: %.3f ms/step; wall %.3f ms/step" % (kernel_ms, ms_per_step), file=sys.stderr)
 
     out = {
-        "metric": "LoRA train tokens/s at SmolLM2-360M shape, seq256x8; % FP32 MFMA peak",
+        "metric": ("LoRA train tokens/s at SmolLM2-360M shape, seq256x8; % FP32 MFMA peak" if args.workload == "360m"
+                   else "LoRA train tokens/s, workload %s; %% FP32 MFMA peak" % args.workload),
         "value": value, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",

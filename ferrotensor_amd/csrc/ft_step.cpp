@@ -153,9 +153,22 @@ int ensure_workspace(ft_model* m, size_t B, size_t S) {
     const size_t D = m->head_dim(), QD = c.num_attention_heads * D, KD = c.num_key_value_heads * D;
     size_t rmax = m->lm_head.r;
     m->acts.resize(c.num_hidden_layers);
+    // Block checkpointing (Lfm2Model::with_block_checkpointing, lfm.rs:338-355): only each
+    // block's input is kept; every block shares one set of internal buffers, refilled by
+    // recomputing the block's forward right before its backward.
+    const bool ckpt = c.checkpoint_blocks != 0 && c.num_hidden_layers > 0;
+    LayerActs shared{};
+    for (size_t l = 0; l < c.num_hidden_layers; l++)
+        for (int i = 0; i < 7; i++)
+            if (m->layers[l].all[i]->r > rmax) rmax = m->layers[l].all[i]->r;
     for (size_t l = 0; l < c.num_hidden_layers; l++) {
         LayerActs& a = m->acts[l];
         Layer& L = m->layers[l];
+        if (ckpt && l > 0) {
+            a = shared;
+            FT_TRY(ws_alloc(m, T * H, &a.x));
+            continue;
+        }
         FT_TRY(ws_alloc(m, T * H, &a.x));
         FT_TRY(ws_alloc(m, T * H, &a.h1));
         FT_TRY(ws_alloc(m, T * QD, &a.q));
@@ -171,11 +184,13 @@ int ensure_workspace(ft_model* m, size_t B, size_t S) {
         float** ts[7] = {&a.tq, &a.tk, &a.tv, &a.to, &a.tgate, &a.tup, &a.tdown};
         for (int i = 0; i < 7; i++) {
             *ts[i] = nullptr;
-            if (L.all[i]->has_lora()) {
+            if (ckpt) {
+                if (rmax > 0) FT_TRY(ws_alloc(m, T * rmax, ts[i]));  // any layer may have an adapter here
+            } else if (L.all[i]->has_lora()) {
                 FT_TRY(ws_alloc(m, T * L.all[i]->r, ts[i]));
-                if (L.all[i]->r > rmax) rmax = L.all[i]->r;
             }
         }
+        if (ckpt) shared = a;
     }
     FT_TRY(ws_alloc(m, T * H, &m->x_final));
     FT_TRY(ws_alloc(m, T * H, &m->hf));
@@ -374,26 +389,15 @@ int linear_backward_group(ft_model* m, LinearW* const* ls, const float* const* t
     return FT_OK;
 }
 
-int model_forward(ft_model* m, const uint32_t* rows_host, size_t B, size_t S) {
+// One transformer block: acts[l].x -> acts[l + 1].x (or x_final), filling acts[l].
+int layer_forward(ft_model* m, size_t l, size_t B, size_t S) {
     ft_context* ctx = m->ctx;
     const ft_model_config& c = m->cfg;
-    FT_CHECK_ARG(m->embed && m->norm_f && m->lm_head.w, "model is missing embed_tokens, norm or lm_head weights");
-    for (auto& L : m->layers) {
-        FT_CHECK_ARG(L.norm1 && L.norm2, "a layer is missing its norm weights");
-        for (auto* l : L.all) FT_CHECK_ARG(l->w, "linear %s has no weight", l->prefix.c_str());
-    }
-    if (m->params_dirty) {
-        rebuild_params(m);
-        ws_free(m);
-    }
-    FT_TRY(ensure_workspace(m, B, S));
     const size_t T = B * S, H = c.hidden_size, F = c.intermediate_size;
     const size_t D = m->head_dim(), nh = c.num_attention_heads, nkv = c.num_key_value_heads;
-    FT_TRY(ft_upload(ctx, m->ids_dev, rows_host, T * sizeof(uint32_t)));
-    FT_TRY(ft_embedding(ctx, m->embed, c.vocab_size, H, m->ids_dev, T, m->acts.empty() ? m->x_final : m->acts[0].x));
     ft_attention_options opts{};
     opts.causal = 1;
-    for (size_t l = 0; l < m->layers.size(); l++) {
+    {
         Layer& L = m->layers[l];
         LayerActs& a = m->acts[l];
         float* x_next = l + 1 < m->layers.size() ? m->acts[l + 1].x : m->x_final;
@@ -435,6 +439,29 @@ int model_forward(ft_model* m, const uint32_t* rows_host, size_t B, size_t S) {
         }
         FT_TRY(linear_forward(ctx, L.down, a.act, a.tdown, x_next, T, a.h));
     }
+    return FT_OK;
+}
+
+int model_forward(ft_model* m, const uint32_t* rows_host, size_t B, size_t S) {
+    ft_context* ctx = m->ctx;
+    const ft_model_config& c = m->cfg;
+    FT_CHECK_ARG(m->embed && m->norm_f && m->lm_head.w, "model is missing embed_tokens, norm or lm_head weights");
+    for (auto& L : m->layers) {
+        FT_CHECK_ARG(L.norm1 && L.norm2, "a layer is missing its norm weights");
+        for (auto* l : L.all) FT_CHECK_ARG(l->w, "linear %s has no weight", l->prefix.c_str());
+    }
+    if (m->params_dirty) {
+        rebuild_params(m);
+        ws_free(m);
+    }
+    FT_TRY(ensure_workspace(m, B, S));
+    const size_t T = B * S, H = c.hidden_size, F = c.intermediate_size;
+    const size_t D = m->head_dim(), nh = c.num_attention_heads, nkv = c.num_key_value_heads;
+    FT_TRY(ft_upload(ctx, m->ids_dev, rows_host, T * sizeof(uint32_t)));
+    FT_TRY(ft_embedding(ctx, m->embed, c.vocab_size, H, m->ids_dev, T, m->acts.empty() ? m->x_final : m->acts[0].x));
+    ft_attention_options opts{};
+    opts.causal = 1;
+    for (size_t l = 0; l < m->layers.size(); l++) FT_TRY(layer_forward(m, l, B, S));
     FT_TRY(ft_rms_norm_eps(ctx, m->x_final, m->norm_f, m->hf, T, H, c.rms_norm_eps));
     FT_TRY(linear_forward(ctx, m->lm_head, m->hf, m->thead, m->logits, T));
     return FT_OK;
@@ -456,6 +483,13 @@ int model_backward(ft_model* m, size_t B, size_t S, bool accumulate) {
     for (size_t li = m->layers.size(); li-- > 0;) {
         Layer& L = m->layers[li];
         LayerActs& a = m->acts[li];
+        if (c.checkpoint_blocks && li + 1 < m->layers.size()) {
+            // The shared block buffers hold the next block's internals, which its factor gradients
+            // (side stream) may still be reading: wait, then recompute this block's forward. (The
+            // last block's internals are still there from the forward pass.)
+            FT_TRY(ft_side_join(ctx, 0));
+            FT_TRY(layer_forward(m, li, B, S));
+        }
         // x_next = h + down(silu(gate) * up)
         if (!L.down.has_lora()) {
             FT_TRY(ft_mlp_down_backward(ctx, g, L.down.w, L.down.dtype, a.gate, a.up, m->d_gate, m->d_up, m->d_act, T,

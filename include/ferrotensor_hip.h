@@ -329,6 +329,9 @@ typedef struct ft_model_config {
     float rms_norm_eps, rope_theta;
     int32_t tie_word_embeddings;
     int32_t f16_linears;   /* frozen linear weights stored as f16 (CLI default, main.rs:230-234) */
+    /* Lfm2Model::with_block_checkpointing (lfm.rs:338-355): keep only each block's input
+     * during training and recompute the block in backward (one extra forward per block). */
+    int32_t checkpoint_blocks;
 } ft_model_config;
 
 typedef struct ft_model ft_model;

@@ -232,6 +232,38 @@ def test_fresh_adapters_are_seeded_like_the_builder(ctx):
     assert all(after[n].any() for n in after if n.endswith(".lora_b"))
 
 
+def test_block_checkpointing_changes_no_bit(ctx):
+    """Recomputing a block in backward runs the same kernels on the same inputs: loss, gradients and
+    updated weights are identical to the plain step (ferrotensor-graph/tests/block_checkpointing.rs)."""
+    import dataclasses
+    from ferrotensor_amd.trainer import Trainer
+    mods = ["q_proj", "k_proj", "v_proj", "o_proj", "gate_proj", "up_proj", "down_proj"]
+    rng = np.random.default_rng(8)
+    rows = rng.integers(0, 256, (2, 32)).astype(np.uint32)
+    targets = np.concatenate([rows[:, 1:], rows[:, :1]], axis=1)
+    masks = (rng.random((2, 32)) > 0.3).astype(np.uint8)
+    results = []
+    for ckpt in (False, True):
+        cfg = dataclasses.replace(tiny_config(True, True), checkpoint_blocks=ckpt, num_hidden_layers=3)
+        hip, _ = build_pair(ctx, cfg, mods, rank=4, alpha=8.0, seed=17)
+        tr = Trainer(hip, lr=1e-3, weight_decay=0.0, clip_grad_norm=1.0)
+        losses = []
+        for _ in range(2):
+            st0 = tr.train_chunk(rows, targets, masks, apply=False)
+            grads = hip.grads()
+            st = tr.train_chunk(rows, targets, masks)
+            losses.append((st0.loss, st.loss, st.grad_norm))
+        results.append((losses, grads, hip.params()))
+        tr.close()
+        hip.close()
+    (l0, g0, p0), (l1, g1, p1) = results
+    assert l0 == l1
+    for n in g0:
+        np.testing.assert_array_equal(g0[n], g1[n])
+    for n in p0:
+        np.testing.assert_array_equal(p0[n], p1[n])
+
+
 def test_targets_masking_is_bit_exact_against_oracle(ctx):
     """Skipped rows (mask 0 or target >= vocab) contribute exactly nothing:
     the loss equals the oracle's and flipping masked targets changes no bit."""
