@@ -130,6 +130,10 @@ SIGNATURES = {
     "ft_model_forward_logits": [_P, _P, _SZ, _SZ, _P],
     "ft_trainer_create": [_P, C.POINTER(TrainerConfigC), C.POINTER(_P)],
     "ft_trainer_destroy": [_P],
+    "ft_trainer_read_moments": [_P, _SZ, _P, _P],
+    "ft_trainer_write_moments": [_P, _SZ, _P, _P],
+    "ft_trainer_get_adam_t": [_P, C.POINTER(_F)],
+    "ft_trainer_set_adam_t": [_P, _F],
     "ft_trainer_optimizer_steps": [_P, C.POINTER(_SZ)],
     "ft_trainer_set_optimizer_steps": [_P, _SZ],
     "ft_lora_seed": [C.c_uint64, C.c_char_p],

@@ -880,6 +880,34 @@ int ft_trainer_optimizer_steps(ft_trainer* t, size_t* steps) {
     return FT_OK;
 }
 
+int ft_trainer_read_moments(ft_trainer* t, size_t index, float* m_host, float* v_host) {
+    FT_CHECK_ARG(t && m_host && v_host, "ft_trainer_read_moments: NULL argument");
+    FT_CHECK_ARG(index < t->m.size(), "ft_trainer_read_moments: index %zu of %zu", index, t->m.size());
+    const size_t bytes = t->model->params[index].n * sizeof(float);
+    FT_TRY(ft_download(t->model->ctx, m_host, t->m[index], bytes));
+    return ft_download(t->model->ctx, v_host, t->v[index], bytes);
+}
+
+int ft_trainer_write_moments(ft_trainer* t, size_t index, const float* m_host, const float* v_host) {
+    FT_CHECK_ARG(t && m_host && v_host, "ft_trainer_write_moments: NULL argument");
+    FT_CHECK_ARG(index < t->m.size(), "ft_trainer_write_moments: index %zu of %zu", index, t->m.size());
+    const size_t bytes = t->model->params[index].n * sizeof(float);
+    FT_TRY(ft_upload(t->model->ctx, t->m[index], m_host, bytes));
+    return ft_upload(t->model->ctx, t->v[index], v_host, bytes);
+}
+
+int ft_trainer_get_adam_t(ft_trainer* t, float* steps) {
+    FT_CHECK_ARG(t && steps, "ft_trainer_get_adam_t: NULL argument");
+    *steps = t->t;
+    return FT_OK;
+}
+
+int ft_trainer_set_adam_t(ft_trainer* t, float steps) {
+    FT_CHECK_ARG(t && steps >= 0.0f, "ft_trainer_set_adam_t: bad argument");
+    t->t = steps;
+    return FT_OK;
+}
+
 int ft_trainer_set_optimizer_steps(ft_trainer* t, size_t steps) {
     FT_CHECK_ARG(t, "ft_trainer_set_optimizer_steps: NULL argument");
     t->optimizer_steps = steps;

@@ -214,6 +214,7 @@ class Trainer:
         self.model = model
         self.length_bucket = length_bucket
         self._lib = model._lib
+        self.hyper = dict(lr=lr, beta1=beta1, beta2=beta2, eps=eps, weight_decay=weight_decay)
         kind = LR_SCHEDULES[lr_schedule]
         cfg = _lib.TrainerConfigC(lr, beta1, beta2, eps, weight_decay,
                                   clip_grad_norm if clip_grad_norm else 0.0, grad_accum_steps,

@@ -414,6 +414,13 @@ int ft_trainer_create(ft_model* m, const ft_trainer_config* cfg, ft_trainer** ou
 int ft_trainer_destroy(ft_trainer* t);
 /* Trainer::optimizer_steps / set_optimizer_steps (trainer/src/lib.rs:199-213): the
  * number of optimizer steps taken; setting it (resume) also advances the schedule. */
+/* AdamW::state / load_state (autograd/src/lib.rs:1554-1640): the first and second
+ * moments of trainable tensor `index` (the order of ft_model_param_info) to / from
+ * host memory, and the optimizer's f32 step counter `t`. */
+int ft_trainer_read_moments(ft_trainer* t, size_t index, float* m_host, float* v_host);
+int ft_trainer_write_moments(ft_trainer* t, size_t index, const float* m_host, const float* v_host);
+int ft_trainer_get_adam_t(ft_trainer* t, float* steps);
+int ft_trainer_set_adam_t(ft_trainer* t, float steps);
 int ft_trainer_optimizer_steps(ft_trainer* t, size_t* steps);
 int ft_trainer_set_optimizer_steps(ft_trainer* t, size_t steps);
 /* Trainer::train_chunk (trainer/src/lib.rs:426-502) for B equally long rows

@@ -264,6 +264,52 @@ def test_block_checkpointing_changes_no_bit(ctx):
         np.testing.assert_array_equal(p0[n], p1[n])
 
 
+def test_resume_from_adapter_and_state_files_is_bit_identical(ctx, tmp_path):
+    """3 steps straight through == 2 steps, save (adapter file + training checkpoint), fresh model and
+    trainer, load, 1 step: weights, moments and the schedule all continue where they stopped."""
+    from ferrotensor_amd import checkpoint as ck
+    from ferrotensor_amd.trainer import Trainer
+    cfg = tiny_config(True, True)
+    mods = ["q_proj", "k_proj", "v_proj", "o_proj"]
+    rng = np.random.default_rng(12)
+    rows = rng.integers(0, 256, (2, 16)).astype(np.uint32)
+    targets = np.concatenate([rows[:, 1:], rows[:, :1]], axis=1)
+    masks = np.ones((2, 16), np.uint8)
+    kw = dict(lr=1e-3, weight_decay=0.01, clip_grad_norm=1.0, lr_schedule="warmup_cosine", warmup_steps=2,
+              total_steps=5, min_lr=1e-4)
+
+    hip, _ = build_pair(ctx, cfg, mods, rank=4, alpha=8.0, seed=19)
+    tr = Trainer(hip, **kw)
+    straight = [tr.train_chunk(rows, targets, masks) for _ in range(3)]
+    want = hip.params()
+
+    hip2, _ = build_pair(ctx, cfg, mods, rank=4, alpha=8.0, seed=19)
+    tr2 = Trainer(hip2, **kw)
+    for _ in range(2):
+        tr2.train_chunk(rows, targets, masks)
+    adapter, state_path = str(tmp_path / "adapter.safetensors"), str(tmp_path / "run.state.json")
+    ck.save_lora_checkpoint(hip2, adapter, ck.LoraMetadata(4, 8.0, mods))
+    ck.save_training_checkpoint(state_path, ck.TrainingState(step=tr2.optimizer_steps, total_steps=5, lr=1e-3),
+                                ck.optimizer_state(tr2))
+    tr2.close()
+    hip2.close()
+
+    hip3, _ = build_pair(ctx, cfg, [], rank=4, alpha=8.0, seed=19)        # base weights only
+    loaded = ck.load_lora_checkpoint(adapter)
+    assert loaded.metadata == ck.LoraMetadata(4, 8.0, mods) and len(loaded.tensors) == 2 * 4 * cfg.num_hidden_layers
+    assert "model.layers.1.self_attn.o_proj.lora_B.weight" in loaded.tensors
+    assert ck.apply_lora_checkpoint(hip3, loaded) == 4 * cfg.num_hidden_layers
+    tr3 = Trainer(hip3, **kw)
+    state, adam = ck.load_training_checkpoint(state_path)
+    assert state.step == 2 and adam.t == 2.0
+    assert ck.restore_optimizer(tr3, adam, state.step) == 2 * 4 * cfg.num_hidden_layers
+    st = tr3.train_chunk(rows, targets, masks)
+    assert (st.loss, st.grad_norm, st.lr) == (straight[2].loss, straight[2].grad_norm, straight[2].lr)
+    got = hip3.params()
+    for n in want:
+        np.testing.assert_array_equal(got[n], want[n])
+
+
 def test_targets_masking_is_bit_exact_against_oracle(ctx):
     """Skipped rows (mask 0 or target >= vocab) contribute exactly nothing:
     the loss equals the oracle's and flipping masked targets changes no bit."""
