@@ -70,6 +70,31 @@ def test_base_logits_without_adapters(ctx, fx):
     assert worst_ratio(m.forward_batch(rows), fx.expected["logits.base"], atol=1e-4, rtol=0.0) <= 1.0
 
 
+def test_model_directory_loader_and_adapter_file_reproduce_the_fixture(ctx, fx, golden_dir, tmp_path):
+    """The reference's fixture directory through the file path a user takes: `load_model` (config.json +
+    model.safetensors, f32 linears as the fixture was made), adapters converted to an adapter file and
+    applied with `apply_lora_checkpoint` -> the PyTorch golden logits and gradients."""
+    import os
+    from ferrotensor_amd import checkpoint as ck
+    from ferrotensor_amd import loader
+    from ferrotensor_amd.trainer import Trainer
+    model = loader.load_model(ctx, os.path.join(golden_dir, "gradient_parity"), f16_linears=False)
+    rows, targets, masks, _, want_loss = fx.case("batch")
+    assert worst_ratio(model.forward_batch(fx.case("single")[0]), fx.expected["logits.base"], atol=1e-4,
+                       rtol=0.0) <= 1.0
+    # the fixture names its adapters <prefix>.lora_a / .lora_b; the adapter file uses lora_A.weight / lora_B.weight
+    tensors = {ck.file_name(n): v for n, v in fx.adapters.items()}
+    path = str(tmp_path / "fixture_adapter.safetensors")
+    ck.write_safetensors(path, tensors, ck.LoraMetadata(4, fx.meta["lora_alpha"], ["all"]).to_map())
+    assert ck.apply_lora_checkpoint(model, ck.load_lora_checkpoint(path)) == 15
+    assert worst_ratio(model.forward_batch(rows), fx.expected["logits.batch"]) <= 1.0
+    st = Trainer(model, lr=1e-3, grad_accum_steps=1).train_chunk(rows, targets, masks, apply=False)
+    assert worst_ratio([st.loss], [want_loss]) <= 1.0
+    want = fx.expected_grads("batch")
+    grads = model.grads()
+    assert max(worst_ratio(grads[n], want[n]) for n in want) <= 1.0
+
+
 def test_padding_to_bucket_changes_nothing(ctx, fx):
     """Rows padded to 32 with their last token and mask 0 (trainer/src/lib.rs:431-450)."""
     from ferrotensor_amd.trainer import Trainer
