@@ -187,6 +187,9 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="360m", choices=sorted(WORKLOADS))
+    ap.add_argument("--micro-batch", type=int, default=0,
+                    help="sequences per forward/backward pass (default: the whole batch); gradients accumulate "
+                         "over the batch and one optimizer step follows, as `ferrotensor train --batch m --accum B/m`")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--breakdown", action="store_true", help="print the per-kernel event-time table to stderr")
     args = ap.parse_args()
@@ -210,15 +213,25 @@ def main():
     for name, a, b in lora_factors(model, w):
         model.set_lora(name, a, b, w["alpha"])
     # CLI defaults of `ferrotensor train`: lr 2e-4, weight decay 0, clip 1.0, accumulation = batch.
-    trainer = Trainer(model, lr=2e-4, weight_decay=0.0, clip_grad_norm=1.0)
     rows, targets, masks = synthetic_batch(w)
+    mb = args.micro_batch or w["B"]
+    if w["B"] % mb:
+        sys.exit("bench.py: --micro-batch must divide the batch of %d sequences" % w["B"])
+    # --micro-batch m: the reference's `--batch m --accum B/m` regime, one optimizer step per B sequences.
+    trainer = Trainer(model, lr=2e-4, weight_decay=0.0, clip_grad_norm=1.0, grad_accum_steps=w["B"])
+
+    def one_step():
+        st = None
+        for i in range(0, w["B"], mb):
+            st = trainer.train_chunk(rows[i:i + mb], targets[i:i + mb], masks[i:i + mb])
+        return st
 
     for _ in range(args.warmup):
-        st = trainer.train_chunk(rows, targets, masks)
+        st = one_step()
     ctx.synchronize()
     t0 = time.perf_counter()
     for _ in range(args.steps):
-        st = trainer.train_chunk(rows, targets, masks)
+        st = one_step()
     ctx.synchronize()
     elapsed = time.perf_counter() - t0
     ms_per_step = elapsed / args.steps * 1e3
@@ -231,7 +244,7 @@ def main():
     from ferrotensor_amd._lib import check
     check(ctx._lib.ft_profile_begin(ctx.handle))
     for _ in range(args.steps):
-        trainer.train_chunk(rows, targets, masks)
+        one_step()
     prof = read_profile(ctx)
     gemms = [r for r in prof if r["name"].startswith("gemm_")]
     dom = gemms[0]
@@ -254,7 +267,7 @@ def main():
         "value": value, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
-        "config": {"workload": w["label"], "global_batch": w["B"], "seq_len": w["S"],
+        "config": {"workload": w["label"], "global_batch": w["B"], "seq_len": w["S"], "micro_batch": mb,
                    "lora": "rank %d alpha %g on %s" % (w["rank"], w["alpha"], "/".join(w["targets"])),
                    "base_weights": "f16 storage, f32 arithmetic", "optimizer": "AdamW lr 2e-4 wd 0 clip 1.0",
                    "supervised_tokens": int(st.tokens), "loss": float(st.loss)},

@@ -27,6 +27,8 @@ struct ft_context {
 
     // Partial sums of the sliced thin products (LoRA dA, dB); allocated on first use.
     float* thin_scratch = nullptr;
+    // Partial tiles of split-K GEMMs (few output tiles, long K); allocated on first use.
+    float* gemm_scratch = nullptr;
 
     // Extra streams ("lanes") for work that can run beside the main stream:
     // lane 0 carries the LoRA factor gradients of a training step (only the

@@ -578,13 +578,19 @@ struct AsyncProb {
     const float* e1;
     const float* e2;
     int N, ldc, tiles_n, tile_begin, nseg;
+    long partial_off;  // split-K: this product's slice of AsyncBatch::partial, [splits][M][N]
 };
 
 constexpr int kEpiPlain = 0, kEpiGateUp = 1, kEpiSiluBwd = 2;
 
+// Split-K (few tiles, e.g. one sequence per pass: M = 256): blockIdx.y takes a
+// contiguous share of the K tiles and writes its partial tile to `partial`;
+// splitk_reduce_kernel adds the shares in order (and the residual) into `out`.
 struct AsyncBatch {
     AsyncProb p[kAsyncMaxProb];
     int count, M;
+    int splits;        // 1 = none
+    float* partial;
 };
 
 template <int NSEG, typename T>
@@ -592,6 +598,32 @@ __device__ __forceinline__ T seg_pick(const T (&v)[NSEG], int s) {
     if constexpr (NSEG == 1) return v[0];
     else if constexpr (NSEG == 2) return s == 0 ? v[0] : v[1];
     else return s == 0 ? v[0] : (s == 1 ? v[1] : v[2]);
+}
+
+// out = (add +) sum over the K shares, in share order. One thread per 4 outputs;
+// blockIdx.y = product of the batch.
+struct SplitReduceArgs {
+    const float* partial[kAsyncMaxProb];
+    const float* add[kAsyncMaxProb];
+    float* out[kAsyncMaxProb];
+    long n4[kAsyncMaxProb];  // M * N / 4
+    int splits;
+};
+
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(SplitReduceArgs a) {
+    const int pi = blockIdx.y;
+    const long i = (long)blockIdx.x * 256 + threadIdx.x;
+    if (i >= a.n4[pi]) return;
+    const float4* src = reinterpret_cast<const float4*>(a.partial[pi]) + i;
+    float4 v = a.add[pi] ? reinterpret_cast<const float4*>(a.add[pi])[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int s = 0; s < a.splits; s++) {
+        const float4 t = src[(long)s * a.n4[pi]];
+        v.x += t.x;
+        v.y += t.y;
+        v.z += t.z;
+        v.w += t.w;
+    }
+    reinterpret_cast<float4*>(a.out[pi])[i] = v;
 }
 
 template <int BM, int BN, int WM, int WN, int LAYOUT, int NSEG, int EPI = kEpiPlain>
@@ -656,7 +688,15 @@ __global__ __launch_bounds__(256) void gemm_async_kernel(AsyncBatch g) {
         has_ext[s] = NB == 1 && s < p.nseg && sg.a2 != nullptr;
     }
     const char* balt = reinterpret_cast<const char*>(p.b_alt);
-    const int nt = tend[NSEG - 1];
+    // This workgroup's share of the K tiles: [t0, nt).
+    const int nt_all = tend[NSEG - 1];
+    const int split = (int)blockIdx.y;
+    const int t0 = (int)(((long)nt_all * split) / g.splits);
+    const int nt = (int)(((long)nt_all * (split + 1)) / g.splits);
+    if (split > 0) {
+#pragma unroll
+        for (int s = 0; s < NSEG; s++) has_ext[s] = false;  // the rank-r term is added once, by share 0
+    }
 
     // The rank-r products' operands: ordinary loads, issued first, consumed last.
     ExA xa[NSEG];
@@ -798,10 +838,10 @@ __global__ __launch_bounds__(256) void gemm_async_kernel(AsyncBatch g) {
         }
     };
 
-    // Prologue: tiles 0 .. NST-2 in flight.
-    issue(0, St0);
-    issue(1, St1);
-    for (int t = 0; t < nt; t += NST) {
+    // Prologue: tiles t0 .. t0+NST-2 in flight.
+    issue(t0, St0);
+    issue(t0 + 1, St1);
+    for (int t = t0; t < nt; t += NST) {
         iter(t, St0, St2);
         if (t + 1 < nt) iter(t + 1, St1, St0);
         if (t + 2 < nt) iter(t + 2, St2, St1);
@@ -841,7 +881,9 @@ __global__ __launch_bounds__(256) void gemm_async_kernel(AsyncBatch g) {
                 const int row = m0 + wm0 + i * 32 + (r / 4) * 8 + half * 4 + (r % 4);
                 if (row < M) {
                     const long o = (long)row * p.ldc + col;
-                    if constexpr (EPI == kEpiGateUp) {
+                    if (EPI == kEpiPlain && g.splits > 1) {
+                        g.partial[p.partial_off + ((long)split * M + row) * p.N + col] = acc[i][j][r];
+                    } else if constexpr (EPI == kEpiGateUp) {
                         const float up = acc[i][j][r], x = acc[i][FN + j][r];
                         p.out[o] = up;
                         p.out2[o] = x;
@@ -967,6 +1009,8 @@ __global__ __launch_bounds__(256) void skinny_kernel(const float* __restrict__ x
 // Host side
 // ---------------------------------------------------------------------------
 
+constexpr size_t kSplitScratchFloats = (size_t)16 << 20;  // 64 MiB of split-K partial tiles
+
 template <int BM, int BN, int WM, int WN>
 int launch_async(ft_context* ctx, AsyncBatch g, int layout, int epi = kEpiPlain) {
     const int tiles_m = (g.M + BM - 1) / BM;
@@ -985,7 +1029,56 @@ int launch_async(ft_context* ctx, AsyncBatch g, int layout, int epi = kEpiPlain)
         }
         bytes += (p.add ? 8.0 : 4.0) * g.M * (double)p.N;
     }
-    const dim3 grid((unsigned)tiles);
+    g.splits = 1;
+    g.partial = nullptr;
+    // Split-K when the tiles alone cannot occupy the chip and the K loop is long enough to share
+    // out (at least 4 K tiles per share): aims at about two workgroups per CU.
+    int min_kt = 1 << 30;
+    bool mn4 = true;
+    size_t out_floats = 0;
+    for (int i = 0; i < g.count; i++) {
+        int kt = 0;
+        for (int s = 0; s < g.p[i].nseg; s++) kt += g.p[i].seg[s].nt;
+        if (kt < min_kt) min_kt = kt;
+        mn4 = mn4 && ((size_t)g.M * g.p[i].N) % 4 == 0 && g.p[i].ldc == g.p[i].N;
+        out_floats += (size_t)g.M * g.p[i].N;
+    }
+    if (epi == kEpiPlain && mn4 && tiles > 0 && (size_t)tiles * 2 <= (size_t)ctx->num_cus) {
+        int want = (int)((2 * (size_t)ctx->num_cus + tiles - 1) / tiles);
+        if (want > 8) want = 8;
+        if (want > min_kt / 4) want = min_kt / 4;
+        if (want >= 2 && out_floats * want <= kSplitScratchFloats) {
+            if (!ctx->gemm_scratch) {
+                FT_HIP(hipSetDevice(ctx->device));
+                FT_HIP(hipMalloc((void**)&ctx->gemm_scratch, kSplitScratchFloats * sizeof(float)));
+            }
+            g.splits = want;
+            g.partial = ctx->gemm_scratch;
+            long off = 0;
+            for (int i = 0; i < g.count; i++) {
+                g.p[i].partial_off = off;
+                off += (long)want * g.M * g.p[i].N;
+            }
+        }
+    }
+    const dim3 grid((unsigned)tiles, (unsigned)g.splits);
+    auto reduce_shares = [&]() -> int {
+        if (g.splits == 1) return FT_OK;
+        SplitReduceArgs ra{};
+        long n4max = 0;
+        for (int i = 0; i < g.count; i++) {
+            ra.partial[i] = g.partial + g.p[i].partial_off;
+            ra.add[i] = g.p[i].add;
+            ra.out[i] = g.p[i].out;
+            ra.n4[i] = (long)g.M * g.p[i].N / 4;
+            if (ra.n4[i] > n4max) n4max = ra.n4[i];
+        }
+        ra.splits = g.splits;
+        hipLaunchKernelGGL(splitk_reduce_kernel, dim3(ft_div_up((size_t)n4max, 256), (unsigned)g.count), dim3(256), 0,
+                           ctx->stream, ra);
+        FT_LAUNCH_CHECK();
+        return FT_OK;
+    };
     char name[96];
     if (epi != kEpiPlain) {
         // both fused forms: one product, one segment, 64x64 tiles (the only instantiation)
@@ -1025,7 +1118,7 @@ int launch_async(ft_context* ctx, AsyncBatch g, int layout, int epi = kEpiPlain)
                                ctx->stream, g);
     }
     FT_LAUNCH_CHECK();
-    return FT_OK;
+    return reduce_shares();
 }
 
 // Tile choice, from measurements of the whole step on MI355X at M = 2048: 128x128

@@ -302,26 +302,26 @@ int linear_backward(ft_model* m, LinearW& l, const float* x, const float* t, con
     if (l.has_lora()) {
         FT_TRY(ft_side_join(ctx, 0));  // factor gradients still in flight read m->dt
         FT_TRY(ft_lora_grad_down(ctx, dy, l.b, m->dt, T, l.out, l.r, l.scale()));
-        if (accumulate) {
+        // dB = t^T dy and dA = x^T dt in one sliced launch when possible (added to the
+        // gradients of the earlier micro-batches when `accumulate`).
+        const int acc = accumulate ? 1 : 0;
+        ft_thin_problem pb[2] = {
+            {dy, t, l.gb, (int)T, 0, (int)l.out, (int)l.r, (long)l.out, (long)l.r, (long)l.out, 1.0f, 0, 1, 0, acc},
+            {x, m->dt, l.ga, (int)T, 0, (int)l.in, (int)l.r, (long)l.in, (long)l.r, (long)l.r, 1.0f, 0, 0, 0, acc}};
+        if (ft_thin_colwise_ok(pb[0]) && ft_thin_colwise_ok(pb[1])) {
+            // Only the optimizer reads dA and dB: they run beside the input-gradient GEMM.
+            FT_TRY(ft_side_begin(ctx));
+            const int rc = ft_thin_colwise(ctx, pb, 2);
+            FT_TRY(ft_side_end(ctx));
+            FT_TRY(rc);
+        } else if (accumulate) {
             FT_TRY(ft_lora_grad_b(ctx, t, dy, m->gtmp, T, l.out, l.r));
             FT_TRY(ft_gradient_accumulate(ctx, l.gb, m->gtmp, l.r * l.out));
             FT_TRY(ft_lora_grad_a(ctx, x, m->dt, m->gtmp, T, l.in, l.r));
             FT_TRY(ft_gradient_accumulate(ctx, l.ga, m->gtmp, l.in * l.r));
         } else {
-            // dB = t^T dy and dA = x^T dt in one sliced launch when possible.
-            ft_thin_problem pb[2] = {
-                {dy, t, l.gb, (int)T, 0, (int)l.out, (int)l.r, (long)l.out, (long)l.r, (long)l.out, 1.0f, 0, 1, 0},
-                {x, m->dt, l.ga, (int)T, 0, (int)l.in, (int)l.r, (long)l.in, (long)l.r, (long)l.r, 1.0f, 0, 0, 0}};
-            if (ft_thin_colwise_ok(pb[0]) && ft_thin_colwise_ok(pb[1])) {
-                // Only the optimizer reads dA and dB: they run beside the input-gradient GEMM.
-                FT_TRY(ft_side_begin(ctx));
-                const int rc = ft_thin_colwise(ctx, pb, 2);
-                FT_TRY(ft_side_end(ctx));
-                FT_TRY(rc);
-            } else {
-                FT_TRY(ft_lora_grad_b(ctx, t, dy, l.gb, T, l.out, l.r));
-                FT_TRY(ft_lora_grad_a(ctx, x, m->dt, l.ga, T, l.in, l.r));
-            }
+            FT_TRY(ft_lora_grad_b(ctx, t, dy, l.gb, T, l.out, l.r));
+            FT_TRY(ft_lora_grad_a(ctx, x, m->dt, l.ga, T, l.in, l.r));
         }
         if (dx)
             FT_TRY(ft_lora_linear_dx(ctx, dy, l.w, l.dtype, m->dt, l.a, dx_add ? dx : nullptr, dx, T, l.in, l.out,
@@ -337,12 +337,13 @@ int linear_backward(ft_model* m, LinearW& l, const float* x, const float* t, con
 // dT, dA and dB products of all of them go into two batched launches. The input
 // gradients are summed into dx (NULL: not wanted) by one GEMM whose K loop runs
 // over all the output gradients. Falls back to one linear at a time when the
-// adapters cannot be batched or gradients are being accumulated.
+// adapters cannot be batched.
 int linear_backward_group(ft_model* m, LinearW* const* ls, const float* const* ts, const float* const* dys,
                           float* dx, int n, const float* x, size_t T, bool accumulate) {
     ft_context* ctx = m->ctx;
     float* dts[3] = {m->dt, m->dt2, m->dt3};
-    bool batch = !accumulate && n <= 3;
+    bool batch = n <= 3;
+    const int acc = accumulate ? 1 : 0;
     ft_thin_problem rows[3], cols[6];
     for (int i = 0; i < n && batch; i++) {
         const LinearW& l = *ls[i];
@@ -353,9 +354,9 @@ int linear_backward_group(ft_model* m, LinearW* const* ls, const float* const* t
         rows[i] = ft_thin_problem{dys[i], l.b, dts[i], (int)T, (int)l.out, 0, (int)l.r, (long)l.out, (long)l.out,
                                   (long)l.r, l.scale(), 1, 0, 0};
         cols[2 * i] = ft_thin_problem{dys[i], ts[i], l.gb, (int)T, 0, (int)l.out, (int)l.r, (long)l.out, (long)l.r,
-                                      (long)l.out, 1.0f, 0, 1, 0};
+                                      (long)l.out, 1.0f, 0, 1, 0, acc};
         cols[2 * i + 1] = ft_thin_problem{x, dts[i], l.ga, (int)T, 0, (int)l.in, (int)l.r, (long)l.in, (long)l.r,
-                                          (long)l.r, 1.0f, 0, 0, 0};
+                                          (long)l.r, 1.0f, 0, 0, 0, acc};
         batch = ft_thin_rowwise_ok(rows[i]) && ft_thin_colwise_ok(cols[2 * i]) && ft_thin_colwise_ok(cols[2 * i + 1]);
     }
     if (!batch) {

@@ -15,6 +15,7 @@ struct ft_thin_problem {
     int y_transposed;    // row-wise only
     int out_transposed;  // col-wise only
     long scratch_offset; // filled in by ft_thin_colwise
+    int accumulate;      // col-wise only: out += result (gradient accumulation) instead of out = result
 };
 
 bool ft_thin_rank_supported(size_t r);

@@ -170,10 +170,8 @@ __global__ __launch_bounds__(256) void thin_finish_kernel(ThinBatch b, const flo
     }
     for (; s < slices; s++) v += src[(long)s * total];
     const int n = e / p.C, j = e % p.C;
-    if (p.out_transposed)
-        p.out[(long)j * p.ldo + n] = v * p.scale;
-    else
-        p.out[(long)n * p.ldo + j] = v * p.scale;
+    float* o = p.out_transposed ? p.out + (long)j * p.ldo + n : p.out + (long)n * p.ldo + j;
+    *o = p.accumulate ? *o + v * p.scale : v * p.scale;
 }
 
 bool aligned16(const void* q) { return (((uintptr_t)q) & 15) == 0; }

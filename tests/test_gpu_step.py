@@ -335,6 +335,38 @@ def test_resume_from_adapter_and_state_files_is_bit_identical(ctx, tmp_path):
         np.testing.assert_array_equal(got[n], want[n])
 
 
+def test_micro_batches_accumulate_to_the_batched_step(ctx):
+    """`--batch 1 --accum 4` == `--batch 4` (ferrotensor-trainer/tests/gpu_training.rs:127-186): four
+    one-sequence chunks accumulate into the gradients of the four-sequence chunk, and the optimizer
+    steps once, after the last one."""
+    from ferrotensor_amd.trainer import Trainer
+    mods = ["q_proj", "k_proj", "v_proj", "o_proj", "gate_proj", "up_proj", "down_proj"]
+    rng = np.random.default_rng(14)
+    rows = rng.integers(0, 256, (4, 32)).astype(np.uint32)
+    targets = np.concatenate([rows[:, 1:], rows[:, :1]], axis=1)
+    masks = (rng.random((4, 32)) > 0.25).astype(np.uint8)
+    out = []
+    for micro in (4, 1, 2):
+        hip, _ = build_pair(ctx, tiny_config(True, True), mods, rank=4, alpha=8.0, seed=23)
+        tr = Trainer(hip, lr=1e-3, weight_decay=0.0, clip_grad_norm=1.0, grad_accum_steps=4)
+        steps, loss = [], 0.0
+        for i in range(0, 4, micro):
+            st = tr.train_chunk(rows[i:i + micro], targets[i:i + micro], masks[i:i + micro])
+            steps.append(st.optimizer_step)
+            loss += st.loss
+        assert steps == [False] * (4 // micro - 1) + [True] and tr.optimizer_steps == 1
+        out.append((loss, st.grad_norm, hip.grads(), hip.params()))
+        tr.close()
+        hip.close()
+    (l0, n0, g0, p0) = out[0]
+    for (l, n, g, p) in out[1:]:
+        assert_close("loss", [l], [l0])
+        assert_close("grad_norm", [n], [n0])
+        for k in g0:
+            assert_close("grad " + k, g[k], g0[k])
+            assert_close("param " + k, p[k], p0[k], atol=1e-6, rtol=1e-4)
+
+
 def test_targets_masking_is_bit_exact_against_oracle(ctx):
     """Skipped rows (mask 0 or target >= vocab) contribute exactly nothing:
     the loss equals the oracle's and flipping masked targets changes no bit."""
