@@ -128,6 +128,7 @@ SIGNATURES = {
     "ft_model_read_param": [_P, _SZ, _P],
     "ft_model_read_grad": [_P, _SZ, _P],
     "ft_model_forward_logits": [_P, _P, _SZ, _SZ, _P],
+    "ft_model_eval_chunk": [_P, _P, _P, _P, _SZ, _SZ, _P, _P],
     "ft_trainer_create": [_P, C.POINTER(TrainerConfigC), C.POINTER(_P)],
     "ft_trainer_destroy": [_P],
     "ft_trainer_read_moments": [_P, _SZ, _P, _P],

@@ -856,6 +856,80 @@ int ft_trainer_destroy(ft_trainer* t) {
     return FT_OK;
 }
 
+}  // extern "C"
+
+namespace {
+
+// Host half of masked_cross_entropy_batch (trainer/src/lib.rs:689-722): per-row target or
+// MASKED_CE_SKIP, weight 1 / supervised tokens of the row's sequence. Returns the total.
+size_t build_targets(const uint32_t* targets, const uint8_t* loss_mask, size_t B, size_t S, size_t V,
+                     std::vector<uint32_t>& tg, std::vector<float>& wt, std::vector<size_t>& tokens) {
+    const size_t T = B * S;
+    tg.assign(T, FT_MASKED_CE_SKIP);
+    wt.assign(T, 0.0f);
+    tokens.assign(B, 0);
+    auto supervised = [&](size_t r) { return loss_mask[r] != 0 && (size_t)targets[r] < V; };
+    size_t total = 0;
+    for (size_t s = 0; s < B; s++) {
+        for (size_t i = 0; i < S; i++) tokens[s] += supervised(s * S + i) ? 1 : 0;
+        total += tokens[s];
+    }
+    for (size_t r = 0; r < T; r++) {
+        if (supervised(r)) {
+            tg[r] = targets[r];
+            wt[r] = 1.0f / (float)tokens[r / S];
+        }
+    }
+    return total;
+}
+
+// Per-sequence mean losses from the device row losses (f64 sums, as the reference's host code).
+int read_sequence_losses(ft_model* m, size_t B, size_t S, const std::vector<size_t>& tokens, float* per_sequence,
+                         float* total_out) {
+    std::vector<float> losses(B * S);
+    FT_TRY(ft_download(m->ctx, losses.data(), m->row_loss, B * S * sizeof(float)));
+    float total = 0.0f;
+    for (size_t s = 0; s < B; s++) {
+        double sum = 0.0;
+        for (size_t i = 0; i < S; i++) sum += (double)losses[s * S + i];
+        const float mean = (float)(sum / (double)(tokens[s] ? tokens[s] : 1));
+        if (per_sequence) per_sequence[s] = mean;
+        total += mean;
+    }
+    if (total_out) *total_out = total;
+    return FT_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int ft_model_eval_chunk(ft_model* m, const uint32_t* rows, const uint32_t* targets, const uint8_t* loss_mask,
+                        size_t B, size_t S, float* per_sequence_loss, uint32_t* per_sequence_tokens) {
+    return guarded([&]() -> int {
+        FT_CHECK_ARG(m && rows && targets && loss_mask && per_sequence_loss && per_sequence_tokens,
+                     "ft_model_eval_chunk: NULL argument");
+        FT_CHECK_ARG(B > 0 && S > 0, "ft_model_eval_chunk: empty chunk");
+        const size_t T = B * S, V = m->cfg.vocab_size;
+        std::vector<uint32_t> tg;
+        std::vector<float> wt;
+        std::vector<size_t> tokens;
+        const size_t total = build_targets(targets, loss_mask, B, S, V, tg, wt, tokens);
+        for (size_t s = 0; s < B; s++) {
+            per_sequence_tokens[s] = (uint32_t)tokens[s];
+            per_sequence_loss[s] = 0.0f;
+        }
+        if (total == 0) return FT_OK;
+        FT_TRY(model_forward(m, rows, B, S));
+        FT_TRY(ft_upload(m->ctx, m->targets_dev, tg.data(), T * sizeof(uint32_t)));
+        FT_TRY(ft_upload(m->ctx, m->weights_dev, wt.data(), T * sizeof(float)));
+        // forward only: the gradient the kernel writes (in place of the logits) is discarded
+        FT_TRY(ft_masked_cross_entropy_weighted(m->ctx, m->logits, m->targets_dev, m->weights_dev, m->logits,
+                                                m->row_loss, T, V, 1.0f));
+        return read_sequence_losses(m, B, S, tokens, per_sequence_loss, nullptr);
+    });
+}
+
 float ft_lr_schedule(uint32_t kind, float peak_lr, float min_lr, uint32_t warmup_steps, uint32_t total_steps,
                      uint32_t step) {
     const float pi = 3.14159265358979323846f;
@@ -927,17 +1001,10 @@ int ft_trainer_train_chunk(ft_trainer* t, const uint32_t* rows, const uint32_t* 
         std::memset(stats, 0, sizeof(*stats));
         stats->clip_scale = 1.0f;
 
-        // Host half of masked_cross_entropy_batch (trainer/src/lib.rs:689-722):
-        // per-row target or MASKED_CE_SKIP, weight 1 / supervised tokens of the row's sequence.
-        std::vector<uint32_t> tg(T);
-        std::vector<float> wt(T);
-        std::vector<size_t> tokens(B, 0);
-        auto supervised = [&](size_t r) { return loss_mask[r] != 0 && (size_t)targets[r] < V; };
-        size_t total_tokens = 0;
-        for (size_t s = 0; s < B; s++) {
-            for (size_t i = 0; i < S; i++) tokens[s] += supervised(s * S + i) ? 1 : 0;
-            total_tokens += tokens[s];
-        }
+        std::vector<uint32_t> tg;
+        std::vector<float> wt;
+        std::vector<size_t> tokens;
+        const size_t total_tokens = build_targets(targets, loss_mask, B, S, V, tg, wt, tokens);
         stats->supervised_tokens = (uint32_t)total_tokens;
         if (total_tokens == 0) {
             // masked_cross_entropy_batch returns None: no forward result is used, no backward.
@@ -945,15 +1012,6 @@ int ft_trainer_train_chunk(ft_trainer* t, const uint32_t* rows, const uint32_t* 
             if (per_sequence_loss)
                 for (size_t s = 0; s < B; s++) per_sequence_loss[s] = 0.0f;
         } else {
-            for (size_t r = 0; r < T; r++) {
-                if (supervised(r)) {
-                    tg[r] = targets[r];
-                    wt[r] = 1.0f / (float)tokens[r / S];
-                } else {
-                    tg[r] = FT_MASKED_CE_SKIP;
-                    wt[r] = 0.0f;
-                }
-            }
             FT_TRY(model_forward(m, rows, B, S));
             FT_TRY(ft_upload(ctx, m->targets_dev, tg.data(), T * sizeof(uint32_t)));
             FT_TRY(ft_upload(ctx, m->weights_dev, wt.data(), T * sizeof(float)));
@@ -986,19 +1044,7 @@ int ft_trainer_train_chunk(ft_trainer* t, const uint32_t* rows, const uint32_t* 
         }
 
         // The step's only wait: row losses and the control block.
-        if (total_tokens > 0) {
-            std::vector<float> losses(T);
-            FT_TRY(ft_download(ctx, losses.data(), m->row_loss, T * sizeof(float)));
-            float total = 0.0f;
-            for (size_t s = 0; s < B; s++) {
-                double sum = 0.0;
-                for (size_t i = 0; i < S; i++) sum += (double)losses[s * S + i];
-                const float mean = (float)(sum / (double)(tokens[s] ? tokens[s] : 1));
-                if (per_sequence_loss) per_sequence_loss[s] = mean;
-                total += mean;
-            }
-            stats->loss = total;
-        }
+        if (total_tokens > 0) FT_TRY(read_sequence_losses(m, B, S, tokens, per_sequence_loss, &stats->loss));
         if (window_full) {
             float control[3];
             FT_TRY(ft_download(ctx, control, t->control, sizeof(control)));

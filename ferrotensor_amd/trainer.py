@@ -151,6 +151,23 @@ class Lfm2Model:
                                                 out.ctypes.data_as(C.c_void_p)))
         return out
 
+    def evaluate(self, seqs, batch: int = 8, length_bucket: int = 32) -> Tuple[float, int]:
+        """`evaluate` of the CLI (ferrotensor-cli/src/main.rs:1110-1137): token-weighted mean loss
+        over [(input_ids, target_ids, loss_mask)] and the number of supervised tokens; (nan, 0) when
+        nothing is supervised. Forward only."""
+        loss_sum, tokens = 0.0, 0
+        kept = [(i, t, m) for i, t, m in seqs if len(i) > 0 and len(t) > 0]
+        for at in range(0, len(kept), batch):
+            rows, targets, masks = pad_chunk(kept[at:at + batch], length_bucket)
+            B, S = rows.shape
+            per, cnt = np.zeros(B, np.float32), np.zeros(B, np.uint32)
+            check(self._lib.ft_model_eval_chunk(self.handle, rows.ctypes.data_as(C.c_void_p),
+                                                targets.ctypes.data_as(C.c_void_p), masks.ctypes.data_as(C.c_void_p),
+                                                B, S, per.ctypes.data_as(C.c_void_p), cnt.ctypes.data_as(C.c_void_p)))
+            loss_sum += float((per.astype(np.float64) * cnt).sum())
+            tokens += int(cnt.sum())
+        return (float("nan"), 0) if tokens == 0 else (loss_sum / tokens, tokens)
+
     def close(self):
         if self.handle is not None and self.handle.value:
             for ref in self._trainers:

@@ -372,6 +372,13 @@ int ft_model_read_grad(ft_model* m, size_t index, float* out_host);
 /* Lfm2Model::forward_batch (lfm.rs:590-623): logits [B*S, vocab] to the host. */
 int ft_model_forward_logits(ft_model* m, const uint32_t* rows, size_t B, size_t S, float* logits_host);
 
+/* The forward-only loss of `evaluate` (ferrotensor-cli/src/main.rs:1110-1137: no_grad forward +
+ * masked cross-entropy): per sequence, the mean loss over its supervised targets and their count,
+ * for B equally long rows (pad as for training). Nothing is kept for backward and no gradient
+ * or parameter is touched. */
+int ft_model_eval_chunk(ft_model* m, const uint32_t* rows, const uint32_t* targets, const uint8_t* loss_mask,
+                        size_t B, size_t S, float* per_sequence_loss, uint32_t* per_sequence_tokens);
+
 /* Trainer::new + with_clip_grad_norm (trainer/src/lib.rs:113-205) with an
  * AdamW (autograd/src/lib.rs:1502-1515). clip_grad_norm <= 0 disables
  * clipping. */

@@ -367,6 +367,37 @@ def test_micro_batches_accumulate_to_the_batched_step(ctx):
             assert_close("param " + k, p[k], p0[k], atol=1e-6, rtol=1e-4)
 
 
+def test_evaluate_is_the_token_weighted_forward_loss(ctx):
+    """`evaluate` (ferrotensor-cli/src/main.rs:1110-1137): sum(loss_i * n_i) / sum(n_i) over ragged
+    examples, forward only: parameters and gradients are untouched."""
+    from ferrotensor_amd.data import TrainingExample
+    cfg = tiny_config(True, True)
+    hip, orc = build_pair(ctx, cfg, ["q_proj", "v_proj"], rank=4, alpha=8.0, seed=27)
+    rng = np.random.default_rng(3)
+    examples = [TrainingExample.from_sft_prompt_response(rng.integers(0, 256, p).tolist(),
+                                                         rng.integers(0, 256, r).tolist())
+                for p, r in [(5, 9), (12, 3), (1, 30), (20, 20), (7, 1)]]
+    examples.append(TrainingExample([1, 2, 3], [2, 3, 4], [0, 0, 0]))       # nothing supervised
+    before = hip.params()
+    loss, tokens = hip.evaluate([e.as_tuple() for e in examples], batch=4)
+    want_sum, want_tokens = 0.0, 0
+    for e in examples:
+        if not any(e.loss_mask):
+            continue
+        logits, _ = orc.forward(np.array([e.input_ids], np.uint32))
+        res = rs.masked_cross_entropy_batch(logits, np.array([e.target_ids], np.uint32),
+                                            np.array([e.loss_mask], np.uint8), 1)
+        (mean, n), = res[1]
+        want_sum += float(mean) * n
+        want_tokens += n
+    assert tokens == want_tokens == sum(sum(e.loss_mask) for e in examples)
+    assert_close("eval loss", [loss], [want_sum / want_tokens])
+    after = hip.params()
+    for n in before:
+        np.testing.assert_array_equal(before[n], after[n])
+    assert hip.evaluate([examples[-1].as_tuple()])[1] == 0
+
+
 def test_targets_masking_is_bit_exact_against_oracle(ctx):
     """Skipped rows (mask 0 or target >= vocab) contribute exactly nothing:
     the loss equals the oracle's and flipping masked targets changes no bit."""
