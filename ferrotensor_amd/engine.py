@@ -8,6 +8,7 @@ shape or dtype violation, these raise (AssertionError for shape checks done
 here, FtError for errors the library reports). All compute happens in the HIP
 library; numpy only carries host data in and out.
 """
+import atexit
 import ctypes as C
 import weakref
 from dataclasses import dataclass
@@ -32,6 +33,22 @@ class DType:
         return 4 if dtype == DType.FP32 else 2
 
 
+# Contexts still open when the interpreter shuts down are closed from an atexit hook, i.e. while
+# the HIP runtime is still alive: finalisers that run during module teardown may come after it.
+_live_contexts = weakref.WeakSet()
+
+
+def _close_live_contexts():
+    for ctx in list(_live_contexts):
+        try:
+            ctx.close()
+        except Exception:
+            pass
+
+
+atexit.register(_close_live_contexts)
+
+
 class HipContext:
     """`WgpuContext` (context.rs): one device, one in-order stream, the buffer pool."""
 
@@ -46,6 +63,7 @@ class HipContext:
         # Objects that hold device memory of this context (models, trainers):
         # closed first, so no handle outlives the context it allocates from.
         self._children = weakref.WeakSet()
+        _live_contexts.add(self)
 
     def _adopt(self, child):
         self._children.add(child)
