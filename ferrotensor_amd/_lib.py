@@ -22,7 +22,8 @@ class AttentionOptionsC(C.Structure):
 
 class LoraLinearDescC(C.Structure):
     _fields_ = [("w", C.c_void_p), ("w_dtype", C.c_int32), ("t", C.c_void_p), ("b", C.c_void_p),
-                ("residual", C.c_void_p), ("y", C.c_void_p), ("N", C.c_size_t), ("r", C.c_size_t)]
+                ("residual", C.c_void_p), ("y", C.c_void_p), ("N", C.c_size_t), ("r", C.c_size_t),
+                ("rope_table", C.c_void_p), ("rope_seq", C.c_size_t)]
 
 
 class LoraDxDescC(C.Structure):
@@ -90,6 +91,8 @@ SIGNATURES = {
     "ft_lora_down": [_P, _P, _P, _P, _SZ, _SZ, _SZ, _F],
     "ft_lora_linear_group": [_P, _P, C.POINTER(LoraLinearDescC), _SZ, _SZ, _SZ],
     "ft_lora_linear_dx_group": [_P, C.POINTER(LoraDxDescC), _SZ, _P, _P, _SZ, _SZ],
+    "ft_rope_table": [_P, _P, _SZ, _SZ, _SZ, _F],
+    "ft_rope_apply": [_P, _P, _P, _SZ, _SZ, _SZ, _SZ, _P, _I],
     "ft_mlp_gate_up": [_P, _P, _P, _P, _I, _P, _P, _P, _SZ, _SZ, _SZ],
     "ft_mlp_down_backward": [_P, _P, _P, _I, _P, _P, _P, _P, _P, _SZ, _SZ, _SZ],
     "ft_lora_linear": [_P, _P, _P, _I, _P, _P, _P, _P, _SZ, _SZ, _SZ, _SZ],

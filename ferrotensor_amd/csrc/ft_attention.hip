@@ -34,6 +34,10 @@ struct AttnArgs {
     int B, Sq, Sk, H, Hkv, D;
     int causal, causal_offset;
     float scale;
+    // Backward only, head_dim 64 on the LDS kernels: when set, dQ and dK leave the kernels already
+    // rotated back through RoPE (the inverse rotation by the (cos, sin) of their token position,
+    // table [Sq or Sk][32] float2), which is what RoPENode::backward does to them next.
+    const float2* rope;
 };
 
 #define MFMA(a, b, c) __builtin_amdgcn_mfma_f32_32x32x2f32((a), (b), (c), 0, 0, 0)
@@ -732,8 +736,19 @@ __global__ __launch_bounds__(512) void attn_bwd_dkdv_lds_kernel(AttnArgs p) {
                 sv += red[w * PRIV + DP * 33 + d * 33 + kk];
             }
             const long o = (((long)b * p.Sk + krow) * p.Hkv + kvh) * DP + d;
-            p.dk[o] = sk * p.scale;  // dK = scale * sum dS Q (Q is read unscaled)
             p.dv[o] = sv;
+            if (DP == 64 && p.rope) {
+                // dK rotated back: this thread also sums the partner element (d +- 32)
+                const int dp = d < 32 ? d + 32 : d - 32;
+                float sp = 0.0f;
+#pragma unroll
+                for (int w = 0; w < NWV; w++) sp += red[w * PRIV + dp * 33 + kk];
+                const float2 cs = p.rope[(long)krow * 32 + (d & 31)];
+                const float x = sk * p.scale, y = sp * p.scale;
+                p.dk[o] = d < 32 ? x * cs.x + y * cs.y : x * cs.x - y * cs.y;
+            } else {
+                p.dk[o] = sk * p.scale;  // dK = scale * sum dS Q (Q is read unscaled)
+            }
         }
     }
 }
@@ -1027,6 +1042,27 @@ __global__ __launch_bounds__(kKeySplitDq * 64) void attn_bwd_dq_lds_kernel(AttnA
 
     if (!q_ok) return;
     float* drow = p.dq + qoff;
+    if constexpr (DP == 64) {
+        if (p.rope) {
+            // pairs (d, d + 32) are registers r of accumulator blocks 0 and 1 of this lane
+            const float2* tb = p.rope + (long)qi * 32;
+#pragma unroll
+            for (int r4 = 0; r4 < 4; r4++) {
+                const int d = r4 * 8 + half * 4;
+                float lo[4], hi[4];
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    const float2 cs = tb[d + e];
+                    const float x1 = acc[0][r4 * 4 + e] * p.scale, x2 = acc[1][r4 * 4 + e] * p.scale;
+                    lo[e] = x1 * cs.x + x2 * cs.y;
+                    hi[e] = x2 * cs.x - x1 * cs.y;
+                }
+                *reinterpret_cast<float4*>(drow + d) = make_float4(lo[0], lo[1], lo[2], lo[3]);
+                *reinterpret_cast<float4*>(drow + 32 + d) = make_float4(hi[0], hi[1], hi[2], hi[3]);
+            }
+            return;
+        }
+    }
 #pragma unroll
     for (int f = 0; f < NF; f++)
 #pragma unroll
@@ -1182,3 +1218,29 @@ int ft_flash_attention_v2_backward_with_stats(ft_context* ctx, const float* q, c
 }
 
 }  // extern "C"
+
+// Can the backward kernels rotate dQ and dK back through RoPE themselves (self-attention over
+// whole rows from position 0, head_dim 64, aligned tensors)?
+bool ft_internal_attention_rope_fusable(const float* q, const float* k, const float* v, const float* out,
+                                        const float* d_out, size_t Sq, size_t Sk, size_t D) {
+    AttnArgs a{};
+    a.D = (int)D;
+    a.q = q; a.k = k; a.v = v; a.out = out; a.d_out = d_out;
+    return D == 64 && Sq == Sk && attn_full(a, 64);
+}
+
+// ft_flash_attention_v2_backward_with_stats followed by the inverse RoPE of dq and dk (positions
+// 0..S-1, table from ft_internal_rope_table), in the same two launches.
+int ft_internal_attention_backward_rope(ft_context* ctx, const float* q, const float* k, const float* v,
+                                        const float* out, const float* d_out, float* dq, float* dk, float* dv,
+                                        float* stats, size_t B, size_t S, size_t H, size_t Hkv,
+                                        const ft_attention_options* opts, const float* rope_table) {
+    FT_TRY(check_common("attention backward", ctx, B, S, S, H, Hkv, 64, opts));
+    FT_CHECK_ARG(q && k && v && out && d_out && dq && dk && dv && stats && rope_table, "attention backward: NULL tensor");
+    FT_CHECK_ARG(ft_internal_attention_rope_fusable(q, k, v, out, d_out, S, S, 64), "attention backward: not fusable");
+    if (B == 0 || H == 0) return FT_OK;
+    AttnArgs a = make_args(B, S, S, H, Hkv, 64, opts);
+    a.q = q; a.k = k; a.v = v; a.out = out; a.d_out = d_out; a.dq = dq; a.dk = dk; a.dv = dv; a.stats = stats;
+    a.rope = reinterpret_cast<const float2*>(rope_table);
+    return launch_bwd<64>(ctx, a);
+}

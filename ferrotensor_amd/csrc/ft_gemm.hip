@@ -579,6 +579,11 @@ struct AsyncProb {
     const float* e2;
     int N, ldc, tiles_n, tile_begin, nseg;
     long partial_off;  // split-K: this product's slice of AsyncBatch::partial, [splits][M][N]
+    // RoPE on the output (64x64 tiles, head_dim 64, so a tile is one head of 64 rows): element
+    // (row, h*64 + i) pairs with (row, h*64 + i + 32) and rotates by the (cos, sin) of token position
+    // row % rope_seq, table [rope_seq][32] float2. NULL = no rotation.
+    const float2* rope;
+    int rope_seq;
 };
 
 constexpr int kEpiPlain = 0, kEpiGateUp = 1, kEpiSiluBwd = 2;
@@ -870,6 +875,33 @@ __global__ __launch_bounds__(256) void gemm_async_kernel(AsyncBatch g) {
     // Nothing may still be landing in LDS when the workgroup retires.
     __builtin_amdgcn_s_waitcnt(0x0F70);
 
+    if constexpr (EPI == kEpiPlain && BM == 64 && BN == 64) {
+        if (p.rope) {  // uniform per workgroup; never together with split-K
+            // The partner column (+-32) belongs to the neighbouring wave: exchange through the
+            // stage memory (free now: every wave has waited for its own loads, the barrier makes
+            // that true of all of them).
+            __syncthreads();
+            float* mine = (wave < 2 ? St0 : St1) + (wave & 1) * 1024;
+            const float* other = (wave < 2 ? St0 : St1) + ((wave & 1) ^ 1) * 1024;
+#pragma unroll
+            for (int r = 0; r < 16; r++) mine[r * 64 + lane] = acc[0][0][r];
+            __syncthreads();
+            const int col = n0 + wn0 + l32;
+            const bool upper = wn0 != 0;  // this wave holds i + 32
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int row = m0 + wm0 + (r / 4) * 8 + half * 4 + (r % 4);
+                if (row < M && col < p.N) {
+                    const float2 cs = p.rope[(long)(row % p.rope_seq) * 32 + l32];
+                    const float self = acc[0][0][r], peer = other[r * 64 + lane];
+                    // lower: x1*c - x2*s ; upper: x1*s + x2*c  (x1 = lower half, x2 = upper half)
+                    p.out[(long)row * p.ldc + col] = upper ? peer * cs.y + self * cs.x : self * cs.x - peer * cs.y;
+                }
+            }
+            return;
+        }
+    }
+
 #pragma unroll
     for (int i = 0; i < FM; i++)
 #pragma unroll
@@ -1043,7 +1075,9 @@ int launch_async(ft_context* ctx, AsyncBatch g, int layout, int epi = kEpiPlain)
         mn4 = mn4 && ((size_t)g.M * g.p[i].N) % 4 == 0 && g.p[i].ldc == g.p[i].N;
         out_floats += (size_t)g.M * g.p[i].N;
     }
-    if (epi == kEpiPlain && mn4 && tiles > 0 && (size_t)tiles * 2 <= (size_t)ctx->num_cus) {
+    bool any_rope = false;
+    for (int i = 0; i < g.count; i++) any_rope = any_rope || g.p[i].rope != nullptr;
+    if (epi == kEpiPlain && mn4 && !any_rope && tiles > 0 && (size_t)tiles * 2 <= (size_t)ctx->num_cus) {
         int want = (int)((2 * (size_t)ctx->num_cus + tiles - 1) / tiles);
         if (want > 8) want = 8;
         if (want > min_kt / 4) want = min_kt / 4;
@@ -1333,10 +1367,17 @@ int ft_lora_linear_group(ft_context* ctx, const float* x, const ft_lora_linear_d
     FT_CHECK_ARG(ctx && linears && count >= 1 && count <= (size_t)kAsyncMaxProb,
                  "ft_lora_linear_group: 1..%d linears per call", kAsyncMaxProb);
     bool batch = M < (1u << 30) && K < (1u << 30) && M > 0;
+    bool any_rope = false;
     for (size_t i = 0; i < count; i++) {
         const ft_lora_linear_desc& d = linears[i];
         FT_CHECK_ARG(d.w_dtype == FT_DTYPE_F32 || d.w_dtype == FT_DTYPE_F16, "ft_lora_linear_group: dtype %d",
                      d.w_dtype);
+        if (d.rope_table) {
+            FT_CHECK_ARG(d.residual == nullptr && d.N % 64 == 0 && d.rope_seq > 0 && M % d.rope_seq == 0,
+                         "ft_lora_linear_group: a rotated output needs head_dim 64, whole rows of rope_seq tokens "
+                         "and no residual");
+            any_rope = true;
+        }
         FT_CHECK_ARG(d.r == 0 || (d.t && d.b), "ft_lora_linear_group: linear %zu has a rank but no factors", i);
         batch = batch && d.w_dtype == FT_DTYPE_F16 && d.N < (1u << 30) &&
                 async_eligible(0, x, d.w, d.y, d.residual, M, K, d.N, d.t, d.b, d.r);
@@ -1353,13 +1394,18 @@ int ft_lora_linear_group(ft_context* ctx, const float* x, const ft_lora_linear_d
             g.p[i].add = d.residual;
             g.p[i].N = (int)d.N;
             g.p[i].ldc = (int)d.N;
+            g.p[i].rope = reinterpret_cast<const float2*>(d.rope_table);
+            g.p[i].rope_seq = (int)d.rope_seq;
         }
-        return launch_async_auto(ctx, g, 0);
+        if (!any_rope) return launch_async_auto(ctx, g, 0);
+        return launch_async<64, 64, 32, 32>(ctx, g, 0);  // the rotation lives in the 64x64 epilogue
     }
     for (size_t i = 0; i < count; i++) {
         const ft_lora_linear_desc& d = linears[i];
         FT_TRY(ft_lora_linear(ctx, x, d.w, d.w_dtype, d.r ? d.t : nullptr, d.r ? d.b : nullptr, d.residual, d.y, M, K,
                               d.N, d.r));
+        if (d.rope_table)
+            FT_TRY(ft_rope_apply(ctx, d.y, d.y, M / d.rope_seq, d.rope_seq, d.N, 64, d.rope_table, 0));
     }
     return FT_OK;
 }

@@ -856,6 +856,20 @@ int ft_embedding(ft_context* ctx, const float* table, size_t vocab, size_t hidde
     return FT_OK;
 }
 
+int ft_rope_table(ft_context* ctx, float* table, size_t seq, size_t head_dim, size_t pos, float theta) {
+    FT_CHECK_ARG(ctx && table, "ft_rope_table: NULL argument");
+    FT_CHECK_ARG(head_dim >= 2 && head_dim % 2 == 0, "ft_rope_table: head_dim %zu must be even", head_dim);
+    return ft_internal_rope_table(ctx, table, seq, head_dim, pos, theta);
+}
+
+int ft_rope_apply(ft_context* ctx, const float* x, float* out, size_t batch, size_t seq, size_t hidden,
+                  size_t head_dim, const float* table, int inverse) {
+    FT_CHECK_ARG(ctx && x && out && table, "ft_rope_apply: NULL argument");
+    FT_CHECK_ARG(head_dim > 0 && hidden % head_dim == 0, "ft_rope_apply: hidden %zu is not a multiple of head_dim %zu",
+                 hidden, head_dim);
+    return ft_internal_rope_pair(ctx, x, out, hidden / head_dim, x, out, 0, table, batch, seq, head_dim, inverse);
+}
+
 int ft_rms_norm_eps(ft_context* ctx, const float* x, const float* w, float* out, size_t rows, size_t size,
                     float eps) {
     FT_CHECK_ARG(ctx && x && w && out, "ft_rms_norm_eps: NULL argument");

@@ -42,6 +42,12 @@ int ft_internal_rope_table(ft_context* ctx, float* table, size_t seq, size_t hea
 int ft_internal_rope_pair(ft_context* ctx, const float* a_src, float* a_dst, size_t heads_a, const float* b_src,
                           float* b_dst, size_t heads_b, const float* table, size_t batch, size_t seq,
                           size_t head_dim, int inverse);
+bool ft_internal_attention_rope_fusable(const float* q, const float* k, const float* v, const float* out,
+                                        const float* d_out, size_t Sq, size_t Sk, size_t D);
+int ft_internal_attention_backward_rope(ft_context* ctx, const float* q, const float* k, const float* v,
+                                        const float* out, const float* d_out, float* dq, float* dk, float* dv,
+                                        float* stats, size_t B, size_t S, size_t H, size_t Hkv,
+                                        const ft_attention_options* opts, const float* rope_table);
 int ft_internal_multi_adamw(ft_context* ctx, const ft_segment* segs_dev, size_t nseg, const ft_adam_params* p,
                             float grad_scale, const float* control_dev);
 
@@ -272,15 +278,18 @@ int linear_gemm(ft_context* ctx, const LinearW& l, const float* x, const float* 
 }
 
 // y_i = x @ W_i (+ t_i @ B_i) for linears that share x, in one launch when they can be batched.
+// The first `n_rope` outputs are rotated through RoPE in the GEMM epilogue when `rope_table` is given.
 int linear_gemm_group(ft_context* ctx, LinearW* const* ls, const float* const* ts, float* const* ys, int n,
-                      const float* x, size_t T) {
+                      const float* x, size_t T, const float* rope_table = nullptr, size_t rope_seq = 0,
+                      int n_rope = 0) {
     ft_lora_linear_desc d[3];
     for (int i = 0; i < n; i++) {
         const LinearW& l = *ls[i];
         FT_CHECK_ARG(l.w, "linear %s has no weight", l.prefix.c_str());
         FT_CHECK_ARG(l.in == ls[0]->in, "grouped linears must share their input width");
         d[i] = ft_lora_linear_desc{l.w, l.dtype, l.has_lora() ? ts[i] : nullptr, l.has_lora() ? l.b : nullptr,
-                                   nullptr, ys[i], l.out, l.has_lora() ? l.r : 0};
+                                   nullptr, ys[i], l.out, l.has_lora() ? l.r : 0,
+                                   i < n_rope ? rope_table : nullptr, i < n_rope ? rope_seq : 0};
     }
     return ft_lora_linear_group(ctx, x, d, (size_t)n, T, ls[0]->in);
 }
@@ -412,9 +421,13 @@ int layer_forward(ft_model* m, size_t l, size_t B, size_t S) {
             LinearW* ls[3] = {&L.q, &L.k, &L.v};
             const float* ts[3] = {a.tq, a.tk, a.tv};
             float* ys[3] = {a.q, a.k, a.v};
-            FT_TRY(linear_gemm_group(ctx, ls, ts, ys, 3, a.h1, T));
+            // head_dim 64: q and k leave the GEMM already rotated
+            const bool fused_rope = m->rope_table && D == 64;
+            FT_TRY(linear_gemm_group(ctx, ls, ts, ys, 3, a.h1, T, fused_rope ? m->rope_table : nullptr, S,
+                                     fused_rope ? 2 : 0));
         }
-        if (m->rope_table) {
+        if (m->rope_table && D == 64) {
+        } else if (m->rope_table) {
             FT_TRY(ft_internal_rope_pair(ctx, a.q, a.q, nh, a.k, a.k, nkv, m->rope_table, B, S, D, 0));
         } else {
             FT_TRY(ft_rope_theta(ctx, a.q, B, S, nh * D, D, 0, c.rope_theta));
@@ -509,13 +522,20 @@ int model_backward(ft_model* m, size_t B, size_t S, bool accumulate) {
         FT_TRY(ft_internal_rms_norm_backward_add(ctx, a.h, L.norm2, m->d_h2, g, g_other, T, H, c.rms_norm_eps));
         // h = x + o_proj(attn)
         FT_TRY(linear_backward(m, L.o, a.attn, a.to, g_other, m->d_attn, T, accumulate));
-        FT_TRY(ft_flash_attention_v2_backward_with_stats(ctx, a.q, a.k, a.v, a.attn, m->d_attn, m->dq, m->dk, m->dv,
-                                                         a.stats, B, S, S, nh, nkv, D, &opts));
-        if (m->rope_table) {
-            FT_TRY(ft_internal_rope_pair(ctx, m->dq, m->dq, nh, m->dk, m->dk, nkv, m->rope_table, B, S, D, 1));
+        if (m->rope_table &&
+            ft_internal_attention_rope_fusable(a.q, a.k, a.v, a.attn, m->d_attn, S, S, D)) {
+            // dq and dk come out of the attention kernels already rotated back through RoPE
+            FT_TRY(ft_internal_attention_backward_rope(ctx, a.q, a.k, a.v, a.attn, m->d_attn, m->dq, m->dk, m->dv,
+                                                       a.stats, B, S, nh, nkv, &opts, m->rope_table));
         } else {
-            FT_TRY(ft_rope_theta_inverse(ctx, m->dq, B, S, nh * D, D, 0, c.rope_theta));
-            FT_TRY(ft_rope_theta_inverse(ctx, m->dk, B, S, nkv * D, D, 0, c.rope_theta));
+            FT_TRY(ft_flash_attention_v2_backward_with_stats(ctx, a.q, a.k, a.v, a.attn, m->d_attn, m->dq, m->dk,
+                                                             m->dv, a.stats, B, S, S, nh, nkv, D, &opts));
+            if (m->rope_table) {
+                FT_TRY(ft_internal_rope_pair(ctx, m->dq, m->dq, nh, m->dk, m->dk, nkv, m->rope_table, B, S, D, 1));
+            } else {
+                FT_TRY(ft_rope_theta_inverse(ctx, m->dq, B, S, nh * D, D, 0, c.rope_theta));
+                FT_TRY(ft_rope_theta_inverse(ctx, m->dk, B, S, nkv * D, D, 0, c.rope_theta));
+            }
         }
         // The first block's input is the frozen embedding: its norm output needs
         // no gradient, so the three input-gradient GEMMs are skipped

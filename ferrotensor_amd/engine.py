@@ -317,15 +317,29 @@ class ComputeEngine:
         assert K == K2 and y.numel() == M * N
         check(self._lib.ft_lora_linear(ctx.handle, _p(x), _p(w), w.dtype, _p(t), _p(b), _p(residual), _p(y), M, K, N, r))
 
-    def lora_linear_group(self, ctx, x, linears):
-        """linears: [(w, t, b, y, residual)] sharing the input x; one launch when all can be batched."""
+    def rope_table(self, ctx, seq, head_dim, pos, theta):
+        """(cos, sin) pairs of `rope_theta` for `seq` positions from `pos`: [seq, head_dim/2, 2] f32."""
+        table = UnifiedTensor.empty(ctx, [seq, head_dim // 2, 2])
+        check(self._lib.ft_rope_table(ctx.handle, _p(table), seq, head_dim, pos, theta))
+        return table
+
+    def rope_apply(self, ctx, x, out, head_dim, table, inverse=False):
+        batch, seq, hidden = x.shape
+        check(self._lib.ft_rope_apply(ctx.handle, _p(x), _p(out), batch, seq, hidden, head_dim, _p(table),
+                                      1 if inverse else 0))
+
+    def lora_linear_group(self, ctx, x, linears, rope_table=None, rope_seq=0, n_rope=0):
+        """linears: [(w, t, b, y, residual)] sharing the input x; one launch when all can be batched.
+        The first `n_rope` outputs are rotated through RoPE (heads of 64, rows of `rope_seq` tokens)."""
         from ._lib import LoraLinearDescC
         M, K = x.shape
         descs = (LoraLinearDescC * len(linears))()
-        for d, (w, t, b, y, residual) in zip(descs, linears):
+        for i, (d, (w, t, b, y, residual)) in enumerate(zip(descs, linears)):
             assert w.shape[0] == K and y.numel() == M * w.shape[1]
             d.w, d.w_dtype, d.t, d.b, d.residual, d.y = _v(w), w.dtype, _v(t), _v(b), _v(residual), _v(y)
             d.N, d.r = w.shape[1], (b.shape[0] if b is not None else 0)
+            if i < n_rope and rope_table is not None:
+                d.rope_table, d.rope_seq = _v(rope_table), rope_seq
         check(self._lib.ft_lora_linear_group(ctx.handle, _p(x), descs, len(linears), M, K))
 
     def lora_linear_dx_group(self, ctx, linears, dx, residual=None):

@@ -146,6 +146,11 @@ typedef struct ft_lora_linear_desc {
     float* y;
     size_t N;
     size_t r;
+    /* RoPENode fused into the projection (Attention::forward, graph/src/lib.rs:367-414, applies
+     * rope to q and k right after their projections): when not NULL, y is rotated with this
+     * (cos, sin) table of ft_rope_table for rows of rope_seq tokens and heads of 64 values. */
+    const float* rope_table;
+    size_t rope_seq;
 } ft_lora_linear_desc;
 int ft_lora_linear_group(ft_context* ctx, const float* x, const ft_lora_linear_desc* linears, size_t count,
                          size_t M, size_t K);
@@ -236,6 +241,14 @@ int ft_rope_theta_inverse(ft_context* ctx, float* t, size_t batch, size_t seq, s
  * make first, autograd/src/lib.rs:509-533, 1122-1139). */
 int ft_rope_theta_to(ft_context* ctx, const float* src, float* dst, size_t batch, size_t seq,
                      size_t hidden, size_t head_dim, size_t pos, float theta, int inverse);
+
+/* The (cos, sin) pairs of rope_theta for `seq` positions starting at `pos`:
+ * table[seq][head_dim/2] float2 = (cos, sin)(position * theta^(-2i/head_dim)), computed exactly
+ * as the rope kernel computes them; and the rotation of x [batch, seq, hidden] through such a
+ * table (inverse != 0: the backward rotation). head_dim must be a multiple of 8 here. */
+int ft_rope_table(ft_context* ctx, float* table, size_t seq, size_t head_dim, size_t pos, float theta);
+int ft_rope_apply(ft_context* ctx, const float* x, float* out, size_t batch, size_t seq, size_t hidden,
+                  size_t head_dim, const float* table, int inverse);
 
 /* ---- attention (engine/attention.rs:165-177, 341-358, 581-594) ----------- */
 

@@ -192,6 +192,43 @@ def test_grouped_linears_match_single_calls(g, M, K, Ns, r, f16):
     assert_close("group dx + residual", dx2.to_numpy(), want_dx + res, atol=3e-3, rtol=1e-4)
 
 
+@pytest.mark.parametrize("B,S,K,heads,kv,r,f16", [(2, 64, 192, 3, 1, 8, True), (1, 32, 64, 2, 2, 0, True),
+                                                  (2, 24, 96, 2, 1, 4, False)])
+def test_grouped_projections_with_rope_in_the_epilogue(g, B, S, K, heads, kv, r, f16):
+    """q and k rotated inside the projection launch (heads of 64) == projection followed by rope."""
+    from ferrotensor_amd import UnifiedTensor
+    ctx, eng = g
+    D, M, theta = 64, B * S, 10000.0
+    x = rnd(1, M, K)
+    table = eng.rope_table(ctx, S, D, 0, theta)
+    items, wants = [], []
+    for i, N in enumerate((heads * D, kv * D, kv * D)):
+        w = rnd(10 + i, K, N, scale=0.05)
+        wr = cpu.round_f16(w) if f16 else w
+        wt = UnifiedTensor.from_f32_as_f16(ctx, w, [K, N]) if f16 else up(ctx, w)
+        want = cpu.matmul(x, wr)
+        t = bm = None
+        if r:
+            tt, bb = rnd(20 + i, M, r), rnd(30 + i, r, N, scale=0.1)
+            want = want + cpu.matmul(tt, bb)
+            t, bm = up(ctx, tt), up(ctx, bb)
+        if i < 2:
+            want = cpu.rope(want.reshape(B, S, N), D, 0, theta).reshape(M, N)
+        items.append((wt, t, bm, empty(ctx, M, N), None))
+        wants.append(want)
+    eng.lora_linear_group(ctx, up(ctx, x), items, rope_table=table, rope_seq=S, n_rope=2)
+    for i, (it, want) in enumerate(zip(items, wants)):
+        assert_close("rotated projection %d" % i, it[3].to_numpy(), want, atol=1e-3, rtol=1e-4)
+    # the table-driven rotation on its own, both directions
+    y = rnd(40, B, S, heads * D)
+    out = empty(ctx, B, S, heads * D)
+    eng.rope_apply(ctx, up(ctx, y.reshape(B, S, heads * D)), out, D, table)
+    assert_close("rope_apply", out.to_numpy().reshape(y.shape), cpu.rope(y, D, 0, theta))
+    back = empty(ctx, B, S, heads * D)
+    eng.rope_apply(ctx, out, back, D, table, inverse=True)
+    assert_close("rope_apply inverse", back.to_numpy().reshape(y.shape), y, atol=1e-5)
+
+
 @pytest.mark.parametrize("M,H,F,f16", [(256, 960, 2560, True), (100, 64, 96, True), (70, 32, 40, True),
                                        (64, 32, 48, False)])
 def test_fused_gated_mlp_halves(g, M, H, F, f16):

@@ -398,6 +398,42 @@ def test_evaluate_is_the_token_weighted_forward_loss(ctx):
     assert hip.evaluate([examples[-1].as_tuple()])[1] == 0
 
 
+@pytest.mark.parametrize("checkpoint", [False, True])
+def test_head_dim_64_step_matches_oracle(ctx, checkpoint):
+    """Head dim 64 takes the fused paths of the 360M shape (RoPE in the q/k projection epilogue, inverse
+    RoPE in the attention backward kernels, LDS attention kernels, fused MLP halves): gradients and two
+    optimizer steps against the oracle."""
+    from ferrotensor_amd.trainer import ModelConfig, Trainer
+    cfg = ModelConfig(vocab_size=256, hidden_size=192, intermediate_size=256, num_hidden_layers=2,
+                      num_attention_heads=3, num_key_value_heads=1, rms_norm_eps=1e-5, rope_theta=100000.0,
+                      tie_word_embeddings=True, f16_linears=True, checkpoint_blocks=checkpoint)
+    hip, orc = build_pair(ctx, cfg, ["q_proj", "k_proj", "v_proj", "o_proj"], rank=8, alpha=16.0, seed=31)
+    rng = np.random.default_rng(4)
+    B, S = 2, 64
+    rows = rng.integers(0, 256, (B, S)).astype(np.uint32)
+    targets = np.concatenate([rows[:, 1:], rows[:, :1]], axis=1)
+    masks = np.ones((B, S), np.uint8)
+    masks[:, :9] = 0
+    want_logits, _ = orc.forward(rows)
+    assert_close("logits", hip.forward_batch(rows), want_logits)
+    tr = Trainer(hip, lr=1e-3, weight_decay=0.0, clip_grad_norm=1.0)
+    opt = rs.AdamW(lr=1e-3, weight_decay=0.0)
+    for step in range(2):
+        tr.train_chunk(rows, targets, masks, apply=False)
+        grads = hip.grads()
+        want_stats, _, want_grads = rs.train_chunk(orc, opt, rows, targets, masks, clip_grad_norm=1.0,
+                                                   return_grads=True)
+        cs = want_stats.clip_scale or 1.0
+        for n in grads:
+            assert_close(f"step {step} grad {n}", grads[n], want_grads[n] / np.float32(cs))
+        st = tr.train_chunk(rows, targets, masks)
+        assert_close("loss", [st.loss], [want_stats.loss])
+        assert_close("grad_norm", [st.grad_norm], [want_stats.grad_norm])
+        params = hip.params()
+        for n, w in orc.lora_params():
+            assert_close(f"step {step} weight {n}", params[n], w, atol=1e-6, rtol=1e-4)
+
+
 def test_targets_masking_is_bit_exact_against_oracle(ctx):
     """Skipped rows (mask 0 or target >= vocab) contribute exactly nothing:
     the loss equals the oracle's and flipping masked targets changes no bit."""
