@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """LoRA train step benchmark on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload 360m|135m|1.7b|tiny]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload 360m|135m|1.7b|tiny|micro]
 
 A step is one full optimizer step (forward, masked cross-entropy, backward,
 gradient norm, clip, AdamW) of the SmolLM2-360M-shaped model on 8 sequences x
@@ -17,6 +17,12 @@ Prints ONE JSON line: tokens/s (positions = B*S / step time), plus
                the 157.3 TFLOP/s dense FP32 matrix peak;
   cpu_baseline the CPU oracle (oracle/) on this host's cores, on a bounded
                sample of the same workload (stated in `sample`).
+
+--workload micro runs the kernel microbenchmark instead (BASELINE.json
+configs[1]: the 2048x576x1536 LoRA GEMM and its two backward GEMMs, attention
+forward + backward at 8 x 256 x 9/3 heads x 64, RMSNorm forward + backward on
+2048 x 576, AdamW over 4M parameters) and prints one JSON line with every
+kernel's HIP-event time against the roofline that bounds it.
 """
 import argparse
 import ctypes as C
@@ -181,12 +187,97 @@ def measured_traffic(kernel, workload):
     return None
 
 
+def micro_bench(args):
+    """The kernel microbenchmark: each kernel `steps` times after `warmup` passes, timed by HIP events on the
+    library's stream; algorithmic flops and bytes are the ones the library records per launch."""
+    from ferrotensor_amd import AdamParams, AttentionOptions, ComputeEngine, HipContext, UnifiedTensor
+    from ferrotensor_amd._lib import check
+
+    ctx = HipContext(0)
+    eng = ComputeEngine(ctx)
+    rng = np.random.default_rng(0)
+
+    def up(*shape, scale=1.0):
+        return UnifiedTensor.new(ctx, rng.standard_normal(shape, dtype=np.float32) * np.float32(scale), list(shape))
+
+    def empty(*shape):
+        return UnifiedTensor.empty(ctx, list(shape))
+
+    M, K, N, r, s = 2048, 576, 1536, 8, 2.0
+    x, dy = up(M, K), up(M, N)
+    w = UnifiedTensor.from_f32_as_f16(ctx, rng.standard_normal((K, N), dtype=np.float32), [K, N])
+    a, b = up(K, r), up(r, N)
+    t_, dt, y, dx = empty(M, r), empty(M, r), empty(M, N), empty(M, K)
+    dw, da, db = empty(K, N), empty(K, r), empty(r, N)
+    B, S, H, Hkv, D = 8, 256, 9, 3, 64
+    q, k, v, do = up(B, S, H, D), up(B, S, Hkv, D), up(B, S, Hkv, D), up(B, S, H, D)
+    o, stats = empty(B, S, H, D), empty(B * H * S, 2)
+    dq, dk, dv = empty(B, S, H, D), empty(B, S, Hkv, D), empty(B, S, Hkv, D)
+    opts = AttentionOptions(causal=True)
+    nx, ng, nw = up(M, K), up(M, K), up(K)
+    ny, ngx, ngw = empty(M, K), empty(M, K), empty(K)
+    n = 4 * 1024 * 1024
+    pw, pg, pm = up(n), up(n), up(n, scale=0.1)
+    pv = UnifiedTensor.new(ctx, np.abs(rng.standard_normal(n, dtype=np.float32)) * np.float32(0.1), [n])
+    adam = AdamParams(lr=2e-4, weight_decay=0.01, t=3.0)
+
+    def one_pass():
+        eng.lora_down(ctx, x, a, t_, s)                      # forward: y = x@W + (x@A * s)@B
+        eng.lora_linear(ctx, x, w, t_, b, y)
+        eng.lora_grad_down(ctx, dy, b, dt, s)                # backward 1: dx = dy@W^T + (dy@B^T * s)@A^T
+        eng.lora_linear_dx(ctx, dy, w, dt, a, dx)
+        eng.matmul_at(ctx, x, dy, dw)                        # backward 2: x^T@dy at full size, and the thin ones
+        eng.lora_grad_a(ctx, x, dt, da)
+        eng.lora_grad_b(ctx, t_, dy, db)
+        eng.flash_attention_v2_with_stats(ctx, q, k, v, o, stats, opts)
+        eng.flash_attention_v2_backward_with_stats(ctx, q, k, v, o, do, dq, dk, dv, stats, opts)
+        eng.rms_norm_eps(ctx, nx, nw, ny, 1e-5)
+        eng.rms_norm_backward(ctx, nx, nw, ng, ngx, ngw, 1e-5)
+        eng.adamw_update(ctx, pw, pg, pm, pv, adam)
+
+    for _ in range(args.warmup):
+        one_pass()
+    ctx.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        one_pass()
+    ctx.synchronize()
+    elapsed = time.perf_counter() - t0
+    check(ctx._lib.ft_profile_begin(ctx.handle))
+    for _ in range(args.steps):
+        one_pass()
+    kernels = []
+    for rec in read_profile(ctx):
+        us = rec["ms"] * 1e3 / rec["launches"]
+        if rec["flops"] > 0:
+            ach = rec["flops"] / (rec["ms"] * 1e-3) / 1e12
+            kernels.append({"kernel": rec["name"], "bound": "mfma", "launches": rec["launches"] // args.steps,
+                            "avg_us": us, "achieved": ach, "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+                            "frac": ach / FP32_MFMA_PEAK_TFLOPS})
+        else:
+            ach = rec["bytes"] / (rec["ms"] * 1e-3) / 1e9
+            kernels.append({"kernel": rec["name"], "bound": "hbm", "launches": rec["launches"] // args.steps,
+                            "avg_us": us, "achieved": ach, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                            "frac": ach / HBM_PEAK_GBS})
+    gemm = max((k_ for k_ in kernels if k_["kernel"].startswith("gemm_")), key=lambda k_: k_["avg_us"] * k_["launches"])
+    print(json.dumps({
+        "metric": "kernel microbench (BASELINE.json configs[1]): FP32-MFMA TFLOP/s of the LoRA GEMM kernel",
+        "value": gemm["achieved"], "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": elapsed / args.steps * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "kernel microbench: GEMM 2048x576x1536 (f16 B, rank-8 LoRA) fwd + 2 bwd; attention "
+                               "8x256, 9/3 heads, 64; RMSNorm 2048x576 fwd+bwd; AdamW 4M"},
+        "roofline": {"bound": "mfma", "kernel": gemm["kernel"], "achieved": gemm["achieved"],
+                     "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": gemm["frac"], "traffic": None},
+        "kernels": kernels}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="360m", choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default="360m", choices=sorted(WORKLOADS) + ["micro"])
     ap.add_argument("--micro-batch", type=int, default=0,
                     help="sequences per forward/backward pass (default: the whole batch); gradients accumulate "
                          "over the batch and one optimizer step follows, as `ferrotensor train --batch m --accum B/m`")
@@ -197,6 +288,8 @@ def main():
         sys.exit("bench.py: this build runs on ONE GPU (one process, one HIP stream); --gpus %d is not supported. "
                  "The step would shard by data parallelism over sequences with one all-reduce of the LoRA "
                  "gradients, which is not built." % args.gpus)
+    if args.workload == "micro":
+        return micro_bench(args)
     w = WORKLOADS[args.workload]
 
     from ferrotensor_amd import HipContext

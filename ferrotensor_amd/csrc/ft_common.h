@@ -32,10 +32,11 @@ struct ft_context {
 
     // Extra streams ("lanes") for work that can run beside the main stream:
     // lane 0 carries the LoRA factor gradients of a training step (only the
-    // optimizer reads them), lane 1 one of the two attention backward kernels.
-    // ft_side_begin makes a lane wait for everything enqueued on the main stream
-    // so far and redirects launches to it, ft_side_end switches back,
-    // ft_side_join makes the main stream wait for one lane or for all of them.
+    // optimizer reads them); lane 1 is free. ft_side_begin makes a lane wait for
+    // everything enqueued on the main stream so far and redirects launches to
+    // it, ft_side_end switches back, ft_side_join makes the main stream wait for
+    // one lane or for all of them. Buffers a lane still reads must not be freed
+    // or rewritten on the main stream before the join.
     static constexpr int kLanes = 2;
     hipStream_t side_stream[kLanes] = {nullptr, nullptr};
     hipEvent_t fork_event[kLanes] = {nullptr, nullptr}, join_event[kLanes] = {nullptr, nullptr};

@@ -391,6 +391,108 @@ __global__ __launch_bounds__(256) void rms_norm_backward_wave_kernel(
     }
 }
 
+// The same with the norm-weight gradient: waves stride over the rows, each lane
+// adds g*x*inv of its columns in registers, the four waves of a workgroup are
+// combined through LDS in wave order and the workgroup writes one partial row;
+// column_sum_sliced_kernel adds the partial rows in a fixed order.
+template <int NV>
+__global__ __launch_bounds__(256) void rms_norm_backward_gw_wave_kernel(
+    const float* __restrict__ x, const float* __restrict__ w, const float* __restrict__ g, float* __restrict__ gx,
+    float* __restrict__ gw_partial, int rows, int size, float eps) {
+    extern __shared__ float4 gw_lds[];  // [3][size / 4]
+    const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+    const int n4 = size / 4;
+    const float4* w4 = reinterpret_cast<const float4*>(w);
+    float4 wv[NV], acc[NV];
+#pragma unroll
+    for (int j = 0; j < NV; j++) {
+        const int i = lane + j * kWave;
+        wv[j] = i < n4 ? w4[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+        acc[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+    for (int row = blockIdx.x * 4 + wave; row < rows; row += gridDim.x * 4) {
+        const float4* x4 = reinterpret_cast<const float4*>(x + (size_t)row * size);
+        const float4* g4 = reinterpret_cast<const float4*>(g + (size_t)row * size);
+        float4 xv[NV], gv[NV];
+        float ss = 0.0f, gwx = 0.0f;
+#pragma unroll
+        for (int j = 0; j < NV; j++) {
+            const int i = lane + j * kWave;
+            if (i < n4) {
+                xv[j] = x4[i];
+                gv[j] = g4[i];
+            } else {
+                xv[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+                gv[j] = xv[j];
+            }
+            ss += xv[j].x * xv[j].x + xv[j].y * xv[j].y + xv[j].z * xv[j].z + xv[j].w * xv[j].w;
+            gwx += gv[j].x * wv[j].x * xv[j].x + gv[j].y * wv[j].y * xv[j].y + gv[j].z * wv[j].z * xv[j].z +
+                   gv[j].w * wv[j].w * xv[j].w;
+        }
+        ss = wave_sum(ss);
+        gwx = wave_sum(gwx);
+        const float inv = 1.0f / sqrtf(ss / (float)size + eps);
+        const float coef = gwx * inv * inv * inv / (float)size;
+        float4* o4 = reinterpret_cast<float4*>(gx + (size_t)row * size);
+#pragma unroll
+        for (int j = 0; j < NV; j++) {
+            const int i = lane + j * kWave;
+            if (i < n4)
+                o4[i] = make_float4(gv[j].x * wv[j].x * inv - xv[j].x * coef, gv[j].y * wv[j].y * inv - xv[j].y * coef,
+                                    gv[j].z * wv[j].z * inv - xv[j].z * coef, gv[j].w * wv[j].w * inv - xv[j].w * coef);
+            acc[j].x += gv[j].x * xv[j].x * inv;
+            acc[j].y += gv[j].y * xv[j].y * inv;
+            acc[j].z += gv[j].z * xv[j].z * inv;
+            acc[j].w += gv[j].w * xv[j].w * inv;
+        }
+    }
+    if (wave > 0) {
+#pragma unroll
+        for (int j = 0; j < NV; j++) {
+            const int i = lane + j * kWave;
+            if (i < n4) gw_lds[(wave - 1) * n4 + i] = acc[j];
+        }
+    }
+    __syncthreads();
+    if (wave == 0) {
+        float4* p4 = reinterpret_cast<float4*>(gw_partial + (size_t)blockIdx.x * size);
+#pragma unroll
+        for (int j = 0; j < NV; j++) {
+            const int i = lane + j * kWave;
+            if (i < n4) {
+                float4 s = acc[j];
+                for (int k = 0; k < 3; k++) {
+                    const float4 o = gw_lds[k * n4 + i];
+                    s = make_float4(s.x + o.x, s.y + o.y, s.z + o.z, s.w + o.w);
+                }
+                p4[i] = s;
+            }
+        }
+    }
+}
+
+// out[i] = sum of partial[p * size + i] over p: 16 columns per workgroup, the
+// partial rows dealt to 16 slices that are added in slice order (deterministic).
+__global__ __launch_bounds__(256) void column_sum_sliced_kernel(const float* __restrict__ partial,
+                                                                float* __restrict__ out, int parts, int size) {
+    __shared__ float red[16][16];
+    const int c = threadIdx.x % 16, slice = threadIdx.x / 16;
+    const int col = blockIdx.x * 16 + c;
+    float acc = 0.0f;
+    if (col < size) {
+#pragma unroll 8
+        for (int p = slice; p < parts; p += 16) acc += partial[(size_t)p * size + col];
+    }
+    red[slice][c] = acc;
+    __syncthreads();
+    if (slice == 0 && col < size) {
+        float s = red[0][c];
+#pragma unroll
+        for (int k = 1; k < 16; k++) s += red[k][c];
+        out[col] = s;
+    }
+}
+
 // ---------------------------------------------------------------------------
 // RoPE through a (cos, sin) table: the angles of a step depend only on
 // (position, i), so they are computed once (exactly as rope_kernel computes
@@ -613,6 +715,26 @@ __device__ __forceinline__ void adamw_one(float& w, float g, float& m, float& v,
     const float m_hat = m / bc1;
     const float v_hat = v / bc2;
     w = w - p.lr * (m_hat / (sqrtf(v_hat) + p.eps) + p.weight_decay * w);
+}
+
+// Four parameters per thread (16-byte accesses); n4 = number of whole float4 groups.
+__global__ __launch_bounds__(256) void adamw_vec4_kernel(float4* __restrict__ w, const float4* __restrict__ g,
+                                                         float4* __restrict__ m, float4* __restrict__ v, size_t n4,
+                                                         ft_adam_params p, float grad_scale) {
+    const float bc1 = 1.0f - powf(p.beta1, p.t);
+    const float bc2 = 1.0f - powf(p.beta2, p.t);
+    const size_t stride = (size_t)gridDim.x * 256;
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n4; i += stride) {
+        float4 wi = w[i], mi = m[i], vi = v[i];
+        const float4 gi = g[i];
+        adamw_one(wi.x, gi.x * grad_scale, mi.x, vi.x, p, bc1, bc2);
+        adamw_one(wi.y, gi.y * grad_scale, mi.y, vi.y, p, bc1, bc2);
+        adamw_one(wi.z, gi.z * grad_scale, mi.z, vi.z, p, bc1, bc2);
+        adamw_one(wi.w, gi.w * grad_scale, mi.w, vi.w, p, bc1, bc2);
+        w[i] = wi;
+        m[i] = mi;
+        v[i] = vi;
+    }
 }
 
 __global__ __launch_bounds__(256) void adamw_kernel(float* __restrict__ w, const float* __restrict__ g,
@@ -905,6 +1027,27 @@ int ft_rms_norm_backward(ft_context* ctx, const float* x, const float* w, const 
         if (gw) return ft_zero(ctx, gw, size * 4);
         return FT_OK;
     }
+    if (gw && size % 4 == 0 && size <= 2048 && rows < (1u << 30) && aligned16(x) && aligned16(w) && aligned16(g) &&
+        aligned16(gx)) {
+        size_t wgs = (rows + 3) / 4;
+        const size_t cap = (size_t)ctx->num_cus;
+        if (wgs > cap) wgs = cap;
+        float* partial = nullptr;
+        FT_TRY(ft_alloc(ctx, wgs * size * sizeof(float), (void**)&partial));
+        ft_prof_scope prof(ctx, "rms_norm_backward_gw_kernel", 0.0, 12.0 * (double)rows * size);
+        const size_t lds = 3 * size * sizeof(float);
+        if (size <= 1024)
+            hipLaunchKernelGGL((rms_norm_backward_gw_wave_kernel<4>), dim3((unsigned)wgs), dim3(256), lds, ctx->stream,
+                               x, w, g, gx, partial, (int)rows, (int)size, eps);
+        else
+            hipLaunchKernelGGL((rms_norm_backward_gw_wave_kernel<8>), dim3((unsigned)wgs), dim3(256), lds, ctx->stream,
+                               x, w, g, gx, partial, (int)rows, (int)size, eps);
+        FT_LAUNCH_CHECK();
+        hipLaunchKernelGGL(column_sum_sliced_kernel, dim3(ft_div_up(size, 16)), dim3(256), 0, ctx->stream, partial, gw,
+                           (int)wgs, (int)size);
+        FT_LAUNCH_CHECK();
+        return ft_free(ctx, partial);
+    }
     constexpr int RPW = 8;
     const size_t wgs = (rows + RPW - 1) / RPW;
     float* partial = nullptr;
@@ -993,11 +1136,26 @@ int ft_adamw_update(ft_context* ctx, float* w, const float* g, float* m, float* 
                     const ft_adam_params* p) {
     FT_CHECK_ARG(ctx && p && (n == 0 || (w && g && m && v)), "ft_adamw_update: NULL argument");
     if (n == 0) return FT_OK;
-    size_t blocks = (n + 255) / 256;
+    ft_prof_scope prof(ctx, "adamw_kernel", 0.0, 28.0 * (double)n);
     const size_t cap = (size_t)ctx->num_cus * 16;
-    if (blocks > cap) blocks = cap;
-    hipLaunchKernelGGL(adamw_kernel, dim3((unsigned)blocks), dim3(256), 0, ctx->stream, w, g, m, v, n, *p, 1.0f);
-    FT_LAUNCH_CHECK();
+    size_t done = 0;
+    if (n >= 4 && aligned16(w) && aligned16(g) && aligned16(m) && aligned16(v)) {
+        const size_t n4 = n / 4;
+        size_t blocks = (n4 + 255) / 256;
+        if (blocks > cap) blocks = cap;
+        hipLaunchKernelGGL(adamw_vec4_kernel, dim3((unsigned)blocks), dim3(256), 0, ctx->stream,
+                           reinterpret_cast<float4*>(w), reinterpret_cast<const float4*>(g),
+                           reinterpret_cast<float4*>(m), reinterpret_cast<float4*>(v), n4, *p, 1.0f);
+        FT_LAUNCH_CHECK();
+        done = n4 * 4;
+    }
+    if (done < n) {
+        size_t blocks = (n - done + 255) / 256;
+        if (blocks > cap) blocks = cap;
+        hipLaunchKernelGGL(adamw_kernel, dim3((unsigned)blocks), dim3(256), 0, ctx->stream, w + done, g + done,
+                           m + done, v + done, n - done, *p, 1.0f);
+        FT_LAUNCH_CHECK();
+    }
     return FT_OK;
 }
 

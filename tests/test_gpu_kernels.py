@@ -258,7 +258,7 @@ def test_fused_gated_mlp_halves(g, M, H, F, f16):
 
 
 @pytest.mark.parametrize("rows,size", [(1, 1), (3, 7), (37, 96), (16, 576), (64, 960), (5, 2048), (3, 2100),
-                                       (2048, 576)])
+                                       (2048, 576), (4100, 960), (2500, 1536)])
 def test_rms_norm_forward_backward(g, rows, size):
     ctx, eng = g
     x, w, gy = rnd(1, rows, size), rnd(2, size), rnd(3, rows, size)
