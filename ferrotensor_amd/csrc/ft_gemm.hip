@@ -19,6 +19,8 @@
 #include "ft_common.h"
 #include "ft_thin.h"
 
+#include <cmath>
+
 namespace {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
@@ -577,7 +579,7 @@ struct AsyncProb {
     float* out3;
     const float* e1;
     const float* e2;
-    int N, ldc, tiles_n, tile_begin, nseg;
+    int N, ldc, tile_begin, nseg;  // tile_begin: first n tile of this product in the batch's row of n tiles
     long partial_off;  // split-K: this product's slice of AsyncBatch::partial, [splits][M][N]
     // RoPE on the output (64x64 tiles, head_dim 64, so a tile is one head of 64 rows): element
     // (row, h*64 + i) pairs with (row, h*64 + i + 32) and rotates by the (cos, sin) of token position
@@ -596,6 +598,9 @@ struct AsyncBatch {
     int count, M;
     int splits;        // 1 = none
     float* partial;
+    int tiles_m, tiles_n;  // row blocks; n tiles of all products together
+    int xcds;              // chunks of the tile order (one per XCD), 1 = workgroup id order
+    int panel;             // n tiles per panel of the tile order
 };
 
 template <int NSEG, typename T>
@@ -657,14 +662,31 @@ __global__ __launch_bounds__(256) void gemm_async_kernel(AsyncBatch g) {
     __shared__ __attribute__((aligned(16))) float ExAs[NB == 1 ? ExA::LDS_FLOATS : 4];
     __shared__ __attribute__((aligned(16))) float ExBs[NB == 1 ? ExB::LDS_FLOATS : 4];
 
+    // Workgroup -> tile. The products of a batch form one row of n tiles per row block
+    // (tile_begin = a product's first n tile). Tile order: panels of `panel` n tiles; inside a
+    // panel row block after row block. Consecutive workgroup ids go to different XCDs, each with
+    // its own L2: XCD x takes the x-th contiguous chunk of that order, so the workgroups resident
+    // on one XCD cover a compact block of rows and columns and share their operand tiles in L2.
+    int bid = (int)blockIdx.x;
+    if (g.xcds > 1) {
+        const int total = (int)gridDim.x, x = bid % g.xcds, q = total / g.xcds, r = total % g.xcds;
+        bid = x * q + (x < r ? x : r) + bid / g.xcds;
+    }
+    const int per_panel = g.tiles_m * g.panel;
+    const int last = (g.tiles_n - 1) / g.panel;
+    int pnl = bid / per_panel;
+    pnl = pnl < last ? pnl : last;
+    const int rem = bid - pnl * per_panel;
+    const int width = pnl == last ? g.tiles_n - last * g.panel : g.panel;
+    const int tm = rem / width;
+    const int tn = pnl * g.panel + rem % width;
     int pi = 0;
-    if (g.count > 1 && (int)blockIdx.x >= g.p[1].tile_begin) pi = 1;
-    if (g.count > 2 && (int)blockIdx.x >= g.p[2].tile_begin) pi = 2;
+    if (g.count > 1 && tn >= g.p[1].tile_begin) pi = 1;
+    if (g.count > 2 && tn >= g.p[2].tile_begin) pi = 2;
     const AsyncProb& p = g.p[pi];
     const int M = g.M;
-    const int tile = (int)blockIdx.x - p.tile_begin;
-    const int m0 = (tile / p.tiles_n) * BM;
-    const int n0 = (tile % p.tiles_n) * BN;
+    const int m0 = tm * BM;
+    const int n0 = (tn - p.tile_begin) * BN;
     const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
     const int wm0 = (wave / WAVES_N) * WM, wn0 = (wave % WAVES_N) * WN;
     const int l32 = lane % 32, half = lane / 32;
@@ -1043,23 +1065,48 @@ __global__ __launch_bounds__(256) void skinny_kernel(const float* __restrict__ x
 
 constexpr size_t kSplitScratchFloats = (size_t)16 << 20;  // 64 MiB of split-K partial tiles
 
+// XCDs of the device (MI355X: 8 of 32 CUs, each with its own L2).
+static int ft_gemm_xcds(ft_context* ctx) { return ctx->num_cus % 8 == 0 && ctx->num_cus >= 64 ? 8 : 1; }
+
 template <int BM, int BN, int WM, int WN>
 int launch_async(ft_context* ctx, AsyncBatch g, int layout, int epi = kEpiPlain) {
     const int tiles_m = (g.M + BM - 1) / BM;
-    int tiles = 0, max_seg = 1;
-    double flops = 0.0, bytes = 0.0;
+    int tiles_n = 0, max_seg = 1;
+    double flops = 0.0, bytes = 0.0, a_bytes = 0.0, b_bytes = 0.0;
     for (int i = 0; i < g.count; i++) {
         AsyncProb& p = g.p[i];
-        p.tiles_n = (p.N + BN - 1) / BN;
-        p.tile_begin = tiles;
-        tiles += tiles_m * p.tiles_n;
+        p.tile_begin = tiles_n;
+        tiles_n += (p.N + BN - 1) / BN;
         if (p.nseg > max_seg) max_seg = p.nseg;
+        double a_this = 0.0;  // the products of a batch share their a operand
+        for (int s = 0; s < p.nseg; s++) {
+            a_this += 4.0 * g.M * 32.0 * p.seg[s].nt;
+            b_bytes += 2.0 * p.N * 32.0 * p.seg[s].nt * (epi == kEpiGateUp ? 2 : 1);
+        }
+        if (a_this > a_bytes) a_bytes = a_this;
         for (int s = 0; s < p.nseg; s++) {
             const double k = 32.0 * p.seg[s].nt, k2 = p.seg[s].a2 ? (double)p.seg[s].K2 : 0.0;
             flops += 2.0 * g.M * (double)p.N * (k + k2);
             bytes += 4.0 * g.M * (k + k2) + 2.0 * p.N * k + 4.0 * p.N * k2;
         }
         bytes += (p.add ? 8.0 : 4.0) * g.M * (double)p.N;
+    }
+    const int tiles = tiles_m * tiles_n;
+    g.tiles_m = tiles_m;
+    g.tiles_n = tiles_n;
+    // Panel width: the tiles resident on one XCD at a time (32 CUs x workgroups per CU) should
+    // need about as many bytes of a (rows x a_bytes per row block) as of b (columns x b_bytes
+    // per n tile).
+    g.xcds = ft_gemm_xcds(ctx);
+    {
+        const double resident = 32.0 * (BM == 64 ? 3 : 2);
+        const double a_blk = a_bytes / tiles_m, b_blk = b_bytes / (tiles_n > 0 ? tiles_n : 1);
+        int want = b_blk > 0 ? (int)(sqrt(resident * a_blk / b_blk) + 0.5) : tiles_n;
+        if (want < 1) want = 1;
+        int panels = (int)((double)tiles_n / want + 0.5);
+        if (panels < 1) panels = 1;
+        g.panel = (tiles_n + panels - 1) / panels;
+        if (g.panel < 1) g.panel = 1;
     }
     g.splits = 1;
     g.partial = nullptr;
@@ -1077,7 +1124,7 @@ int launch_async(ft_context* ctx, AsyncBatch g, int layout, int epi = kEpiPlain)
     }
     bool any_rope = false;
     for (int i = 0; i < g.count; i++) any_rope = any_rope || g.p[i].rope != nullptr;
-    if (epi == kEpiPlain && mn4 && !any_rope && tiles > 0 && (size_t)tiles * 2 <= (size_t)ctx->num_cus) {
+    if (epi == kEpiPlain && mn4 && !any_rope && tiles > 0 && (size_t)tiles * 4 <= (size_t)ctx->num_cus * 5) {
         int want = (int)((2 * (size_t)ctx->num_cus + tiles - 1) / tiles);
         if (want > 8) want = 8;
         if (want > min_kt / 4) want = min_kt / 4;
