@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """LoRA train step benchmark on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload 360m|135m|1.7b|tiny|micro]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload 360m|135m|1.7b|tiny|micro|probe]
 
 A step is one full optimizer step (forward, masked cross-entropy, backward,
 gradient norm, clip, AdamW) of the SmolLM2-360M-shaped model on 8 sequences x
@@ -281,12 +281,51 @@ def micro_bench(args):
         "kernels": kernels}))
 
 
+def mfma_probe(args):
+    """What the FP32 matrix pipes sustain with no memory traffic at all: short and long launches, one to
+    three waves per SIMD, dependent (1 chain) and independent (4 chains) accumulators."""
+    from ferrotensor_amd import HipContext
+
+    ctx = HipContext(0)
+    runs = []
+    for random_operands in (False, True):
+        for waves in (1, 2, 3):
+            for chains in (1, 4):
+                for rounds in (100, 1000, 10000, 100000):
+                    ctx.mfma_probe(rounds, waves, chains, random_operands)
+                    best = None
+                    for _ in range(3 if rounds < 100000 else 2):
+                        s, f = ctx.mfma_probe(rounds, waves, chains, random_operands)
+                        best = s if best is None or s < best else best
+                    runs.append({"operands": "random" if random_operands else "ones", "waves_per_simd": waves,
+                                 "chains": chains, "mfma_per_wave": rounds * 16, "us": best * 1e6,
+                                 "tflops": f / best / 1e12})
+    # A back-to-back train of 1.6 ms launches for about a second: the rate under continuous load.
+    t0 = time.perf_counter()
+    n, total_s, total_f = 0, 0.0, 0.0
+    while time.perf_counter() - t0 < 1.0:
+        s, f = ctx.mfma_probe(10000, 2, 4, True)
+        total_s, total_f, n = total_s + s, total_f + f, n + 1
+    sustained = total_f / total_s / 1e12
+    best = max(r["tflops"] for r in runs)
+    print(json.dumps({
+        "metric": "FP32 MFMA rate of a register-only v_mfma_f32_32x32x2_f32 loop", "value": sustained,
+        "unit": "TFLOP/s", "n_gpus": 1, "steps": n, "warmup": 0, "ms_per_step": total_s / n * 1e3,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "matrix-pipe probe: %d launches of 160000 MFMAs per wave, 2 waves per SIMD, "
+                               "4 independent accumulators, pseudo-random operands" % n},
+        "roofline": {"bound": "mfma", "kernel": "mfma_probe_kernel<4>", "achieved": sustained,
+                     "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": sustained / FP32_MFMA_PEAK_TFLOPS,
+                     "traffic": None},
+        "best_single_launch_tflops": best, "runs": runs}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="360m", choices=sorted(WORKLOADS) + ["micro"])
+    ap.add_argument("--workload", default="360m", choices=sorted(WORKLOADS) + ["micro", "probe"])
     ap.add_argument("--micro-batch", type=int, default=0,
                     help="sequences per forward/backward pass (default: the whole batch); gradients accumulate "
                          "over the batch and one optimizer step follows, as `ferrotensor train --batch m --accum B/m`")
@@ -299,6 +338,8 @@ def main():
                  "gradients, which is not built." % args.gpus)
     if args.workload == "micro":
         return micro_bench(args)
+    if args.workload == "probe":
+        return mfma_probe(args)
     w = WORKLOADS[args.workload]
 
     from ferrotensor_amd import HipContext

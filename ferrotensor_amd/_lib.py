@@ -73,6 +73,7 @@ SIGNATURES = {
     "ft_profile_end": [_P, C.POINTER(_SZ)],
     "ft_profile_kernel": [_P, _SZ, C.POINTER(C.c_char_p), C.POINTER(C.c_uint64), C.POINTER(C.c_double),
                           C.POINTER(C.c_double), C.POINTER(C.c_double)],
+    "ft_mfma_probe": [_P, _SZ, _SZ, _SZ, C.c_int, C.POINTER(C.c_double), C.POINTER(C.c_double)],
     "ft_alloc": [_P, _SZ, C.POINTER(_P)],
     "ft_free": [_P, _P],
     "ft_pool_trim": [_P],

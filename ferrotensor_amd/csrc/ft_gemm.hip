@@ -525,10 +525,11 @@ __global__ __launch_bounds__(256) void gemm_fast_kernel(GemmArgs p) {
 // A lane's 16 bytes land at (LDS base of the instruction) + 16 * lane, so the
 // LDS image of a tile is fixed by which global address each lane is given:
 //   a tile   [BM rows][32 k] f32, 128 B per row, 8 rows per instruction; the
-//            16-byte column c of row r holds k-quad c ^ (r & 7), which makes the
-//            ds_read_b128 of 8 consecutive rows hit 8 different bank groups.
+//            16-byte column c of row r holds k-quad c ^ ((r >> 1) & 7): measured, this
+//            is the swizzle with which the ds_read_b128 of a wave (32 rows x 2 k-quads)
+//            runs at the rate of a linear read (c ^ (r & 7) takes twice as long).
 //   b tile   layout 1 (b[N,K]): [BN rows][32 k] f16, 64 B per row, 16 rows per
-//            instruction, 16-byte column c holds k-octet c ^ ((r >> 1) & 3).
+//            instruction, 16-byte column c holds k-octet c ^ ((r >> 2) & 3) (likewise measured).
 //            layout 0 (b[K,N]): [32 k][BN n] f16 exactly as in memory; a lane
 //            reads its column's 4 k values as four 16-bit loads.
 // The K loop is unrolled over the stages; the waits are explicit (s_waitcnt
@@ -749,7 +750,7 @@ __global__ __launch_bounds__(256) void gemm_async_kernel(AsyncBatch g) {
         int row = m0 + 8 * c + r;
         row = row < M ? row : M - 1;
         rowA[j] = (unsigned)row;
-        colA[j] = (unsigned)((cs ^ r) * 16);
+        colA[j] = (unsigned)((cs ^ ((4 * c + (r >> 1)) & 7)) * 16);
         offA[j] = rowA[j] * (unsigned)lda_b[0] + colA[j];
     }
 #pragma unroll
@@ -760,7 +761,7 @@ __global__ __launch_bounds__(256) void gemm_async_kernel(AsyncBatch g) {
             int n = n0 + 16 * c + r;
             n = n < p.N ? n : p.N - 1;
             rowB[j] = (unsigned)n;
-            colB[j] = (unsigned)((cs ^ ((r >> 1) & 3)) * 16);
+            colB[j] = (unsigned)((cs ^ ((r >> 2) & 3)) * 16);
         } else {
             constexpr int LPR = BN / 8, RPC = 64 / LPR;
             const int kr = lane / LPR, cs = lane % LPR;
@@ -811,13 +812,13 @@ __global__ __launch_bounds__(256) void gemm_async_kernel(AsyncBatch g) {
     };
     auto a_frag = [&](const float* st, int s, int row) -> float4 {
         const int kq = 2 * s + half;
-        return *reinterpret_cast<const float4*>(st + row * 32 + ((kq ^ (row & 7)) * 4));
+        return *reinterpret_cast<const float4*>(st + row * 32 + ((kq ^ ((row >> 1) & 7)) * 4));
     };
     auto b_frag = [&](const float* st, int s, int n, int jb) -> float4 {
         const char* bs = reinterpret_cast<const char*>(st + A_FLOATS + jb * B_FLOATS);
         if constexpr (LAYOUT == 1) {
             const int kq = 2 * s + half;
-            const int col = (kq >> 1) ^ ((n >> 1) & 3);
+            const int col = (kq >> 1) ^ ((n >> 2) & 3);
             const half4_t h = *reinterpret_cast<const half4_t*>(bs + n * 64 + col * 16 + (kq & 1) * 8);
             return make_float4((float)h.x, (float)h.y, (float)h.z, (float)h.w);
         } else {
@@ -1057,6 +1058,47 @@ __global__ __launch_bounds__(256) void skinny_kernel(const float* __restrict__ x
         const int i = e / 32, j = e % 32;
         emit(i, j, ((red[0][i * 33 + j] + red[1][i * 33 + j]) + red[2][i * 33 + j]) + red[3][i * 33 + j]);
     }
+}
+
+// ---------------------------------------------------------------------------
+// Matrix-pipe probe: v_mfma_f32_32x32x2_f32 on register operands only, no memory
+// traffic inside the loop. CHAINS independent accumulators per wave (1 = every
+// MFMA depends on the one before, as in a 32x32 wave tile). Measures what the
+// matrix pipes sustain, the ceiling the GEMM kernels are compared with.
+// ---------------------------------------------------------------------------
+template <int CHAINS>
+__global__ __launch_bounds__(256) void mfma_probe_kernel(float* __restrict__ out, int rounds, int random_operands) {
+    floatx16 acc[CHAINS];
+#pragma unroll
+    for (int c = 0; c < CHAINS; c++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[c][r] = 0.0f;
+    // Operands: 16 pairs of pseudo-random values in (-1, 1) per lane, as a GEMM on N(0,1)-like
+    // data would feed (the power a matrix pipe draws depends on how many operand bits toggle).
+    float a[16], b[16];
+    unsigned h = (blockIdx.x * 256u + threadIdx.x) * 2654435761u + 12345u;
+#pragma unroll
+    for (int u = 0; u < 16; u++) {
+        h = h * 1664525u + 1013904223u;
+        a[u] = random_operands ? (float)(int)(h >> 8) * (1.0f / 8388608.0f) - 1.0f : 1.0f;
+        h = h * 1664525u + 1013904223u;
+        b[u] = random_operands ? (float)(int)(h >> 8) * (1.0f / 8388608.0f) - 1.0f : 1.0f;
+    }
+    for (int i = 0; i < rounds; i++) {
+#pragma unroll
+        for (int u = 0; u < 16 / CHAINS; u++)
+#pragma unroll
+            for (int c = 0; c < CHAINS; c++)
+                acc[c] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u * CHAINS + c], b[u * CHAINS + c], acc[c], 0, 0, 0);
+#pragma unroll
+        for (int u = 0; u < 16; u++) asm volatile("" : "+v"(a[u]), "+v"(b[u]));  // opaque: nothing to hoist
+    }
+    float s = 0.0f;
+#pragma unroll
+    for (int c = 0; c < CHAINS; c++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) s += acc[c][r];
+    out[(size_t)blockIdx.x * 256 + threadIdx.x] = s;
 }
 
 // ---------------------------------------------------------------------------
@@ -1360,6 +1402,46 @@ int skinny_launch(ft_context* ctx, const float* x, const float* y, float* out, s
 }  // namespace
 
 extern "C" {
+
+int ft_mfma_probe(ft_context* ctx, size_t rounds, size_t waves_per_simd, size_t chains, int random_operands,
+                  double* seconds, double* flops) {
+    FT_CHECK_ARG(ctx && seconds && flops, "ft_mfma_probe: NULL argument");
+    FT_CHECK_ARG(rounds >= 1 && rounds <= (1u << 24), "ft_mfma_probe: rounds %zu is outside 1..2^24", rounds);
+    FT_CHECK_ARG(waves_per_simd >= 1 && waves_per_simd <= 4, "ft_mfma_probe: waves_per_simd %zu is outside 1..4",
+                 waves_per_simd);
+    FT_CHECK_ARG(chains == 1 || chains == 2 || chains == 4, "ft_mfma_probe: chains must be 1, 2 or 4");
+    const size_t wgs = (size_t)ctx->num_cus * waves_per_simd;  // 256 threads = one wave per SIMD of a CU
+    float* out = nullptr;
+    FT_TRY(ft_alloc(ctx, wgs * 256 * sizeof(float), (void**)&out));
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    float ms = 0.0f;
+    hipError_t err = hipEventCreate(&e0);
+    if (err == hipSuccess) err = hipEventCreate(&e1);
+    if (err == hipSuccess) err = hipEventRecord(e0, ctx->stream);
+    if (err == hipSuccess) {
+        const dim3 grid((unsigned)wgs);
+        if (chains == 1)
+            hipLaunchKernelGGL(mfma_probe_kernel<1>, grid, dim3(256), 0, ctx->stream, out, (int)rounds,
+                               random_operands);
+        else if (chains == 2)
+            hipLaunchKernelGGL(mfma_probe_kernel<2>, grid, dim3(256), 0, ctx->stream, out, (int)rounds,
+                               random_operands);
+        else
+            hipLaunchKernelGGL(mfma_probe_kernel<4>, grid, dim3(256), 0, ctx->stream, out, (int)rounds,
+                               random_operands);
+        err = hipGetLastError();
+    }
+    if (err == hipSuccess) err = hipEventRecord(e1, ctx->stream);
+    if (err == hipSuccess) err = hipEventSynchronize(e1);
+    if (err == hipSuccess) err = hipEventElapsedTime(&ms, e0, e1);
+    if (e0) (void)hipEventDestroy(e0);
+    if (e1) (void)hipEventDestroy(e1);
+    FT_TRY(ft_free(ctx, out));
+    FT_HIP(err);
+    *seconds = (double)ms * 1e-3;
+    *flops = (double)wgs * 4.0 * (double)rounds * 16.0 * 4096.0;  // waves x MFMAs x 2*32*32*2
+    return FT_OK;
+}
 
 int ft_matmul(ft_context* ctx, const float* a, const float* b, float* out, size_t M, size_t K, size_t N) {
     return gemm_dispatch(ctx, "ft_matmul", 0, false, a, b, out, M, K, N, nullptr, nullptr, 0);

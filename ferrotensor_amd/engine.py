@@ -78,6 +78,13 @@ class HipContext:
     def stream(self) -> int:
         return int(self._lib.ft_context_stream(self.handle) or 0)
 
+    def mfma_probe(self, rounds, waves_per_simd=2, chains=4, random_operands=True):
+        """(seconds, flops) of one launch of the register-only FP32 MFMA loop."""
+        s, f = C.c_double(), C.c_double()
+        check(self._lib.ft_mfma_probe(self.handle, rounds, waves_per_simd, chains, 1 if random_operands else 0,
+                                      C.byref(s), C.byref(f)))
+        return s.value, f.value
+
     def pool_stats(self):
         live, idle = C.c_size_t(), C.c_size_t()
         check(self._lib.ft_pool_stats(self.handle, C.byref(live), C.byref(idle)))

@@ -85,6 +85,16 @@ int ft_profile_end(ft_context* ctx, size_t* kernels);
 int ft_profile_kernel(ft_context* ctx, size_t index, const char** name, uint64_t* launches,
                       double* total_ms, double* flops, double* bytes);
 
+/* Diagnostic with no counterpart in the reference: runs `rounds` x 16
+ * v_mfma_f32_32x32x2_f32 per wave on register operands (no memory traffic) with
+ * `waves_per_simd` (1..4) waves on every SIMD and `chains` (1, 2 or 4)
+ * independent accumulators per wave, on operands that are all 1.0 or
+ * (`random_operands` != 0) pseudo-random in (-1, 1), and reports the HIP-event time of the one
+ * launch and the flops it executed: the rate the FP32 matrix pipes sustain, the
+ * ceiling GEMM kernels are compared with. Waits for the stream. */
+int ft_mfma_probe(ft_context* ctx, size_t rounds, size_t waves_per_simd, size_t chains, int random_operands,
+                  double* seconds, double* flops);
+
 /* ---- buffers: UnifiedTensor storage + BufferPool (tensor.rs, pool.rs) ---- */
 
 /* UnifiedTensor::empty (tensor.rs:184-210): uninitialised device buffer from

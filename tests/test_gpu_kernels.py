@@ -395,6 +395,22 @@ def test_adamw_four_million_parameters(g):
     assert_close("adamw v", tv.to_numpy(), v, atol=1e-7, rtol=1e-5)
 
 
+def test_mfma_probe_reports_time_and_flops(g):
+    """The matrix-pipe probe runs the stated number of MFMAs (4096 flop each) and its rate stays under the peak."""
+    from ferrotensor_amd import FtError
+    ctx, _ = g
+    seconds, flops = ctx.mfma_probe(200, waves_per_simd=2, chains=4)
+    waves = 256 * 2 * 4
+    assert flops == waves * 200 * 16 * 4096.0
+    assert seconds > 0 and flops / seconds < 157.3e12 * 1.02
+    s1, _ = ctx.mfma_probe(200, waves_per_simd=1, chains=1, random_operands=False)
+    assert s1 > 0
+    with pytest.raises(FtError):
+        ctx.mfma_probe(10, waves_per_simd=9)
+    with pytest.raises(FtError):
+        ctx.mfma_probe(10, chains=3)
+
+
 def test_errors_are_reported_not_fatal(g):
     from ferrotensor_amd import FtError
     ctx, eng = g
