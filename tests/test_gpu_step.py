@@ -367,6 +367,74 @@ def test_micro_batches_accumulate_to_the_batched_step(ctx):
             assert_close("param " + k, p[k], p0[k], atol=1e-6, rtol=1e-4)
 
 
+def test_training_on_one_batch_halves_the_loss(ctx):
+    """`lora_training_reduces_loss_on_a_tiny_model` (ferrotensor-trainer/tests/gpu_training.rs:24-54): a tiny
+    model with weights of the reference test's scale (embedding 0.5, linears 0.2, tests/common/mod.rs:102-118),
+    freshly seeded rank-4 adapters on q/k/v/o, one memorisable sequence ((7i + 3) mod 64, common/mod.rs:370-372),
+    AdamW at 1e-2: 40 optimizer steps at least halve the loss."""
+    from ferrotensor_amd.trainer import Lfm2Model, ModelConfig, Trainer
+    cfg = ModelConfig(vocab_size=64, hidden_size=32, intermediate_size=64, num_hidden_layers=2,
+                      num_attention_heads=4, num_key_value_heads=2, rms_norm_eps=1e-5, rope_theta=10000.0,
+                      tie_word_embeddings=False, f16_linears=False)
+    tensors = random_model_tensors(cfg, 3)
+    rng = np.random.default_rng(17)
+    for name, w in tensors.items():
+        if name.endswith("norm.weight") or name.endswith("layernorm.weight"):
+            continue
+        scale = 0.5 if "embed_tokens" in name else 0.2
+        tensors[name] = rng.uniform(-scale, scale, w.shape).astype(np.float32)
+    hip = Lfm2Model(ctx, cfg)
+    hip.load_tensors(tensors)
+    for prefix in hip.linear_prefixes(["q_proj", "k_proj", "v_proj", "o_proj"]):
+        hip.add_lora(prefix, 4, 8.0)
+    seq = np.array([(i * 7 + 3) % 64 for i in range(24)], np.uint32)
+    rows, targets = seq[None, :-1], seq[None, 1:]
+    masks = np.ones_like(rows, dtype=np.uint8)
+    tr = Trainer(hip, lr=1e-2, grad_accum_steps=1)
+    losses = []
+    for _ in range(40):
+        st = tr.train_chunk(rows, targets, masks)
+        assert st.optimizer_step
+        losses.append(st.loss)
+    tr.close()
+    hip.close()
+    assert all(np.isfinite(losses))
+    assert losses[-1] < 0.5 * losses[0], losses
+
+
+def test_the_step_is_deterministic_to_the_bit(ctx):
+    """Two runs of the same three steps from the same state give the same bits in every gradient, weight and
+    moment (gpu_training.rs:224-253): every reduction of the step has a fixed order, including the factor
+    gradients computed on the second stream and the split-K partial sums."""
+    from ferrotensor_amd.trainer import Trainer
+    mods = ["q_proj", "k_proj", "v_proj", "o_proj"]
+    rng = np.random.default_rng(6)
+    rows = rng.integers(0, 256, (3, 64)).astype(np.uint32)
+    targets = np.concatenate([rows[:, 1:], rows[:, :1]], axis=1)
+    masks = (rng.random((3, 64)) > 0.3).astype(np.uint8)
+    from ferrotensor_amd import checkpoint as ck
+    from ferrotensor_amd.trainer import ModelConfig
+    cfg = ModelConfig(vocab_size=256, hidden_size=192, intermediate_size=256, num_hidden_layers=2,
+                      num_attention_heads=3, num_key_value_heads=1, rms_norm_eps=1e-5, rope_theta=100000.0,
+                      tie_word_embeddings=True, f16_linears=True)
+    runs = []
+    for _ in range(2):
+        hip, _ = build_pair(ctx, cfg, mods, rank=8, alpha=16.0, seed=41)
+        tr = Trainer(hip, lr=1e-3, weight_decay=0.01, clip_grad_norm=1.0, grad_accum_steps=3)
+        stats = [tr.train_chunk(rows, targets, masks) for _ in range(3)]
+        adam = ck.optimizer_state(tr)
+        runs.append(([(s.loss, s.grad_norm) for s in stats], hip.grads(), hip.params(), adam.m_states,
+                     adam.v_states))
+        tr.close()
+        hip.close()
+    a, b = runs
+    assert a[0] == b[0]
+    for x, y in zip(a[1:], b[1:]):
+        assert x.keys() == y.keys()
+        for k in x:
+            assert np.array_equal(np.asarray(x[k]).view(np.uint32), np.asarray(y[k]).view(np.uint32)), k
+
+
 def test_evaluate_is_the_token_weighted_forward_loss(ctx):
     """`evaluate` (ferrotensor-cli/src/main.rs:1110-1137): sum(loss_i * n_i) / sum(n_i) over ragged
     examples, forward only: parameters and gradients are untouched."""
