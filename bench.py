@@ -105,16 +105,17 @@ def lora_factors(model, w, seed=2):
         yield name, a, b
 
 
-def step_flops(w):
+def step_flops(w, head_rows=None):
     """Algorithmic flops of one step (SURVEY convention): fwd + dX GEMMs on the
-    frozen base incl. the head, LoRA products, attention fwd + 2.5x bwd."""
+    frozen base incl. the head, LoRA products, attention fwd + 2.5x bwd. The head
+    (and its input gradient) runs on `head_rows` rows: the supervised positions."""
     T = w["B"] * w["S"]
     H, F, V, L = w["hidden"], w["ffn"], w["vocab"], w["layers"]
     D = H // w["heads"]
     p_layer = H * w["heads"] * D * 2 + H * w["kv"] * D * 2 + 3 * H * F
-    p_lin = L * p_layer + H * V
+    head_rows = T if head_rows is None else head_rows
     attn = 2.0 * w["B"] * w["heads"] * w["S"] ** 2 * D * 3.5 * L
-    return 2 * (2.0 * T * p_lin) + attn
+    return 2 * (2.0 * T * L * p_layer + 2.0 * head_rows * H * V) + attn
 
 
 def read_profile(ctx):
@@ -413,9 +414,10 @@ def main():
         "config": {"workload": w["label"], "global_batch": w["B"], "seq_len": w["S"], "micro_batch": mb,
                    "lora": "rank %d alpha %g on %s" % (w["rank"], w["alpha"], "/".join(w["targets"])),
                    "base_weights": "f16 storage, f32 arithmetic", "optimizer": "AdamW lr 2e-4 wd 0 clip 1.0",
-                   "supervised_tokens": int(st.tokens), "loss": float(st.loss)},
-        "step_tflops": step_flops(w) / (elapsed / args.steps) / 1e12,
-        "step_mfma_frac": step_flops(w) / (elapsed / args.steps) / 1e12 / FP32_MFMA_PEAK_TFLOPS,
+                   "supervised_tokens": int(st.tokens), "loss": float(st.loss),
+                   "head": "final norm, vocabulary head and loss on the %d supervised positions" % int(st.tokens)},
+        "step_tflops": step_flops(w, int(st.tokens)) / (elapsed / args.steps) / 1e12,
+        "step_mfma_frac": step_flops(w, int(st.tokens)) / (elapsed / args.steps) / 1e12 / FP32_MFMA_PEAK_TFLOPS,
         "roofline": {"bound": "mfma", "kernel": dom["name"], "achieved": achieved, "peak": FP32_MFMA_PEAK_TFLOPS,
                      "unit": "TFLOP/s", "frac": achieved / FP32_MFMA_PEAK_TFLOPS,
                      "traffic": measured_traffic(dom["name"], args.workload),

@@ -1166,7 +1166,11 @@ int launch_async(ft_context* ctx, AsyncBatch g, int layout, int epi = kEpiPlain)
     }
     bool any_rope = false;
     for (int i = 0; i < g.count; i++) any_rope = any_rope || g.p[i].rope != nullptr;
-    if (epi == kEpiPlain && mn4 && !any_rope && tiles > 0 && (size_t)tiles * 4 <= (size_t)ctx->num_cus * 5) {
+    // Also with fewer than 1.5 tiles per CU when K is very long (the head's input gradient, K = vocabulary):
+    // the extra pass over the output is then a fraction of a percent.
+    const bool few_tiles = (size_t)tiles * 4 <= (size_t)ctx->num_cus * 5;
+    const bool long_k = (size_t)tiles * 2 < 3 * (size_t)ctx->num_cus && min_kt >= 512;
+    if (epi == kEpiPlain && mn4 && !any_rope && tiles > 0 && (few_tiles || long_k)) {
         int want = (int)((2 * (size_t)ctx->num_cus + tiles - 1) / tiles);
         if (want > 8) want = 8;
         if (want > min_kt / 4) want = min_kt / 4;

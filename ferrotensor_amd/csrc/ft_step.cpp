@@ -113,6 +113,12 @@ struct ft_model {
     float *x_final = nullptr, *hf = nullptr, *thead = nullptr, *logits = nullptr;
     uint32_t *ids_dev = nullptr, *targets_dev = nullptr;
     float *weights_dev = nullptr, *row_loss = nullptr;
+    // Head on the supervised rows only: head_idx[k] = k-th supervised row, head_inv[row] = its k
+    // (or head_rows for an unsupervised row, which gathers as a zero row), xc = those rows of x_final.
+    uint32_t *head_idx_dev = nullptr, *head_inv_dev = nullptr;
+    float* xc = nullptr;
+    size_t head_rows = 0;        // rows the head ran on in the last forward
+    bool head_compact = false;   // whether they are a gathered subset
     // backward scratch
     float *g0 = nullptr, *g1 = nullptr, *d_act = nullptr, *d_gate = nullptr, *d_up = nullptr, *d_h2 = nullptr,
           *d_attn = nullptr, *dq = nullptr, *dk = nullptr, *dv = nullptr, *d_h1 = nullptr, *dt = nullptr,
@@ -207,6 +213,9 @@ int ensure_workspace(ft_model* m, size_t B, size_t S) {
     FT_TRY(ws_alloc(m, T, (float**)&m->targets_dev));
     FT_TRY(ws_alloc(m, T, &m->weights_dev));
     FT_TRY(ws_alloc(m, T, &m->row_loss));
+    FT_TRY(ws_alloc(m, T, (float**)&m->head_idx_dev));
+    FT_TRY(ws_alloc(m, T, (float**)&m->head_inv_dev));
+    FT_TRY(ws_alloc(m, T * H, &m->xc));
     FT_TRY(ws_alloc(m, T * H, &m->g0));
     FT_TRY(ws_alloc(m, T * H, &m->g1));
     FT_TRY(ws_alloc(m, T * F, &m->d_act));
@@ -456,7 +465,12 @@ int layer_forward(ft_model* m, size_t l, size_t B, size_t S) {
     return FT_OK;
 }
 
-int model_forward(ft_model* m, const uint32_t* rows_host, size_t B, size_t S) {
+// `head` (optional): the rows whose logits are needed, ascending. The final norm and the
+// vocabulary head then run on those rows only (logits, row losses and d_logits are [head->size(), V]):
+// a row without a supervised target has zero loss and a zero logits gradient whatever its logits are
+// (masked_cross_entropy, kernels.wgsl:684-711), so leaving it out changes no bit of the result.
+int model_forward(ft_model* m, const uint32_t* rows_host, size_t B, size_t S,
+                  const std::vector<uint32_t>* head = nullptr) {
     ft_context* ctx = m->ctx;
     const ft_model_config& c = m->cfg;
     FT_CHECK_ARG(m->embed && m->norm_f && m->lm_head.w, "model is missing embed_tokens, norm or lm_head weights");
@@ -476,8 +490,25 @@ int model_forward(ft_model* m, const uint32_t* rows_host, size_t B, size_t S) {
     ft_attention_options opts{};
     opts.causal = 1;
     for (size_t l = 0; l < m->layers.size(); l++) FT_TRY(layer_forward(m, l, B, S));
-    FT_TRY(ft_rms_norm_eps(ctx, m->x_final, m->norm_f, m->hf, T, H, c.rms_norm_eps));
-    FT_TRY(linear_forward(ctx, m->lm_head, m->hf, m->thead, m->logits, T));
+    const float* xf = m->x_final;
+    m->head_rows = T;
+    m->head_compact = head != nullptr && head->size() < T;
+    if (m->head_compact) {
+        m->head_rows = head->size();
+        std::vector<uint32_t> inv(T, (uint32_t)head->size());
+        for (size_t k = 0; k < head->size(); k++) {
+            FT_CHECK_ARG((*head)[k] < T && (k == 0 || (*head)[k] > (*head)[k - 1]), "head rows must ascend within the chunk");
+            inv[(*head)[k]] = (uint32_t)k;
+        }
+        FT_TRY(ft_upload(ctx, m->head_idx_dev, head->data(), head->size() * sizeof(uint32_t)));
+        FT_TRY(ft_upload(ctx, m->head_inv_dev, inv.data(), T * sizeof(uint32_t)));
+        // gather: row k of xc = row head[k] of x_final
+        FT_TRY(ft_embedding(ctx, m->x_final, T, H, m->head_idx_dev, m->head_rows, m->xc));
+        xf = m->xc;
+    }
+    if (m->head_rows == 0) return FT_OK;
+    FT_TRY(ft_rms_norm_eps(ctx, xf, m->norm_f, m->hf, m->head_rows, H, c.rms_norm_eps));
+    FT_TRY(linear_forward(ctx, m->lm_head, m->hf, m->thead, m->logits, m->head_rows));
     return FT_OK;
 }
 
@@ -489,11 +520,18 @@ int model_backward(ft_model* m, size_t B, size_t S, bool accumulate) {
     const size_t D = m->head_dim(), nh = c.num_attention_heads, nkv = c.num_key_value_heads;
     ft_attention_options opts{};
     opts.causal = 1;
-    // lm_head and final norm
-    FT_TRY(linear_backward(m, m->lm_head, m->hf, m->thead, m->logits, m->d_h2, T, accumulate));
+    // lm_head and final norm, on the rows the head ran on
     float* g = m->g0;
     float* g_other = m->g1;
-    FT_TRY(ft_rms_norm_backward(ctx, m->x_final, m->norm_f, m->d_h2, g, nullptr, T, H, c.rms_norm_eps));
+    const size_t Th = m->head_rows;
+    FT_TRY(linear_backward(m, m->lm_head, m->hf, m->thead, m->logits, m->d_h2, Th, accumulate));
+    if (m->head_compact) {
+        FT_TRY(ft_rms_norm_backward(ctx, m->xc, m->norm_f, m->d_h2, g_other, nullptr, Th, H, c.rms_norm_eps));
+        // scatter: row r of g = row head_inv[r] of the compact gradient, zero where the head did not run
+        FT_TRY(ft_embedding(ctx, g_other, Th, H, m->head_inv_dev, T, g));
+    } else {
+        FT_TRY(ft_rms_norm_backward(ctx, m->x_final, m->norm_f, m->d_h2, g, nullptr, T, H, c.rms_norm_eps));
+    }
     for (size_t li = m->layers.size(); li-- > 0;) {
         Layer& L = m->layers[li];
         LayerActs& a = m->acts[li];
@@ -881,12 +919,15 @@ int ft_trainer_destroy(ft_trainer* t) {
 namespace {
 
 // Host half of masked_cross_entropy_batch (trainer/src/lib.rs:689-722): per-row target or
-// MASKED_CE_SKIP, weight 1 / supervised tokens of the row's sequence. Returns the total.
+// MASKED_CE_SKIP, weight 1 / supervised tokens of the row's sequence; kept for the supervised rows
+// only (`head`, ascending), in that order. Returns the total.
 size_t build_targets(const uint32_t* targets, const uint8_t* loss_mask, size_t B, size_t S, size_t V,
-                     std::vector<uint32_t>& tg, std::vector<float>& wt, std::vector<size_t>& tokens) {
+                     std::vector<uint32_t>& tg, std::vector<float>& wt, std::vector<size_t>& tokens,
+                     std::vector<uint32_t>& head) {
     const size_t T = B * S;
-    tg.assign(T, FT_MASKED_CE_SKIP);
-    wt.assign(T, 0.0f);
+    tg.clear();
+    wt.clear();
+    head.clear();
     tokens.assign(B, 0);
     auto supervised = [&](size_t r) { return loss_mask[r] != 0 && (size_t)targets[r] < V; };
     size_t total = 0;
@@ -896,23 +937,25 @@ size_t build_targets(const uint32_t* targets, const uint8_t* loss_mask, size_t B
     }
     for (size_t r = 0; r < T; r++) {
         if (supervised(r)) {
-            tg[r] = targets[r];
-            wt[r] = 1.0f / (float)tokens[r / S];
+            head.push_back((uint32_t)r);
+            tg.push_back(targets[r]);
+            wt.push_back(1.0f / (float)tokens[r / S]);
         }
     }
     return total;
 }
 
-// Per-sequence mean losses from the device row losses (f64 sums, as the reference's host code).
-int read_sequence_losses(ft_model* m, size_t B, size_t S, const std::vector<size_t>& tokens, float* per_sequence,
-                         float* total_out) {
-    std::vector<float> losses(B * S);
-    FT_TRY(ft_download(m->ctx, losses.data(), m->row_loss, B * S * sizeof(float)));
+// Per-sequence mean losses from the device row losses of the head rows (f64 sums in row order, as the
+// reference's host code; the rows left out are the ones that would add 0).
+int read_sequence_losses(ft_model* m, size_t B, size_t S, const std::vector<size_t>& tokens,
+                         const std::vector<uint32_t>& head, float* per_sequence, float* total_out) {
+    std::vector<float> losses(head.size());
+    FT_TRY(ft_download(m->ctx, losses.data(), m->row_loss, head.size() * sizeof(float)));
+    std::vector<double> sums(B, 0.0);
+    for (size_t k = 0; k < head.size(); k++) sums[head[k] / S] += (double)losses[k];
     float total = 0.0f;
     for (size_t s = 0; s < B; s++) {
-        double sum = 0.0;
-        for (size_t i = 0; i < S; i++) sum += (double)losses[s * S + i];
-        const float mean = (float)(sum / (double)(tokens[s] ? tokens[s] : 1));
+        const float mean = (float)(sums[s] / (double)(tokens[s] ? tokens[s] : 1));
         if (per_sequence) per_sequence[s] = mean;
         total += mean;
     }
@@ -930,23 +973,24 @@ int ft_model_eval_chunk(ft_model* m, const uint32_t* rows, const uint32_t* targe
         FT_CHECK_ARG(m && rows && targets && loss_mask && per_sequence_loss && per_sequence_tokens,
                      "ft_model_eval_chunk: NULL argument");
         FT_CHECK_ARG(B > 0 && S > 0, "ft_model_eval_chunk: empty chunk");
-        const size_t T = B * S, V = m->cfg.vocab_size;
+        const size_t V = m->cfg.vocab_size;
         std::vector<uint32_t> tg;
         std::vector<float> wt;
         std::vector<size_t> tokens;
-        const size_t total = build_targets(targets, loss_mask, B, S, V, tg, wt, tokens);
+        std::vector<uint32_t> head;
+        const size_t total = build_targets(targets, loss_mask, B, S, V, tg, wt, tokens, head);
         for (size_t s = 0; s < B; s++) {
             per_sequence_tokens[s] = (uint32_t)tokens[s];
             per_sequence_loss[s] = 0.0f;
         }
         if (total == 0) return FT_OK;
-        FT_TRY(model_forward(m, rows, B, S));
-        FT_TRY(ft_upload(m->ctx, m->targets_dev, tg.data(), T * sizeof(uint32_t)));
-        FT_TRY(ft_upload(m->ctx, m->weights_dev, wt.data(), T * sizeof(float)));
+        FT_TRY(model_forward(m, rows, B, S, &head));
+        FT_TRY(ft_upload(m->ctx, m->targets_dev, tg.data(), total * sizeof(uint32_t)));
+        FT_TRY(ft_upload(m->ctx, m->weights_dev, wt.data(), total * sizeof(float)));
         // forward only: the gradient the kernel writes (in place of the logits) is discarded
         FT_TRY(ft_masked_cross_entropy_weighted(m->ctx, m->logits, m->targets_dev, m->weights_dev, m->logits,
-                                                m->row_loss, T, V, 1.0f));
-        return read_sequence_losses(m, B, S, tokens, per_sequence_loss, nullptr);
+                                                m->row_loss, total, V, 1.0f));
+        return read_sequence_losses(m, B, S, tokens, head, per_sequence_loss, nullptr);
     });
 }
 
@@ -1024,7 +1068,8 @@ int ft_trainer_train_chunk(ft_trainer* t, const uint32_t* rows, const uint32_t* 
         std::vector<uint32_t> tg;
         std::vector<float> wt;
         std::vector<size_t> tokens;
-        const size_t total_tokens = build_targets(targets, loss_mask, B, S, V, tg, wt, tokens);
+        std::vector<uint32_t> head;
+        const size_t total_tokens = build_targets(targets, loss_mask, B, S, V, tg, wt, tokens, head);
         stats->supervised_tokens = (uint32_t)total_tokens;
         if (total_tokens == 0) {
             // masked_cross_entropy_batch returns None: no forward result is used, no backward.
@@ -1032,15 +1077,15 @@ int ft_trainer_train_chunk(ft_trainer* t, const uint32_t* rows, const uint32_t* 
             if (per_sequence_loss)
                 for (size_t s = 0; s < B; s++) per_sequence_loss[s] = 0.0f;
         } else {
-            FT_TRY(model_forward(m, rows, B, S));
-            FT_TRY(ft_upload(ctx, m->targets_dev, tg.data(), T * sizeof(uint32_t)));
-            FT_TRY(ft_upload(ctx, m->weights_dev, wt.data(), T * sizeof(float)));
+            FT_TRY(model_forward(m, rows, B, S, &head));
+            FT_TRY(ft_upload(ctx, m->targets_dev, tg.data(), total_tokens * sizeof(uint32_t)));
+            FT_TRY(ft_upload(ctx, m->weights_dev, wt.data(), total_tokens * sizeof(float)));
             // Loss + d loss / d logits in place, with the backward seed
             // 1 / grad_accum_steps folded in (trainer/src/lib.rs:474-480, 553-572).
             const float seed = 1.0f / (float)accum;
             const float gscale = std::fabs(seed - 1.0f) > kF32Epsilon ? seed : 1.0f;
             FT_TRY(ft_masked_cross_entropy_weighted(ctx, m->logits, m->targets_dev, m->weights_dev, m->logits,
-                                                    m->row_loss, T, V, gscale));
+                                                    m->row_loss, total_tokens, V, gscale));
             FT_TRY(model_backward(m, B, S, t->step_in_accum > 0));
             t->step_in_accum += B;
         }
@@ -1064,7 +1109,7 @@ int ft_trainer_train_chunk(ft_trainer* t, const uint32_t* rows, const uint32_t* 
         }
 
         // The step's only wait: row losses and the control block.
-        if (total_tokens > 0) FT_TRY(read_sequence_losses(m, B, S, tokens, per_sequence_loss, &stats->loss));
+        if (total_tokens > 0) FT_TRY(read_sequence_losses(m, B, S, tokens, head, per_sequence_loss, &stats->loss));
         if (window_full) {
             float control[3];
             FT_TRY(ft_download(ctx, control, t->control, sizeof(control)));

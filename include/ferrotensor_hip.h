@@ -458,7 +458,10 @@ int ft_trainer_set_optimizer_steps(ft_trainer* t, size_t steps);
  * with seed 1/grad_accum_steps, gradient norm, clip, AdamW. rows/targets are
  * [B,S] u32 and loss_mask [B,S] u8 in host memory; per_sequence_loss (B
  * values) may be NULL. `apply` = 0 stops after backward (gradients readable,
- * no optimizer step). */
+ * no optimizer step). The final norm, the vocabulary head and the loss run on
+ * the supervised positions only (a position without a target has zero loss and
+ * a zero logits gradient, kernels.wgsl:684-711, so every result keeps its bits);
+ * ft_model_forward_logits still returns the logits of every position. */
 int ft_trainer_train_chunk(ft_trainer* t, const uint32_t* rows, const uint32_t* targets,
                            const uint8_t* loss_mask, size_t B, size_t S, int apply,
                            ft_step_stats* stats, float* per_sequence_loss);
