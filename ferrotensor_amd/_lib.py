@@ -40,7 +40,8 @@ class ModelConfigC(C.Structure):
     _fields_ = [("vocab_size", C.c_uint32), ("hidden_size", C.c_uint32), ("intermediate_size", C.c_uint32),
                 ("num_hidden_layers", C.c_uint32), ("num_attention_heads", C.c_uint32),
                 ("num_key_value_heads", C.c_uint32), ("rms_norm_eps", C.c_float), ("rope_theta", C.c_float),
-                ("tie_word_embeddings", C.c_int32), ("f16_linears", C.c_int32), ("checkpoint_blocks", C.c_int32)]
+                ("tie_word_embeddings", C.c_int32), ("f16_linears", C.c_int32), ("checkpoint_blocks", C.c_int32),
+                ("head_all_rows", C.c_int32)]
 
 
 class TrainerConfigC(C.Structure):

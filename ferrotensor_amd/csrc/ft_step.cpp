@@ -492,7 +492,7 @@ int model_forward(ft_model* m, const uint32_t* rows_host, size_t B, size_t S,
     for (size_t l = 0; l < m->layers.size(); l++) FT_TRY(layer_forward(m, l, B, S));
     const float* xf = m->x_final;
     m->head_rows = T;
-    m->head_compact = head != nullptr && head->size() < T;
+    m->head_compact = head != nullptr && head->size() < T && !c.head_all_rows;
     if (m->head_compact) {
         m->head_rows = head->size();
         std::vector<uint32_t> inv(T, (uint32_t)head->size());
@@ -945,14 +945,37 @@ size_t build_targets(const uint32_t* targets, const uint8_t* loss_mask, size_t B
     return total;
 }
 
+// Targets and weights of the rows the head ran on in the last forward (the supervised rows, or all
+// T rows with MASKED_CE_SKIP / 0 in between) to the device; returns how many rows that is.
+int upload_targets(ft_model* m, size_t T, const std::vector<uint32_t>& tg, const std::vector<float>& wt,
+                   const std::vector<uint32_t>& head, size_t* rows_out) {
+    if (m->head_compact) {
+        FT_TRY(ft_upload(m->ctx, m->targets_dev, tg.data(), tg.size() * sizeof(uint32_t)));
+        FT_TRY(ft_upload(m->ctx, m->weights_dev, wt.data(), wt.size() * sizeof(float)));
+        *rows_out = tg.size();
+        return FT_OK;
+    }
+    std::vector<uint32_t> tg_all(T, FT_MASKED_CE_SKIP);
+    std::vector<float> wt_all(T, 0.0f);
+    for (size_t k = 0; k < head.size(); k++) {
+        tg_all[head[k]] = tg[k];
+        wt_all[head[k]] = wt[k];
+    }
+    FT_TRY(ft_upload(m->ctx, m->targets_dev, tg_all.data(), T * sizeof(uint32_t)));
+    FT_TRY(ft_upload(m->ctx, m->weights_dev, wt_all.data(), T * sizeof(float)));
+    *rows_out = T;
+    return FT_OK;
+}
+
 // Per-sequence mean losses from the device row losses of the head rows (f64 sums in row order, as the
 // reference's host code; the rows left out are the ones that would add 0).
 int read_sequence_losses(ft_model* m, size_t B, size_t S, const std::vector<size_t>& tokens,
                          const std::vector<uint32_t>& head, float* per_sequence, float* total_out) {
-    std::vector<float> losses(head.size());
-    FT_TRY(ft_download(m->ctx, losses.data(), m->row_loss, head.size() * sizeof(float)));
+    const size_t rows = m->head_compact ? head.size() : B * S;
+    std::vector<float> losses(rows);
+    FT_TRY(ft_download(m->ctx, losses.data(), m->row_loss, rows * sizeof(float)));
     std::vector<double> sums(B, 0.0);
-    for (size_t k = 0; k < head.size(); k++) sums[head[k] / S] += (double)losses[k];
+    for (size_t k = 0; k < head.size(); k++) sums[head[k] / S] += (double)losses[m->head_compact ? k : head[k]];
     float total = 0.0f;
     for (size_t s = 0; s < B; s++) {
         const float mean = (float)(sums[s] / (double)(tokens[s] ? tokens[s] : 1));
@@ -985,11 +1008,11 @@ int ft_model_eval_chunk(ft_model* m, const uint32_t* rows, const uint32_t* targe
         }
         if (total == 0) return FT_OK;
         FT_TRY(model_forward(m, rows, B, S, &head));
-        FT_TRY(ft_upload(m->ctx, m->targets_dev, tg.data(), total * sizeof(uint32_t)));
-        FT_TRY(ft_upload(m->ctx, m->weights_dev, wt.data(), total * sizeof(float)));
+        size_t ce_rows = 0;
+        FT_TRY(upload_targets(m, B * S, tg, wt, head, &ce_rows));
         // forward only: the gradient the kernel writes (in place of the logits) is discarded
         FT_TRY(ft_masked_cross_entropy_weighted(m->ctx, m->logits, m->targets_dev, m->weights_dev, m->logits,
-                                                m->row_loss, total, V, 1.0f));
+                                                m->row_loss, ce_rows, V, 1.0f));
         return read_sequence_losses(m, B, S, tokens, head, per_sequence_loss, nullptr);
     });
 }
@@ -1078,14 +1101,14 @@ int ft_trainer_train_chunk(ft_trainer* t, const uint32_t* rows, const uint32_t* 
                 for (size_t s = 0; s < B; s++) per_sequence_loss[s] = 0.0f;
         } else {
             FT_TRY(model_forward(m, rows, B, S, &head));
-            FT_TRY(ft_upload(ctx, m->targets_dev, tg.data(), total_tokens * sizeof(uint32_t)));
-            FT_TRY(ft_upload(ctx, m->weights_dev, wt.data(), total_tokens * sizeof(float)));
+            size_t ce_rows = 0;
+            FT_TRY(upload_targets(m, T, tg, wt, head, &ce_rows));
             // Loss + d loss / d logits in place, with the backward seed
             // 1 / grad_accum_steps folded in (trainer/src/lib.rs:474-480, 553-572).
             const float seed = 1.0f / (float)accum;
             const float gscale = std::fabs(seed - 1.0f) > kF32Epsilon ? seed : 1.0f;
             FT_TRY(ft_masked_cross_entropy_weighted(ctx, m->logits, m->targets_dev, m->weights_dev, m->logits,
-                                                    m->row_loss, total_tokens, V, gscale));
+                                                    m->row_loss, ce_rows, V, gscale));
             FT_TRY(model_backward(m, B, S, t->step_in_accum > 0));
             t->step_in_accum += B;
         }

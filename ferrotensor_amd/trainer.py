@@ -32,12 +32,13 @@ class ModelConfig:
     tie_word_embeddings: bool = False
     f16_linears: bool = False
     checkpoint_blocks: bool = False
+    head_all_rows: bool = False
 
     def c(self):
         return _lib.ModelConfigC(self.vocab_size, self.hidden_size, self.intermediate_size, self.num_hidden_layers,
                                  self.num_attention_heads, self.num_key_value_heads, self.rms_norm_eps,
                                  self.rope_theta, 1 if self.tie_word_embeddings else 0, 1 if self.f16_linears else 0,
-                                 1 if self.checkpoint_blocks else 0)
+                                 1 if self.checkpoint_blocks else 0, 1 if self.head_all_rows else 0)
 
 
 @dataclass

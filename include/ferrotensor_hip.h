@@ -355,6 +355,12 @@ typedef struct ft_model_config {
     /* Lfm2Model::with_block_checkpointing (lfm.rs:338-355): keep only each block's input
      * during training and recompute the block in backward (one extra forward per block). */
     int32_t checkpoint_blocks;
+    /* 0 (default): training and evaluation run the final norm, the vocabulary head and the loss
+     * on the supervised positions only. 1: on every position, as the reference does. A row's
+     * results do not depend on which other rows share a launch, so both give the same bits,
+     * unless the row count moves the head's input-gradient GEMM across the tile count at which
+     * it splits K (a different summation order: rounding-level differences). */
+    int32_t head_all_rows;
 } ft_model_config;
 
 typedef struct ft_model ft_model;
@@ -460,7 +466,7 @@ int ft_trainer_set_optimizer_steps(ft_trainer* t, size_t steps);
  * values) may be NULL. `apply` = 0 stops after backward (gradients readable,
  * no optimizer step). The final norm, the vocabulary head and the loss run on
  * the supervised positions only (a position without a target has zero loss and
- * a zero logits gradient, kernels.wgsl:684-711, so every result keeps its bits);
+ * a zero logits gradient, kernels.wgsl:684-711; see ft_model_config.head_all_rows);
  * ft_model_forward_logits still returns the logits of every position. */
 int ft_trainer_train_chunk(ft_trainer* t, const uint32_t* rows, const uint32_t* targets,
                            const uint8_t* loss_mask, size_t B, size_t S, int apply,

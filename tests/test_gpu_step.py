@@ -435,6 +435,40 @@ def test_the_step_is_deterministic_to_the_bit(ctx):
             assert np.array_equal(np.asarray(x[k]).view(np.uint32), np.asarray(y[k]).view(np.uint32)), k
 
 
+def test_head_on_supervised_rows_changes_no_bit(ctx):
+    """The step runs the final norm, the vocabulary head and the loss on the supervised positions only; with
+    `head_all_rows` it runs them on every position as the reference does. Losses, gradients, weights after
+    two steps and the evaluation loss agree to the bit, with ragged masks and a sequence without any target."""
+    from ferrotensor_amd.trainer import Lfm2Model, ModelConfig, Trainer
+    rng = np.random.default_rng(8)
+    B, S = 4, 64
+    rows = rng.integers(0, 256, (B, S)).astype(np.uint32)
+    targets = np.concatenate([rows[:, 1:], rows[:, :1]], axis=1)
+    masks = (rng.random((B, S)) > 0.4).astype(np.uint8)
+    masks[1, :] = 0                      # a sequence with nothing to learn from
+    masks[2, :40] = 0                    # a long prompt
+    targets[3, 5] = 100000               # out of vocabulary: not supervised either
+    mods = ["q_proj", "k_proj", "v_proj", "o_proj"]
+    out = []
+    for all_rows in (False, True):
+        cfg = ModelConfig(vocab_size=256, hidden_size=192, intermediate_size=256, num_hidden_layers=2,
+                          num_attention_heads=3, num_key_value_heads=1, rms_norm_eps=1e-5, rope_theta=100000.0,
+                          tie_word_embeddings=True, f16_linears=True, head_all_rows=all_rows)
+        hip, _ = build_pair(ctx, cfg, mods, rank=8, alpha=16.0, seed=52)
+        tr = Trainer(hip, lr=1e-3, weight_decay=0.0, clip_grad_norm=1.0, grad_accum_steps=B)
+        stats = [tr.train_chunk(rows, targets, masks) for _ in range(2)]
+        seqs = [(list(r), list(t_), list(m)) for r, t_, m in zip(rows, targets, masks)]
+        out.append(([(s.loss, s.grad_norm, s.tokens) for s in stats], hip.evaluate(seqs), hip.grads(),
+                    hip.params()))
+        tr.close()
+        hip.close()
+    a, b = out
+    assert a[0] == b[0] and a[1] == b[1]
+    for x, y in zip(a[2:], b[2:]):
+        for k in x:
+            assert np.array_equal(x[k].view(np.uint32), y[k].view(np.uint32)), k
+
+
 def test_evaluate_is_the_token_weighted_forward_loss(ctx):
     """`evaluate` (ferrotensor-cli/src/main.rs:1110-1137): sum(loss_i * n_i) / sum(n_i) over ragged
     examples, forward only: parameters and gradients are untouched."""
