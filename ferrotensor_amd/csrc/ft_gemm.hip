@@ -1467,7 +1467,7 @@ int ft_lora_down(ft_context* ctx, const float* x, const float* a, float* t, size
                  float scale) {
     FT_CHECK_ARG(ctx && x && a && t, "ft_lora_down: NULL argument");
     FT_CHECK_ARG(r >= 1 && r <= 32, "ft_lora_down: rank %zu is outside 1..32", r);
-    ft_thin_problem tp{x, a, t, (int)M, (int)K, 0, (int)r, (long)K, (long)r, (long)r, scale, 0, 0, 0};
+    ft_thin_problem tp{x, a, t, (int)M, (int)K, 0, (int)r, (long)K, (long)r, (long)r, scale, 0, 0, 0, 0};
     if (ft_thin_rowwise_ok(tp)) return ft_thin_rowwise(ctx, &tp, 1);
     return skinny_launch<false, false, false>(ctx, x, a, t, M, K, r, (long)K, (long)r, (long)r, scale);
 }
@@ -1483,7 +1483,7 @@ int ft_lora_grad_down(ft_context* ctx, const float* dy, const float* b, float* d
     FT_CHECK_ARG(ctx && dy && b && dt, "ft_lora_grad_down: NULL argument");
     FT_CHECK_ARG(r >= 1 && r <= 32, "ft_lora_grad_down: rank %zu is outside 1..32", r);
     // dt[m][j] = sum_n dy[m][n] * b[j][n]
-    ft_thin_problem tp{dy, b, dt, (int)M, (int)N, 0, (int)r, (long)N, (long)N, (long)r, scale, 1, 0, 0};
+    ft_thin_problem tp{dy, b, dt, (int)M, (int)N, 0, (int)r, (long)N, (long)N, (long)r, scale, 1, 0, 0, 0};
     if (ft_thin_rowwise_ok(tp)) return ft_thin_rowwise(ctx, &tp, 1);
     return skinny_launch<false, true, false>(ctx, dy, b, dt, M, N, r, (long)N, (long)N, (long)r, scale);
 }
@@ -1639,7 +1639,7 @@ int ft_lora_grad_b(ft_context* ctx, const float* t, const float* dy, float* db, 
     FT_CHECK_ARG(ctx && t && dy && db, "ft_lora_grad_b: NULL argument");
     FT_CHECK_ARG(r >= 1 && r <= 32, "ft_lora_grad_b: rank %zu is outside 1..32", r);
     // db^T[n][j] = sum_m dy[m][n] * t[m][j]: rows = n (dy read transposed), output stored transposed.
-    ft_thin_problem tp{dy, t, db, (int)M, 0, (int)N, (int)r, (long)N, (long)r, (long)N, 1.0f, 0, 1, 0};
+    ft_thin_problem tp{dy, t, db, (int)M, 0, (int)N, (int)r, (long)N, (long)r, (long)N, 1.0f, 0, 1, 0, 0};
     if (ft_thin_colwise_ok(tp)) return ft_thin_colwise(ctx, &tp, 1);
     return skinny_launch<true, false, true>(ctx, dy, t, db, N, M, r, (long)N, (long)r, (long)N, 1.0f);
 }
@@ -1648,7 +1648,7 @@ int ft_lora_grad_a(ft_context* ctx, const float* x, const float* dt, float* da, 
     FT_CHECK_ARG(ctx && x && dt && da, "ft_lora_grad_a: NULL argument");
     FT_CHECK_ARG(r >= 1 && r <= 32, "ft_lora_grad_a: rank %zu is outside 1..32", r);
     // da[k][j] = sum_m x[m][k] * dt[m][j]: rows = k (x read transposed).
-    ft_thin_problem tp{x, dt, da, (int)M, 0, (int)K, (int)r, (long)K, (long)r, (long)r, 1.0f, 0, 0, 0};
+    ft_thin_problem tp{x, dt, da, (int)M, 0, (int)K, (int)r, (long)K, (long)r, (long)r, 1.0f, 0, 0, 0, 0};
     if (ft_thin_colwise_ok(tp)) return ft_thin_colwise(ctx, &tp, 1);
     return skinny_launch<true, false, false>(ctx, x, dt, da, K, M, r, (long)K, (long)r, (long)r, 1.0f);
 }

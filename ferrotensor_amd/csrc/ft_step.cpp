@@ -267,7 +267,7 @@ int lora_down_group(ft_context* ctx, LinearW* const* ls, float* const* ts, int n
         if (!ls[i]->has_lora()) continue;
         const LinearW& l = *ls[i];
         probs[cnt] = ft_thin_problem{x, l.a, ts[i], (int)T, (int)l.in, 0, (int)l.r, (long)l.in, (long)l.r, (long)l.r,
-                                     l.scale(), 0, 0, 0};
+                                     l.scale(), 0, 0, 0, 0};
         batch = batch && ft_thin_rowwise_ok(probs[cnt]) && l.r == ls[0]->r;
         cnt++;
     }
@@ -370,7 +370,7 @@ int linear_backward_group(ft_model* m, LinearW* const* ls, const float* const* t
             break;
         }
         rows[i] = ft_thin_problem{dys[i], l.b, dts[i], (int)T, (int)l.out, 0, (int)l.r, (long)l.out, (long)l.out,
-                                  (long)l.r, l.scale(), 1, 0, 0};
+                                  (long)l.r, l.scale(), 1, 0, 0, 0};
         cols[2 * i] = ft_thin_problem{dys[i], ts[i], l.gb, (int)T, 0, (int)l.out, (int)l.r, (long)l.out, (long)l.r,
                                       (long)l.out, 1.0f, 0, 1, 0, acc};
         cols[2 * i + 1] = ft_thin_problem{x, dts[i], l.ga, (int)T, 0, (int)l.in, (int)l.r, (long)l.in, (long)l.r,
@@ -483,12 +483,9 @@ int model_forward(ft_model* m, const uint32_t* rows_host, size_t B, size_t S,
         ws_free(m);
     }
     FT_TRY(ensure_workspace(m, B, S));
-    const size_t T = B * S, H = c.hidden_size, F = c.intermediate_size;
-    const size_t D = m->head_dim(), nh = c.num_attention_heads, nkv = c.num_key_value_heads;
+    const size_t T = B * S, H = c.hidden_size;
     FT_TRY(ft_upload(ctx, m->ids_dev, rows_host, T * sizeof(uint32_t)));
     FT_TRY(ft_embedding(ctx, m->embed, c.vocab_size, H, m->ids_dev, T, m->acts.empty() ? m->x_final : m->acts[0].x));
-    ft_attention_options opts{};
-    opts.causal = 1;
     for (size_t l = 0; l < m->layers.size(); l++) FT_TRY(layer_forward(m, l, B, S));
     const float* xf = m->x_final;
     m->head_rows = T;

@@ -97,7 +97,7 @@ __global__ __launch_bounds__(kRowWaves * 64) void thin_rowwise_kernel(ThinBatch 
 template <int C>
 __global__ __launch_bounds__(256) void thin_colwise_kernel(ThinBatch b, float* __restrict__ scratch, int slices) {
     const ft_thin_problem& p = b.p[blockIdx.y];
-    if (blockIdx.x * 256 >= p.R) return;  // whole workgroup past this problem's width
+    if ((int)blockIdx.x * 256 >= p.R) return;  // whole workgroup past this problem's width
     __shared__ float red[3][4 * C][kWave + 1];
     const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
     const int n = (blockIdx.x * 64 + lane) * 4;
