@@ -957,6 +957,142 @@ __global__ __launch_bounds__(256) void gemm_async_kernel(AsyncBatch g) {
 }
 
 // ---------------------------------------------------------------------------
+// f32 x f32 on the same pipeline (global -> LDS DMA, three stages, explicit
+// waits): the plain matmul / matmul_bt / matmul_at of the engine, where b is an
+// f32 tensor. An operand tile is either
+//   KC  k-contiguous in memory (a[M,K]; b[N,K]): [64 rows][32 k], 128 B per row,
+//       swizzled as in gemm_async_kernel, one ds_read_b128 per k-quad, or
+//   KM  k-major (a[K,M] of matmul_at; b[K,N]): [32 k][64] exactly as in memory
+//       (4 k rows per DMA instruction), four ds_read_b32 per k-quad.
+// 64x64 tiles, 32x32 per wave; K a multiple of 32, M / N multiples of 4 where an
+// operand is KM. Tile order as in gemm_async_kernel.
+// ---------------------------------------------------------------------------
+struct F32AsyncArgs {
+    const float* a;
+    const float* b;
+    float* out;
+    int M, N, nt;        // nt = K / 32
+    int lda, ldb, ldc;
+    int tiles_m, tiles_n, xcds, panel;
+    int splits;          // shares of the K tiles (blockIdx.y); > 1: partial tiles go to `partial` [splits][M][N]
+    float* partial;
+};
+
+template <bool A_KM, bool B_KM>
+__global__ __launch_bounds__(256) void gemm_f32_async_kernel(F32AsyncArgs g) {
+    constexpr int NST = 3, TILE = 64 * 32, STAGE = 2 * TILE;
+    constexpr int LPT = 4;                         // 2 + 2 load instructions per wave per K tile
+    __shared__ __attribute__((aligned(16))) float St0[STAGE];
+    __shared__ __attribute__((aligned(16))) float St1[STAGE];
+    __shared__ __attribute__((aligned(16))) float St2[STAGE];
+    int bid = (int)blockIdx.x;
+    if (g.xcds > 1) {
+        const int total = (int)gridDim.x, x = bid % g.xcds, q = total / g.xcds, r = total % g.xcds;
+        bid = x * q + (x < r ? x : r) + bid / g.xcds;
+    }
+    const int per_panel = g.tiles_m * g.panel;
+    const int last = (g.tiles_n - 1) / g.panel;
+    int pnl = bid / per_panel;
+    pnl = pnl < last ? pnl : last;
+    const int rem = bid - pnl * per_panel;
+    const int width = pnl == last ? g.tiles_n - last * g.panel : g.panel;
+    const int m0 = (rem / width) * 64, n0 = (pnl * g.panel + rem % width) * 64;
+    const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
+    const int wm0 = (wave / 2) * 32, wn0 = (wave % 2) * 32;
+    const int l32 = lane % 32, half = lane / 32;
+
+    // Per-lane byte offsets of the two DMA instructions a wave issues per operand and K tile.
+    unsigned offA[2], offB[2];
+    auto offsets = [&](bool km, int base0, int extent, int ld, unsigned (&off)[2]) {
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            const int c = wave + 4 * j;  // chunk of 1 KiB
+            if (km) {
+                const int kr = lane / 16, cs = lane % 16;
+                int col = base0 + cs * 4;
+                col = col + 4 <= extent ? col : extent - 4;
+                off[j] = (unsigned)(4 * c + kr) * (unsigned)ld * 4u + (unsigned)col * 4u;
+            } else {
+                const int r = lane / 8, cs = lane % 8;
+                int row = base0 + 8 * c + r;
+                row = row < extent ? row : extent - 1;
+                off[j] = (unsigned)row * (unsigned)ld * 4u + (unsigned)((cs ^ ((4 * c + (r >> 1)) & 7)) * 16);
+            }
+        }
+    };
+    offsets(A_KM, m0, g.M, g.lda, offA);
+    offsets(B_KM, n0, g.N, g.ldb, offB);
+    const long a_step = A_KM ? 32L * g.lda * 4 : 128L, b_step = B_KM ? 32L * g.ldb * 4 : 128L;
+    const char* abase = reinterpret_cast<const char*>(g.a);
+    const char* bbase = reinterpret_cast<const char*>(g.b);
+    // This workgroup's share of the K tiles: [t0, nt).
+    const int split = (int)blockIdx.y;
+    const int t0 = (int)(((long)g.nt * split) / g.splits);
+    const int nt = (int)(((long)g.nt * (split + 1)) / g.splits);
+    auto issue = [&](int t, float* st) {
+        t = t < nt ? t : nt - 1;  // past the end: re-read the last tile into a stage nobody reads
+        const char* at = abase + (long)t * a_step;
+        const char* bt = bbase + (long)t * b_step;
+#pragma unroll
+        for (int j = 0; j < 2; j++) glds16(at, offA[j], st + (wave + 4 * j) * 256);
+#pragma unroll
+        for (int j = 0; j < 2; j++) glds16(bt, offB[j], st + TILE + (wave + 4 * j) * 256);
+    };
+    auto frag = [&](const float* tile, bool km, int s, int idx) -> float4 {
+        const int kq = 2 * s + half;
+        if (km) {
+            const float* q = tile + (4 * kq) * 64 + idx;
+            return make_float4(q[0], q[64], q[128], q[192]);
+        }
+        return *reinterpret_cast<const float4*>(tile + idx * 32 + ((kq ^ ((idx >> 1) & 7)) * 4));
+    };
+    floatx16 acc;
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc[r] = 0.0f;
+    auto iter = [&](int t, const float* cur, float* refill) {
+        __builtin_amdgcn_s_waitcnt(0x0F70 | LPT);
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+        issue(t + NST - 1, refill);
+        __builtin_amdgcn_sched_barrier(0);
+        float4 af[2], bf[2];
+        af[0] = frag(cur, A_KM, 0, wm0 + l32);
+        bf[0] = frag(cur + TILE, B_KM, 0, wn0 + l32);
+#pragma unroll
+        for (int s = 0; s < 4; s++) {
+            const int c = s & 1, nx = c ^ 1;
+            if (s + 1 < 4) {
+                af[nx] = frag(cur, A_KM, s + 1, wm0 + l32);
+                bf[nx] = frag(cur + TILE, B_KM, s + 1, wn0 + l32);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(af[c].x, bf[c].x, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(af[c].y, bf[c].y, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(af[c].z, bf[c].z, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(af[c].w, bf[c].w, acc, 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    issue(t0, St0);
+    issue(t0 + 1, St1);
+    for (int t = t0; t < nt; t += NST) {
+        iter(t, St0, St2);
+        if (t + 1 < nt) iter(t + 1, St1, St0);
+        if (t + 2 < nt) iter(t + 2, St2, St1);
+    }
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // nothing may still be landing in LDS when the workgroup retires
+    const int col = n0 + wn0 + l32;
+    if (col >= g.N) return;
+    float* dst = g.splits > 1 ? g.partial + (long)split * g.M * g.N : g.out;
+    const int ld = g.splits > 1 ? g.N : g.ldc;
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+        const int row = m0 + wm0 + (r / 4) * 8 + half * 4 + (r % 4);
+        if (row < g.M) dst[(long)row * ld + col] = acc[r];
+    }
+}
+
+// ---------------------------------------------------------------------------
 // out[R, C] (C <= 32) = scale * X[R, Kr] @ Y[Kr, C].
 //   XT:  X is stored [Kr, R] (element (row,k) at x[k*ldx + row])
 //   YT:  Y is stored [C, Kr] (element (k,col) at y[col*ldy + k])
@@ -1329,6 +1465,82 @@ int launch_cfg(ft_context* ctx, GemmArgs p, int layout, bool half_b, bool fast) 
     return FT_OK;
 }
 
+// Operands of the f32 DMA kernel: 16-byte aligned, K in whole tiles, at least two of them per
+// workgroup, k-major operands in whole float4 groups, 32-bit per-lane offsets.
+bool f32_async_eligible(int layout, const float* a, const void* b, const float* out, size_t M, size_t K, size_t N) {
+    if (M == 0 || N == 0 || K < 64 || K % 32 != 0) return false;
+    if (!aligned16p(a) || !aligned16p(b) || !out) return false;
+    const bool a_km = layout == 2, b_km = layout != 1;
+    if (a_km && (M % 4 != 0 || M < 4)) return false;
+    if (b_km && (N % 4 != 0 || N < 4)) return false;
+    if (M * N < 128 * 128) return false;  // tiny products: the register-staged kernels
+    const double lim = 4294967296.0;
+    const double a_span = a_km ? 4.0 * 36 * (double)M : 4.0 * ((double)M + 64) * (double)K;
+    const double b_span = b_km ? 4.0 * 36 * (double)N : 4.0 * ((double)N + 64) * (double)K;
+    return a_span < lim && b_span < lim;
+}
+
+int launch_f32_async(ft_context* ctx, int layout, const float* a, const float* b, float* out, size_t M, size_t K,
+                     size_t N) {
+    F32AsyncArgs g{};
+    g.a = a;
+    g.b = b;
+    g.out = out;
+    g.M = (int)M;
+    g.N = (int)N;
+    g.nt = (int)(K / 32);
+    g.lda = layout == 2 ? (int)M : (int)K;
+    g.ldb = layout == 1 ? (int)K : (int)N;
+    g.ldc = (int)N;
+    g.tiles_m = (int)((M + 63) / 64);
+    g.tiles_n = (int)((N + 63) / 64);
+    g.xcds = ft_gemm_xcds(ctx);
+    // panels of about sqrt(96) n tiles: equal bytes of a and b per XCD-resident block of tiles
+    int panels = (int)((double)g.tiles_n / 10.0 + 0.5);
+    if (panels < 1) panels = 1;
+    g.panel = (g.tiles_n + panels - 1) / panels;
+    // Split K when the tiles occupy at most half of the CUs and K is long enough to share out
+    // (at least 4 K tiles per share); the shares are added in order. (At 216 tiles of K = 2048
+    // a three-way split measured no gain: 44.4 us against 42.6.)
+    const size_t tiles = (size_t)g.tiles_m * g.tiles_n;
+    g.splits = 1;
+    if (tiles * 2 <= (size_t)ctx->num_cus && (M * N) % 4 == 0) {
+        int want = (int)((2 * (size_t)ctx->num_cus + tiles - 1) / tiles);
+        if (want > 8) want = 8;
+        if (want > g.nt / 4) want = g.nt / 4;
+        if (want >= 2 && M * N * (size_t)want <= kSplitScratchFloats) {
+            if (!ctx->gemm_scratch) {
+                FT_HIP(hipSetDevice(ctx->device));
+                FT_HIP(hipMalloc((void**)&ctx->gemm_scratch, kSplitScratchFloats * sizeof(float)));
+            }
+            g.splits = want;
+            g.partial = ctx->gemm_scratch;
+        }
+    }
+    const dim3 grid((unsigned)tiles, (unsigned)g.splits);
+    char name[64];
+    snprintf(name, sizeof(name), "gemm_f32_async_kernel<%d>", layout);
+    ft_prof_scope prof(ctx, name, 2.0 * M * (double)N * K, 4.0 * ((double)M * K + (double)N * K + (double)M * N));
+    if (layout == 0)
+        hipLaunchKernelGGL((gemm_f32_async_kernel<false, true>), grid, dim3(256), 0, ctx->stream, g);
+    else if (layout == 1)
+        hipLaunchKernelGGL((gemm_f32_async_kernel<false, false>), grid, dim3(256), 0, ctx->stream, g);
+    else
+        hipLaunchKernelGGL((gemm_f32_async_kernel<true, true>), grid, dim3(256), 0, ctx->stream, g);
+    FT_LAUNCH_CHECK();
+    if (g.splits > 1) {
+        SplitReduceArgs ra{};
+        ra.partial[0] = g.partial;
+        ra.add[0] = nullptr;
+        ra.out[0] = out;
+        ra.n4[0] = (long)(M * N / 4);
+        ra.splits = g.splits;
+        hipLaunchKernelGGL(splitk_reduce_kernel, dim3(ft_div_up(M * N / 4, 256), 1), dim3(256), 0, ctx->stream, ra);
+        FT_LAUNCH_CHECK();
+    }
+    return FT_OK;
+}
+
 int gemm_dispatch(ft_context* ctx, const char* who, int layout, bool half_b, const float* a, const void* b,
                   float* out, size_t M, size_t K, size_t N, const float* a2, const float* b2, size_t K2,
                   const float* add = nullptr) {
@@ -1366,6 +1578,8 @@ int gemm_dispatch(ft_context* ctx, const char* who, int layout, bool half_b, con
         g.p[0].ldc = (int)N;
         return launch_async_auto(ctx, g, layout);
     }
+    if (!half_b && !p.a2 && !add && f32_async_eligible(layout, a, b, out, M, K, N))
+        return launch_f32_async(ctx, layout, a, static_cast<const float*>(b), out, M, K, N);
     // Tile choice for the register-staged kernels, from measurements on MI355X at
     // M = 2048: 128x128 tiles when there are many per CU, else 64x64; a deep K
     // loop on few tiles prefers BK = 64 (half the barriers per MFMA).

@@ -37,7 +37,9 @@ def empty(ctx, *shape):
 
 
 MATMUL_SHAPES = [(1, 1, 1), (1, 7, 1), (3, 5, 7), (16, 16, 16), (17, 33, 9), (64, 64, 64), (65, 1, 130),
-                 (127, 129, 65), (1, 512, 300), (300, 512, 1), (256, 384, 128), (130, 70, 200), (256, 96, 320)]
+                 (127, 129, 65), (1, 512, 300), (300, 512, 1), (256, 384, 128), (130, 70, 200), (256, 96, 320),
+                 # the DMA-fed f32 kernels: ragged last tiles, rows that are no multiple of 4, one and many K tiles
+                 (200, 128, 132), (132, 64, 260), (130, 64, 256), (260, 2048, 128), (129, 96, 131), (2048, 576, 1536), (256, 4096, 192)]
 
 # GEMM tolerance of the reference's f64 comparisons (gpu_kernels.rs:989-1084): 1e-3 + 1e-4*|want|
 # for N(0,1) operands; the oracle itself adds in f32, so compare against f64 here.
