@@ -10,7 +10,8 @@ base weights, f32 LoRA rank 8 alpha 16 on q/k/v/o, AdamW lr 2e-4. Weights and
 inputs are resident in HBM when the timed region starts, except the 2048 token
 ids / targets / weights the step uploads itself (24 KiB).
 
-Prints ONE JSON line: tokens/s (positions = B*S / step time), plus
+Prints ONE JSON line: tokens/s (positions = B*S / step time; the reference CLI's
+tok/s counts supervised tokens only: `supervised_tokens_per_s`), plus
   roofline     the dominant GEMM kernel: algorithmic 2*M*N*K flops per launch
                over its HIP-event duration (events on the library's stream,
                taken over K further steps identical to the timed ones), against
@@ -416,6 +417,7 @@ def main():
                    "base_weights": "f16 storage, f32 arithmetic", "optimizer": "AdamW lr 2e-4 wd 0 clip 1.0",
                    "supervised_tokens": int(st.tokens), "loss": float(st.loss),
                    "head": "final norm, vocabulary head and loss on the %d supervised positions" % int(st.tokens)},
+        "supervised_tokens_per_s": int(st.tokens) / (elapsed / args.steps),
         "step_tflops": step_flops(w, int(st.tokens)) / (elapsed / args.steps) / 1e12,
         "step_mfma_frac": step_flops(w, int(st.tokens)) / (elapsed / args.steps) / 1e12 / FP32_MFMA_PEAK_TFLOPS,
         "roofline": {"bound": "mfma", "kernel": dom["name"], "achieved": achieved, "peak": FP32_MFMA_PEAK_TFLOPS,
