@@ -123,6 +123,13 @@ struct ft_model {
     float *g0 = nullptr, *g1 = nullptr, *d_act = nullptr, *d_gate = nullptr, *d_up = nullptr, *d_h2 = nullptr,
           *d_attn = nullptr, *dq = nullptr, *dk = nullptr, *dv = nullptr, *d_h1 = nullptr, *dt = nullptr,
           *dt2 = nullptr, *dt3 = nullptr, *gtmp = nullptr, *rope_table = nullptr;
+    // Factor gradients (dA, dB) waiting for their launch on the side stream: the products of up to
+    // four linears go out together (one fork per block instead of one per linear). Each waiting
+    // linear keeps its own dT buffer from dt_pool until the main stream has joined the side stream.
+    static constexpr int kDtPool = 8;
+    float* dt_pool[kDtPool] = {};
+    int dt_used = 0;
+    std::vector<ft_thin_problem> pending_cols;
 
     size_t head_dim() const { return cfg.hidden_size / cfg.num_attention_heads; }
 };
@@ -233,9 +240,12 @@ int ensure_workspace(ft_model* m, size_t B, size_t S) {
         FT_TRY(ws_alloc(m, S * m->head_dim(), &m->rope_table));
         FT_TRY(ft_internal_rope_table(m->ctx, m->rope_table, S, m->head_dim(), 0, c.rope_theta));
     }
-    FT_TRY(ws_alloc(m, T * (rmax ? rmax : 1), &m->dt));
-    FT_TRY(ws_alloc(m, T * (rmax ? rmax : 1), &m->dt2));
-    FT_TRY(ws_alloc(m, T * (rmax ? rmax : 1), &m->dt3));
+    for (int i = 0; i < ft_model::kDtPool; i++) FT_TRY(ws_alloc(m, T * (rmax ? rmax : 1), &m->dt_pool[i]));
+    m->dt = m->dt_pool[0];
+    m->dt2 = m->dt_pool[1];
+    m->dt3 = m->dt_pool[2];
+    m->dt_used = 0;
+    m->pending_cols.clear();
     size_t gmax = 1;
     for (auto& p : m->params) gmax = p.n > gmax ? p.n : gmax;
     FT_TRY(ws_alloc(m, gmax, &m->gtmp));
@@ -312,37 +322,75 @@ int linear_forward(ft_context* ctx, LinearW& l, const float* x, float* t, float*
     return linear_gemm(ctx, l, x, t, y, T, residual);
 }
 
+// Launches the waiting factor-gradient products on the side stream, in batches of equal rank.
+int flush_cols(ft_model* m) {
+    if (m->pending_cols.empty()) return FT_OK;
+    ft_context* ctx = m->ctx;
+    FT_TRY(ft_side_begin(ctx));
+    int rc = FT_OK;
+    size_t i = 0;
+    while (i < m->pending_cols.size() && rc == FT_OK) {
+        size_t n = 1;
+        while (i + n < m->pending_cols.size() && n < (size_t)FT_THIN_MAX_BATCH &&
+               m->pending_cols[i + n].C == m->pending_cols[i].C)
+            n++;
+        rc = ft_thin_colwise(ctx, &m->pending_cols[i], (int)n);
+        i += n;
+    }
+    m->pending_cols.clear();
+    FT_TRY(ft_side_end(ctx));
+    return rc;
+}
+
+// The main stream waits for the side stream; afterwards every dT buffer is free again.
+int join_cols(ft_model* m) {
+    FT_TRY(ft_side_join(m->ctx, 0));
+    if (m->pending_cols.empty()) m->dt_used = 0;
+    return FT_OK;
+}
+
+// A dT buffer nobody on the side stream still reads.
+int take_dt(ft_model* m, float** dt) {
+    if (m->dt_used == ft_model::kDtPool) {
+        FT_TRY(flush_cols(m));
+        FT_TRY(join_cols(m));
+    }
+    *dt = m->dt_pool[m->dt_used++];
+    return FT_OK;
+}
+
 // Gradients of one linear given dy: LoRA factor gradients (written, or added
 // when `accumulate`), and dx when wanted (added to what dx holds when `dx_add`).
 int linear_backward(ft_model* m, LinearW& l, const float* x, const float* t, const float* dy, float* dx, size_t T,
                     bool accumulate, bool dx_add = false) {
     ft_context* ctx = m->ctx;
     if (l.has_lora()) {
-        FT_TRY(ft_side_join(ctx, 0));  // factor gradients still in flight read m->dt
-        FT_TRY(ft_lora_grad_down(ctx, dy, l.b, m->dt, T, l.out, l.r, l.scale()));
+        float* dt = nullptr;
+        FT_TRY(take_dt(m, &dt));
+        FT_TRY(ft_lora_grad_down(ctx, dy, l.b, dt, T, l.out, l.r, l.scale()));
         // dB = t^T dy and dA = x^T dt in one sliced launch when possible (added to the
         // gradients of the earlier micro-batches when `accumulate`).
         const int acc = accumulate ? 1 : 0;
         ft_thin_problem pb[2] = {
             {dy, t, l.gb, (int)T, 0, (int)l.out, (int)l.r, (long)l.out, (long)l.r, (long)l.out, 1.0f, 0, 1, 0, acc},
-            {x, m->dt, l.ga, (int)T, 0, (int)l.in, (int)l.r, (long)l.in, (long)l.r, (long)l.r, 1.0f, 0, 0, 0, acc}};
+            {x, dt, l.ga, (int)T, 0, (int)l.in, (int)l.r, (long)l.in, (long)l.r, (long)l.r, 1.0f, 0, 0, 0, acc}};
         if (ft_thin_colwise_ok(pb[0]) && ft_thin_colwise_ok(pb[1])) {
-            // Only the optimizer reads dA and dB: they run beside the input-gradient GEMM.
-            FT_TRY(ft_side_begin(ctx));
-            const int rc = ft_thin_colwise(ctx, pb, 2);
-            FT_TRY(ft_side_end(ctx));
-            FT_TRY(rc);
+            // Only the optimizer reads dA and dB: they wait for the next launch on the side stream,
+            // which runs beside an input-gradient GEMM.
+            m->pending_cols.push_back(pb[0]);
+            m->pending_cols.push_back(pb[1]);
+            if (m->pending_cols.size() >= (size_t)FT_THIN_MAX_BATCH) FT_TRY(flush_cols(m));
         } else if (accumulate) {
             FT_TRY(ft_lora_grad_b(ctx, t, dy, m->gtmp, T, l.out, l.r));
             FT_TRY(ft_gradient_accumulate(ctx, l.gb, m->gtmp, l.r * l.out));
-            FT_TRY(ft_lora_grad_a(ctx, x, m->dt, m->gtmp, T, l.in, l.r));
+            FT_TRY(ft_lora_grad_a(ctx, x, dt, m->gtmp, T, l.in, l.r));
             FT_TRY(ft_gradient_accumulate(ctx, l.ga, m->gtmp, l.in * l.r));
         } else {
             FT_TRY(ft_lora_grad_b(ctx, t, dy, l.gb, T, l.out, l.r));
-            FT_TRY(ft_lora_grad_a(ctx, x, m->dt, l.ga, T, l.in, l.r));
+            FT_TRY(ft_lora_grad_a(ctx, x, dt, l.ga, T, l.in, l.r));
         }
         if (dx)
-            FT_TRY(ft_lora_linear_dx(ctx, dy, l.w, l.dtype, m->dt, l.a, dx_add ? dx : nullptr, dx, T, l.in, l.out,
+            FT_TRY(ft_lora_linear_dx(ctx, dy, l.w, l.dtype, dt, l.a, dx_add ? dx : nullptr, dx, T, l.in, l.out,
                                      l.r));
     } else if (dx) {
         FT_TRY(ft_lora_linear_dx(ctx, dy, l.w, l.dtype, nullptr, nullptr, dx_add ? dx : nullptr, dx, T, l.in, l.out,
@@ -357,18 +405,22 @@ int linear_backward(ft_model* m, LinearW& l, const float* x, const float* t, con
 // over all the output gradients. Falls back to one linear at a time when the
 // adapters cannot be batched.
 int linear_backward_group(ft_model* m, LinearW* const* ls, const float* const* ts, const float* const* dys,
-                          float* dx, int n, const float* x, size_t T, bool accumulate) {
+                          float* dx, int n, const float* x, size_t T, bool accumulate, bool flush) {
     ft_context* ctx = m->ctx;
-    float* dts[3] = {m->dt, m->dt2, m->dt3};
     bool batch = n <= 3;
+    for (int i = 0; i < n; i++) batch = batch && ls[i]->has_lora() && ls[i]->r == ls[0]->r;
+    float* dts[3] = {nullptr, nullptr, nullptr};
+    if (batch) {
+        if (m->dt_used + n > ft_model::kDtPool) {
+            FT_TRY(flush_cols(m));
+            FT_TRY(join_cols(m));
+        }
+        for (int i = 0; i < n; i++) FT_TRY(take_dt(m, &dts[i]));
+    }
     const int acc = accumulate ? 1 : 0;
     ft_thin_problem rows[3], cols[6];
     for (int i = 0; i < n && batch; i++) {
         const LinearW& l = *ls[i];
-        if (!l.has_lora() || l.r != ls[0]->r) {
-            batch = false;
-            break;
-        }
         rows[i] = ft_thin_problem{dys[i], l.b, dts[i], (int)T, (int)l.out, 0, (int)l.r, (long)l.out, (long)l.out,
                                   (long)l.r, l.scale(), 1, 0, 0, 0};
         cols[2 * i] = ft_thin_problem{dys[i], ts[i], l.gb, (int)T, 0, (int)l.out, (int)l.r, (long)l.out, (long)l.r,
@@ -383,22 +435,20 @@ int linear_backward_group(ft_model* m, LinearW* const* ls, const float* const* t
         if (any_lora || n > 3) {
             for (int i = 0; i < n; i++)
                 FT_TRY(linear_backward(m, *ls[i], x, ts[i], dys[i], dx, T, accumulate, i > 0));
+            if (flush) FT_TRY(flush_cols(m));
             return FT_OK;
         }
         // frozen linears: only the summed input gradient is wanted
+        if (flush) FT_TRY(flush_cols(m));
         if (!dx) return FT_OK;
         ft_lora_dx_desc d[3];
         for (int i = 0; i < n; i++) d[i] = ft_lora_dx_desc{dys[i], ls[i]->w, ls[i]->dtype, nullptr, nullptr, ls[i]->out, 0};
         return ft_lora_linear_dx_group(ctx, d, (size_t)n, nullptr, dx, T, ls[0]->in);
     }
-    FT_TRY(ft_side_join(ctx, 0));  // factor gradients still in flight read the dt buffers
     FT_TRY(ft_thin_rowwise(ctx, rows, n));
-    {
-        FT_TRY(ft_side_begin(ctx));
-        const int rc = ft_thin_colwise(ctx, cols, 2 * n);
-        FT_TRY(ft_side_end(ctx));
-        FT_TRY(rc);
-    }
+    if (m->pending_cols.size() + 2 * (size_t)n > (size_t)FT_THIN_MAX_BATCH) FT_TRY(flush_cols(m));
+    for (int i = 0; i < 2 * n; i++) m->pending_cols.push_back(cols[i]);
+    if (flush || m->pending_cols.size() >= (size_t)FT_THIN_MAX_BATCH) FT_TRY(flush_cols(m));
     if (dx) {
         ft_lora_dx_desc d[3];
         for (int i = 0; i < n; i++)
@@ -532,11 +582,15 @@ int model_backward(ft_model* m, size_t B, size_t S, bool accumulate) {
     for (size_t li = m->layers.size(); li-- > 0;) {
         Layer& L = m->layers[li];
         LayerActs& a = m->acts[li];
+        // The factor gradients of the block above (side stream) read its output gradients (g_other,
+        // dq/dk/dv; d_up/d_gate when the MLP has adapters) and, with checkpointing, the shared block
+        // buffers. All of those are rewritten below: wait for the side stream before the first such
+        // write, as late as possible so that short GEMMs (one sequence per pass) still hide it.
+        const bool join_at_top = c.checkpoint_blocks || L.up.has_lora() || L.gate.has_lora() || L.down.has_lora();
+        if (join_at_top) FT_TRY(join_cols(m));
         if (c.checkpoint_blocks && li + 1 < m->layers.size()) {
-            // The shared block buffers hold the next block's internals, which its factor gradients
-            // (side stream) may still be reading: wait, then recompute this block's forward. (The
-            // last block's internals are still there from the forward pass.)
-            FT_TRY(ft_side_join(ctx, 0));
+            // Recompute this block's forward. (The last block's internals are still there from the
+            // forward pass.)
             FT_TRY(layer_forward(m, li, B, S));
         }
         // x_next = h + down(silu(gate) * up)
@@ -551,9 +605,10 @@ int model_backward(ft_model* m, size_t B, size_t S, bool accumulate) {
             LinearW* ls[2] = {&L.up, &L.gate};
             const float* ts[2] = {a.tup, a.tgate};
             const float* dys[2] = {m->d_up, m->d_gate};
-            FT_TRY(linear_backward_group(m, ls, ts, dys, m->d_h2, 2, a.h2, T, accumulate));
+            FT_TRY(linear_backward_group(m, ls, ts, dys, m->d_h2, 2, a.h2, T, accumulate, false));
         }
         // g_h = g + norm2_backward(d_h2) (into g_other)
+        if (!join_at_top) FT_TRY(join_cols(m));
         FT_TRY(ft_internal_rms_norm_backward_add(ctx, a.h, L.norm2, m->d_h2, g, g_other, T, H, c.rms_norm_eps));
         // h = x + o_proj(attn)
         FT_TRY(linear_backward(m, L.o, a.attn, a.to, g_other, m->d_attn, T, accumulate));
@@ -581,13 +636,17 @@ int model_backward(ft_model* m, size_t B, size_t S, bool accumulate) {
             const float* ts[3] = {a.tq, a.tk, a.tv};
             const float* dys[3] = {m->dq, m->dk, m->dv};
             // d_h1 = dx_q + dx_k + dx_v
-            FT_TRY(linear_backward_group(m, ls, ts, dys, need_dx ? m->d_h1 : nullptr, 3, a.h1, T, accumulate));
+            // the block's last adapters: everything that waited goes to the side stream now
+            FT_TRY(linear_backward_group(m, ls, ts, dys, need_dx ? m->d_h1 : nullptr, 3, a.h1, T, accumulate, true));
         }
         if (!need_dx) break;
+        // g is rewritten next; the down projection's factor gradients read it
+        if (L.down.has_lora()) FT_TRY(join_cols(m));
         // g = g_h + norm1_backward(d_h1)
         FT_TRY(ft_internal_rms_norm_backward_add(ctx, a.x, L.norm1, m->d_h1, g_other, g, T, H, c.rms_norm_eps));
     }
-    return ft_side_join(ctx);
+    FT_TRY(flush_cols(m));
+    return join_cols(m);
 }
 
 LinearW* find_linear(ft_model* m, const std::string& prefix) {

@@ -252,6 +252,22 @@ int ft_thin_colwise(ft_context* ctx, const ft_thin_problem* probs, int count) {
     int slices = mmax / 128;
     if (slices > 16) slices = 16;
     if (slices < 1) slices = 1;
+    // A batch whose partial sums do not fit the scratch buffer goes out in pieces (the launches of
+    // one stream run in order, so the pieces may share the buffer).
+    {
+        size_t need = 0;
+        int fit = 0;
+        while (fit < count && need + (size_t)slices * probs[fit].R * probs[fit].C <= kScratchFloats) {
+            need += (size_t)slices * probs[fit].R * probs[fit].C;
+            fit++;
+        }
+        FT_CHECK_ARG(fit >= 1, "thin colwise: %zu partial sums of one product exceed the scratch buffer",
+                     (size_t)slices * probs[0].R * probs[0].C);
+        if (fit < count) {
+            FT_TRY(ft_thin_colwise(ctx, probs, fit));
+            return ft_thin_colwise(ctx, probs + fit, count - fit);
+        }
+    }
     size_t off = 0;
     for (int i = 0; i < count; i++) {
         b.p[i] = probs[i];
