@@ -19,7 +19,10 @@
  *    `UnifiedTensor::from_f32_as_f16` (tensor.rs:258-269): element i at byte 2*i.
  *  - Ops only enqueue work on the context's stream and return
  *    (context.rs:291-317); order of execution = order of calls;
- *    `ft_synchronize` waits (context.rs:380-391).
+ *    `ft_synchronize` waits (context.rs:380-391). The training step also uses a
+ *    second stream that the context owns (the LoRA factor gradients run there,
+ *    beside the input-gradient GEMMs); it is joined before anything reads them
+ *    and by `ft_synchronize` / `ft_download`.
  *  - Outputs are caller-allocated and written, never accumulated into, except
  *    the in-place ops (rope, gradient_scale, clip_grad_by_norm,
  *    gradient_accumulate, adamw_update), as in the reference.
