@@ -1,0 +1,92 @@
+"""The step at BASELINE.json's full headline size (SmolLM2-360M shape, 8 x 256, vocabulary 49152).
+
+The oracle finishes one 256-token sequence of this model in seconds, so one sequence is compared with
+it element by element (loss, gradient norm, every LoRA gradient); the full batch is checked through
+properties that do not depend on size: two runs agree to the bit, and eight one-sequence passes
+accumulate to the batched step (loss, gradient norm and every gradient).
+"""
+import numpy as np
+import pytest
+
+import bench
+from oracle import reference_step as rs
+from tests.gpu_util import assert_close
+
+pytestmark = pytest.mark.gpu
+
+W = bench.WORKLOADS["360m"]
+
+
+@pytest.fixture(scope="module")
+def world():
+    from ferrotensor_amd import HipContext
+    from ferrotensor_amd.trainer import Lfm2Model, ModelConfig
+    ctx = HipContext(0)
+    cfg = ModelConfig(vocab_size=W["vocab"], hidden_size=W["hidden"], intermediate_size=W["ffn"],
+                      num_hidden_layers=W["layers"], num_attention_heads=W["heads"], num_key_value_heads=W["kv"],
+                      rms_norm_eps=1e-5, rope_theta=100000.0, tie_word_embeddings=True, f16_linears=True)
+    tensors = dict(bench.synthetic_tensors(W))
+    model = Lfm2Model(ctx, cfg)
+    model.load_tensors(tensors)
+    factors = list(bench.lora_factors(model, W))
+    yield ctx, model, tensors, factors
+    model.close()
+    ctx.close()
+
+
+def reset_adapters(model, factors):
+    for name, a, b in factors:
+        model.set_lora(name, a, b, W["alpha"])
+
+
+def run_step(model, factors, rows, targets, masks, micro):
+    from ferrotensor_amd.trainer import Trainer
+    reset_adapters(model, factors)
+    tr = Trainer(model, lr=2e-4, weight_decay=0.0, clip_grad_norm=1.0, grad_accum_steps=len(rows))
+    per_seq = []
+    st = None
+    for i in range(0, len(rows), micro):
+        st = tr.train_chunk(rows[i:i + micro], targets[i:i + micro], masks[i:i + micro], apply=False)
+        per_seq.append(st.loss)
+    grads = model.grads()
+    tr.close()
+    return st, per_seq, grads
+
+
+def test_full_size_batch_properties(world):
+    ctx, model, _, factors = world
+    rows, targets, masks = bench.synthetic_batch(W)
+    st_a, _, g_a = run_step(model, factors, rows, targets, masks, micro=8)
+    st_b, _, g_b = run_step(model, factors, rows, targets, masks, micro=8)
+    assert np.isfinite(st_a.loss) and st_a.tokens == int(masks.sum())
+    # determinism at the real shape: every reduction of the step has a fixed order
+    assert (st_a.loss, st_a.grad_norm) == (st_b.loss, st_b.grad_norm)
+    for k in g_a:
+        assert np.array_equal(g_a[k].view(np.uint32), g_b[k].view(np.uint32)), k
+    # eight one-sequence passes (split-K GEMMs, accumulated factor gradients) add up to the batched step
+    st_c, per_seq, g_c = run_step(model, factors, rows, targets, masks, micro=1)
+    assert_close("sum of the per-sequence losses", [sum(per_seq)], [st_a.loss])
+    assert_close("grad norm", [st_c.grad_norm], [st_a.grad_norm])
+    scale = max(float(np.abs(g).max()) for g in g_a.values())
+    for k in g_a:
+        # gradients of this model are ~1e-3 and smaller: the absolute term of the parity bar, scaled to them
+        assert_close("accumulated " + k, g_c[k], g_a[k], atol=1e-4 * scale, rtol=1e-3)
+
+
+def test_one_full_size_sequence_matches_the_oracle(world):
+    ctx, model, tensors, factors = world
+    cfg = rs.ModelConfig(W["vocab"], W["hidden"], W["ffn"], W["layers"], W["heads"], W["kv"], 1e-5, 100000.0, True)
+    orc = rs.Model.from_hf_tensors(cfg, tensors, f16_linears=True)
+    for name, a, b in factors:
+        orc.set_lora(name, a, b, W["alpha"])
+    rows, targets, masks = bench.synthetic_batch(W, B=1)
+    st, _, grads = run_step(model, factors, rows, targets, masks, micro=1)
+    want_stats, _, want_grads = rs.train_chunk(orc, rs.AdamW(lr=2e-4, weight_decay=0.0), rows, targets, masks,
+                                               grad_accum_steps=1, clip_grad_norm=1.0, return_grads=True)
+    clip = np.float32(want_stats.clip_scale or 1.0)   # the oracle hands back the clipped gradients
+    assert_close("loss", [st.loss], [want_stats.loss])
+    assert_close("grad norm", [st.grad_norm], [want_stats.grad_norm])
+    scale = max(float(np.abs(g).max()) for g in want_grads.values()) / float(clip)
+    for k in grads:
+        # gradients of this model are ~1e-2 and smaller: the absolute term of the parity bar, scaled to them
+        assert_close("grad " + k, grads[k], want_grads[k] / clip, atol=1e-4 * scale, rtol=1e-3)
