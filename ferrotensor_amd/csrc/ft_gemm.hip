@@ -660,8 +660,11 @@ __global__ __launch_bounds__(256) void gemm_async_kernel(AsyncBatch g) {
     __shared__ __attribute__((aligned(16))) float St0[STAGE];
     __shared__ __attribute__((aligned(16))) float St1[STAGE];
     __shared__ __attribute__((aligned(16))) float St2[STAGE];
-    __shared__ __attribute__((aligned(16))) float ExAs[NB == 1 ? ExA::LDS_FLOATS : 4];
-    __shared__ __attribute__((aligned(16))) float ExBs[NB == 1 ? ExB::LDS_FLOATS : 4];
+    // The rank-r products' operand tiles take the first stage's place once the K loop is over:
+    // a stage set of their own would cost the 128x128 tile its second workgroup per CU.
+    static_assert(ExA::LDS_FLOATS % 4 == 0 && ExA::LDS_FLOATS + ExB::LDS_FLOATS <= STAGE, "rank-r tiles fit a stage");
+    float* const ExAs = St0;
+    float* const ExBs = St0 + ExA::LDS_FLOATS;
 
     // Workgroup -> tile. The products of a batch form one row of n tiles per row block
     // (tile_begin = a product's first n tile). Tile order: panels of `panel` n tiles; inside a
@@ -875,12 +878,13 @@ __global__ __launch_bounds__(256) void gemm_async_kernel(AsyncBatch g) {
         if (t + 2 < nt) iter(t + 2, St2, St1);
     }
 
-    bool ext_used = false;
 #pragma unroll
     for (int s = 0; s < NSEG; s++) {
         if (has_ext[s]) {  // never with two b matrices
-            if (ext_used) __syncthreads();  // the previous segment's tile is still being read
-            ext_used = true;
+            // The stage is free when every wave's loads have landed and every wave has left the
+            // last K tile (or the previous segment's rank-r tile).
+            __builtin_amdgcn_s_waitcnt(0x0F70);
+            __syncthreads();
             xa[s].template store<float>(ExAs);
             xb[s].template store<float>(ExBs);
             __syncthreads();
@@ -1277,7 +1281,7 @@ int launch_async(ft_context* ctx, AsyncBatch g, int layout, int epi = kEpiPlain)
     // per n tile).
     g.xcds = ft_gemm_xcds(ctx);
     {
-        const double resident = 32.0 * (BM == 64 ? 3 : 2);
+        const double resident = 32.0 * (BM == 64 ? (epi == kEpiGateUp ? 3 : 4) : 2);
         const double a_blk = a_bytes / tiles_m, b_blk = b_bytes / (tiles_n > 0 ? tiles_n : 1);
         int want = b_blk > 0 ? (int)(sqrt(resident * a_blk / b_blk) + 0.5) : tiles_n;
         if (want < 1) want = 1;
@@ -1387,8 +1391,8 @@ int launch_async(ft_context* ctx, AsyncBatch g, int layout, int epi = kEpiPlain)
 // Tile choice, from measurements of the whole step on MI355X at M = 2048: 128x128
 // tiles (64x64 per wave) reach the highest MFMA rate but only pay off when there
 // are many of them per CU (the vocabulary head); everything else runs best as
-// 64x64 tiles, three workgroups resident per CU (128x64 and 64x128 tiles were
-// measured too: no gain inside the step).
+// 64x64 tiles, four workgroups resident per CU (three with two b tiles per stage; 128x64
+// and 64x128 tiles were measured too: no gain inside the step).
 int launch_async_auto(ft_context* ctx, const AsyncBatch& g, int layout) {
     size_t tiles128 = 0;
     for (int i = 0; i < g.count; i++) tiles128 += (size_t)((g.M + 127) / 128) * (size_t)((g.p[i].N + 127) / 128);
