@@ -141,6 +141,7 @@ SIGNATURES = {
     "ft_trainer_get_adam_t": [_P, C.POINTER(_F)],
     "ft_trainer_set_adam_t": [_P, _F],
     "ft_trainer_optimizer_steps": [_P, C.POINTER(_SZ)],
+    "ft_trainer_step_in_accum": [_P, C.POINTER(_SZ)],
     "ft_trainer_set_optimizer_steps": [_P, _SZ],
     "ft_lora_seed": [C.c_uint64, C.c_char_p],
     "ft_lora_init_a": [_P, _SZ, _SZ, _SZ, C.c_uint64],

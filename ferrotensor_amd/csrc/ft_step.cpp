@@ -140,6 +140,7 @@ struct ft_trainer {
     float t = 0.0f;                 // AdamW step counter (f32, as in the reference)
     size_t optimizer_steps = 0;     // steps taken = position of the LR schedule
     size_t step_in_accum = 0;
+    bool window_has_grads = false;  // a backward pass has written the gradient buffers in this window
     std::vector<float*> m, v;       // per parameter
     ft_segment* segs_dev = nullptr;
     size_t nseg = 0;
@@ -1126,6 +1127,12 @@ int ft_trainer_set_adam_t(ft_trainer* t, float steps) {
     return FT_OK;
 }
 
+int ft_trainer_step_in_accum(ft_trainer* t, size_t* sequences) {
+    FT_CHECK_ARG(t && sequences, "ft_trainer_step_in_accum: NULL argument");
+    *sequences = t->step_in_accum;
+    return FT_OK;
+}
+
 int ft_trainer_set_optimizer_steps(ft_trainer* t, size_t steps) {
     FT_CHECK_ARG(t, "ft_trainer_set_optimizer_steps: NULL argument");
     t->optimizer_steps = steps;
@@ -1165,11 +1172,17 @@ int ft_trainer_train_chunk(ft_trainer* t, const uint32_t* rows, const uint32_t* 
             const float gscale = std::fabs(seed - 1.0f) > kF32Epsilon ? seed : 1.0f;
             FT_TRY(ft_masked_cross_entropy_weighted(ctx, m->logits, m->targets_dev, m->weights_dev, m->logits,
                                                     m->row_loss, ce_rows, V, gscale));
-            FT_TRY(model_backward(m, B, S, t->step_in_accum > 0));
+            // The first backward of a window overwrites the gradient buffers (the reference's
+            // zero_grad after every optimizer step); later ones add to them.
+            FT_TRY(model_backward(m, B, S, t->window_has_grads));
+            t->window_has_grads = true;
             t->step_in_accum += B;
         }
 
         const bool window_full = t->step_in_accum >= accum;
+        // A window without any supervised token has no gradients: apply_gradients returns
+        // before the norm and the optimizer (trainer/src/lib.rs:301-307).
+        const bool have_grads = t->window_has_grads;
         bool launched_update = false;
         // Step k (1-based) uses the schedule's value at k (trainer/src/lib.rs:345-352).
         const float lr = ft_lr_schedule(t->cfg.lr_schedule, t->cfg.lr, t->cfg.min_lr, t->cfg.warmup_steps,
@@ -1177,7 +1190,8 @@ int ft_trainer_train_chunk(ft_trainer* t, const uint32_t* rows, const uint32_t* 
         ft_adam_params ap{lr, t->cfg.beta1, t->cfg.beta2, t->cfg.eps, t->cfg.weight_decay, t->t + 1.0f};
         if (window_full) {
             t->step_in_accum = 0;
-            if (total_tokens > 0 || true) {
+            t->window_has_grads = false;
+            if (have_grads) {
                 FT_TRY(ft_internal_multi_grad_norm(ctx, t->segs_dev, t->nseg, t->partials, t->cfg.clip_grad_norm,
                                                    t->control));
                 if (apply) {
@@ -1189,7 +1203,7 @@ int ft_trainer_train_chunk(ft_trainer* t, const uint32_t* rows, const uint32_t* 
 
         // The step's only wait: row losses and the control block.
         if (total_tokens > 0) FT_TRY(read_sequence_losses(m, B, S, tokens, head, per_sequence_loss, &stats->loss));
-        if (window_full) {
+        if (window_full && have_grads) {
             float control[3];
             FT_TRY(ft_download(ctx, control, t->control, sizeof(control)));
             int applied;

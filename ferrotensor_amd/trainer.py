@@ -231,6 +231,7 @@ class Trainer:
         ferrotensor-cli/src/main.rs:1686-1695); `lr` is the peak rate."""
         self.model = model
         self.length_bucket = length_bucket
+        self.grad_accum_steps = grad_accum_steps
         self._lib = model._lib
         self.hyper = dict(lr=lr, beta1=beta1, beta2=beta2, eps=eps, weight_decay=weight_decay)
         kind = LR_SCHEDULES[lr_schedule]
@@ -267,12 +268,28 @@ class Trainer:
         """Resume: restores the step counter, which is also the position of the LR schedule."""
         check(self._lib.ft_trainer_set_optimizer_steps(self.handle, steps))
 
-    def train_batch(self, seqs, apply: bool = True) -> StepStats:
-        """Ragged sequences [(input_ids, target_ids, loss_mask)]: dropped when
-        unsupervised or shorter than 2 tokens (trainer/src/lib.rs:385-398), padded, trained."""
-        kept = [(i, t, m) for i, t, m in seqs if len(i) >= 2 and len(t) > 0 and any(m)]
-        rows, targets, masks = pad_chunk(kept, self.length_bucket)
-        return self.train_chunk(rows, targets, masks, apply)
+    @property
+    def step_in_accum(self) -> int:
+        """Sequences counted into the open accumulation window."""
+        n = C.c_size_t()
+        check(self._lib.ft_trainer_step_in_accum(self.handle, C.byref(n)))
+        return n.value
+
+    def train_batch(self, seqs, apply: bool = True) -> List[StepStats]:
+        """`Trainer::train_batch` (trainer/src/lib.rs:371-423) for ragged sequences
+        [(input_ids, target_ids, loss_mask)]: those without a supervised token or shorter
+        than 2 tokens are dropped; the rest go through `train_chunk` in chunks that end at
+        the accumulation boundary, so the optimizer steps after the same sequence as when
+        they are trained one at a time. One StepStats per chunk; none when nothing is left."""
+        kept = [(i, t, m) for i, t, m in seqs if min(len(i), len(t)) >= 2 and any(m[:min(len(i), len(t))])]
+        out = []
+        accum = self.grad_accum_steps
+        while kept:
+            room = max(accum - self.step_in_accum, 1) if accum else len(kept)
+            chunk, kept = kept[:room], kept[room:]
+            rows, targets, masks = pad_chunk(chunk, self.length_bucket)
+            out.append(self.train_chunk(rows, targets, masks, apply))
+        return out
 
     def close(self):
         if self.handle is not None and self.handle.value:

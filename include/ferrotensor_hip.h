@@ -462,6 +462,10 @@ int ft_trainer_get_adam_t(ft_trainer* t, float* steps);
 int ft_trainer_set_adam_t(ft_trainer* t, float steps);
 int ft_trainer_optimizer_steps(ft_trainer* t, size_t* steps);
 int ft_trainer_set_optimizer_steps(ft_trainer* t, size_t steps);
+/* Trainer::step_in_accum (trainer/src/lib.rs:463-466): sequences counted into the open
+ * accumulation window. train_batch cuts its chunks at grad_accum_steps minus this, so the
+ * optimizer steps after the same sequence as in the one-at-a-time path (:413-423). */
+int ft_trainer_step_in_accum(ft_trainer* t, size_t* sequences);
 /* Trainer::train_chunk (trainer/src/lib.rs:426-502) for B equally long rows
  * (already padded; see ft_pad_chunk): forward, masked cross-entropy, backward
  * with seed 1/grad_accum_steps, gradient norm, clip, AdamW. rows/targets are
@@ -470,7 +474,12 @@ int ft_trainer_set_optimizer_steps(ft_trainer* t, size_t steps);
  * no optimizer step). The final norm, the vocabulary head and the loss run on
  * the supervised positions only (a position without a target has zero loss and
  * a zero logits gradient, kernels.wgsl:684-711; see ft_model_config.head_all_rows);
- * ft_model_forward_logits still returns the logits of every position. */
+ * ft_model_forward_logits still returns the logits of every position.
+ * Accumulation follows the reference: the sequences of a chunk count towards
+ * grad_accum_steps; the chunk that fills the window takes the norm / clip /
+ * optimizer step; a chunk without a supervised token runs no backward, and a
+ * window in which no chunk had one takes no step (apply_gradients returns early,
+ * trainer/src/lib.rs:301-307: grad_norm 0, optimizer_step 0). */
 int ft_trainer_train_chunk(ft_trainer* t, const uint32_t* rows, const uint32_t* targets,
                            const uint8_t* loss_mask, size_t B, size_t S, int apply,
                            ft_step_stats* stats, float* per_sequence_loss);

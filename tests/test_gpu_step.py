@@ -97,16 +97,87 @@ def test_model_directory_loader_and_adapter_file_reproduce_the_fixture(ctx, fx, 
 
 def test_padding_to_bucket_changes_nothing(ctx, fx):
     """Rows padded to 32 with their last token and mask 0 (trainer/src/lib.rs:431-450)."""
-    from ferrotensor_amd.trainer import Trainer
+    from ferrotensor_amd.trainer import Trainer, pad_chunk
     rows, targets, masks, _, want_loss = fx.case("masked")
     model = hip_model_from_fixture(ctx, fx)
     tr = Trainer(model, lr=1e-3, grad_accum_steps=1)
     seqs = [(list(r), list(t), list(m)) for r, t, m in zip(rows, targets, masks)]
-    st = tr.train_batch(seqs, apply=False)
+    prow, ptgt, pmask = pad_chunk(seqs, 32)
+    assert prow.shape == (len(seqs), 32)
+    st = tr.train_chunk(prow, ptgt, pmask, apply=False)
     assert worst_ratio([st.loss], [want_loss]) <= 1.0
     want = fx.expected_grads("masked")
     grads = model.grads()
     assert max(worst_ratio(grads[n], want[n]) for n in want) <= 1.0
+
+
+def test_train_batch_steps_after_the_same_sequences_as_one_at_a_time(ctx, fx):
+    """`train_batch` drops unsupervised sequences and cuts its chunks at the accumulation
+    boundary (trainer/src/lib.rs:385-423; the reference's gpu_training.rs:127-186 checks the
+    same equivalence): three kept sequences with grad_accum_steps 2 step after the second one
+    and leave the third in an open window, batched or one at a time."""
+    from ferrotensor_amd.trainer import Trainer
+    rows, targets, masks, _, _ = fx.case("masked")
+    seqs = [(list(r), list(t), list(m)) for r, t, m in zip(rows, targets, masks)]
+    third = (seqs[0][0][::-1], seqs[0][1][::-1], seqs[0][2])
+    batch = [seqs[0], (seqs[1][0], seqs[1][1], [0] * len(seqs[1][2])), (seqs[0][0][:1], seqs[0][1][:1], [1]),
+             seqs[1], third]
+
+    def run(one_at_a_time):
+        model = hip_model_from_fixture(ctx, fx)
+        tr = Trainer(model, lr=1e-2, weight_decay=0.0, grad_accum_steps=2, clip_grad_norm=1.0)
+        if one_at_a_time:
+            stats = [s for q in batch for s in tr.train_batch([q])]
+        else:
+            stats = tr.train_batch(batch)
+        out = (stats, tr.optimizer_steps, tr.step_in_accum, model.params(), model.grads())
+        tr.close()
+        model.close()
+        return out
+
+    stats_b, steps_b, open_b, params_b, grads_b = run(False)
+    stats_s, steps_s, open_s, params_s, grads_s = run(True)
+    assert [len(s.per_sequence) for s in stats_b] == [2, 1] and len(stats_s) == 3
+    assert [s.optimizer_step for s in stats_b] == [True, False]
+    assert [s.optimizer_step for s in stats_s] == [False, True, False]
+    assert (steps_b, open_b) == (1, 1) and (steps_s, open_s) == (1, 1)
+    assert worst_ratio([stats_b[0].loss], [stats_s[0].loss + stats_s[1].loss]) <= 1.0
+    assert worst_ratio([stats_b[0].grad_norm], [stats_s[1].grad_norm]) <= 1.0
+    for n in params_b:
+        assert worst_ratio(params_b[n], params_s[n]) <= 1.0, n
+        assert worst_ratio(grads_b[n], grads_s[n]) <= 1.0, n   # the open window: the third sequence alone
+    assert Trainer(hip_model_from_fixture(ctx, fx), lr=1e-2).train_batch([batch[1], batch[2]]) == []
+
+
+def test_a_window_without_supervised_tokens_takes_no_step(ctx, fx):
+    """No supervised token: no backward; a window of such chunks has no gradients and
+    apply_gradients returns before the norm and the optimizer (trainer/src/lib.rs:301-307).
+    The stale gradients of the previous window must neither be applied nor added to."""
+    from ferrotensor_amd.trainer import Trainer
+    rows, targets, masks, _, _ = fx.case("masked")
+    model = hip_model_from_fixture(ctx, fx)
+    tr = Trainer(model, lr=1e-2, weight_decay=0.0, grad_accum_steps=2)
+    first = tr.train_chunk(rows, targets, masks)
+    assert first.optimizer_step and tr.optimizer_steps == 1
+    before = model.params()
+    blank = tr.train_chunk(rows, targets, np.zeros_like(masks))
+    assert not blank.optimizer_step and blank.tokens == 0 and blank.loss == 0.0 and blank.grad_norm == 0.0
+    assert tr.optimizer_steps == 1 and tr.step_in_accum == 0
+    after = model.params()
+    for n in before:
+        assert np.array_equal(before[n], after[n]), n
+    # an empty chunk that opens a window, then a supervised one that closes it: its gradient alone
+    tr.train_chunk(rows[:1], targets[:1], np.zeros_like(masks[:1]))
+    assert tr.step_in_accum == 1
+    tr.train_chunk(rows[:1], targets[:1], masks[:1], apply=False)
+    got = model.grads()
+    ref_model = hip_model_from_fixture(ctx, fx)
+    ref_tr = Trainer(ref_model, lr=1e-2, weight_decay=0.0, grad_accum_steps=2)
+    ref_tr.train_chunk(rows, targets, masks)          # the same first step: same adapters as `model`
+    ref_tr.train_chunk(rows[:1], targets[:1], masks[:1], apply=False)
+    want = ref_model.grads()                           # one sequence in a window of two: never closed, seed 1/2
+    for n in want:
+        assert worst_ratio(got[n], want[n]) <= 1.0, n
 
 
 # ---- BASELINE config 1: tiny Llama, one full step vs the oracle ----------------
