@@ -703,6 +703,40 @@ __global__ __launch_bounds__(256) void gemm_async_kernel(AsyncBatch g) {
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
 
+    // Epilogue operands (the residual of `out = a@b + add`, gate and up of the SiLU-gate
+    // backward) are fetched before the K loop: their latency would otherwise be paid after the
+    // last MFMA, when the workgroups of a CU all finish together. Older than every tile load, so
+    // the loop's vmcnt waits cover them.
+    constexpr bool PRE = BM == 64 && BN == 64 && NSEG == 1 && (EPI == kEpiPlain || EPI == kEpiSiluBwd);
+    float pre1[PRE ? 16 : 1], pre2[PRE ? 16 : 1];  // plain: residual | (cos, sin); SiLU backward: gate, up
+    bool pre_add = false;
+    if constexpr (PRE) {
+        const float* s1 = EPI == kEpiSiluBwd ? p.e1 : p.add;
+        pre_add = EPI == kEpiSiluBwd || (p.add != nullptr && g.splits == 1 && p.rope == nullptr);
+        if (pre_add) {
+            const int col = n0 + wn0 + l32;
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int row = m0 + wm0 + (r / 4) * 8 + half * 4 + (r % 4);
+                const bool ok = row < M && col < p.N;
+                const long o = (long)row * p.ldc + col;
+                pre1[r] = ok ? s1[o] : 0.0f;
+                if constexpr (EPI == kEpiSiluBwd) pre2[r] = ok ? p.e2[o] : 0.0f;
+            }
+        }
+        if constexpr (EPI == kEpiPlain) {
+            if (p.rope) {  // the rotation's (cos, sin) of this lane's 16 rows
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const int row = m0 + wm0 + (r / 4) * 8 + half * 4 + (r % 4);
+                    const float2 cs = p.rope[(long)(row % p.rope_seq) * 32 + l32];
+                    pre1[r] = cs.x;
+                    pre2[r] = cs.y;
+                }
+            }
+        }
+    }
+
     // Uniform description of the segments (a missing one repeats the last: never reached).
     const char* abase[NSEG];
     const char* bbase[NSEG];
@@ -919,7 +953,9 @@ __global__ __launch_bounds__(256) void gemm_async_kernel(AsyncBatch g) {
             for (int r = 0; r < 16; r++) {
                 const int row = m0 + wm0 + (r / 4) * 8 + half * 4 + (r % 4);
                 if (row < M && col < p.N) {
-                    const float2 cs = p.rope[(long)(row % p.rope_seq) * 32 + l32];
+                    float2 cs;
+                    if constexpr (PRE) cs = make_float2(pre1[r], pre2[r]);
+                    else cs = p.rope[(long)(row % p.rope_seq) * 32 + l32];
                     const float self = acc[0][0][r], peer = other[r * 64 + lane];
                     // lower: x1*c - x2*s ; upper: x1*s + x2*c  (x1 = lower half, x2 = upper half)
                     p.out[(long)row * p.ldc + col] = upper ? peer * cs.y + self * cs.x : self * cs.x - peer * cs.y;
@@ -948,12 +984,16 @@ __global__ __launch_bounds__(256) void gemm_async_kernel(AsyncBatch g) {
                         p.out2[o] = x;
                         p.out3[o] = x * (1.0f / (1.0f + __expf(-x))) * up;
                     } else if constexpr (EPI == kEpiSiluBwd) {
-                        const float d = acc[i][j][r], x = p.e1[o], y = p.e2[o];
+                        const float d = acc[i][j][r], x = pre1[r], y = pre2[r];
                         const float sg = 1.0f / (1.0f + __expf(-x));
                         p.out2[o] = d * (x * sg);
                         p.out[o] = d * y * (sg * (1.0f + x * (1.0f - sg)));
                     } else {
-                        p.out[o] = p.add ? acc[i][j][r] + p.add[o] : acc[i][j][r];
+                        if constexpr (PRE) {
+                            p.out[o] = pre_add ? acc[i][j][r] + pre1[r] : (p.add ? acc[i][j][r] + p.add[o] : acc[i][j][r]);
+                        } else {
+                            p.out[o] = p.add ? acc[i][j][r] + p.add[o] : acc[i][j][r];
+                        }
                     }
                 }
             }
