@@ -38,9 +38,16 @@ struct AttnArgs {
     // rotated back through RoPE (the inverse rotation by the (cos, sin) of their token position,
     // table [Sq or Sk][32] float2), which is what RoPENode::backward does to them next.
     const float2* rope;
+    // dK/dV on the LDS kernel with few (key block, kv head) items: one workgroup per query head
+    // instead of per kv head writes that head's unscaled sums to part[2 * g + {0: dK, 1: dV}]
+    // (each laid out like dk), and attn_dkdv_combine_kernel adds the group in head order.
+    float* part;
+    int split_g;
 };
 
 #define MFMA(a, b, c) __builtin_amdgcn_mfma_f32_32x32x2f32((a), (b), (c), 0, 0, 0)
+
+constexpr size_t kAttnScratchFloats = (size_t)8 << 20;  // 32 MiB of per-head partial dK/dV
 
 __device__ __forceinline__ floatx16 zero16() {
     floatx16 z;
@@ -589,9 +596,13 @@ __global__ __launch_bounds__(512) void attn_bwd_dkdv_lds_kernel(AttnArgs p) {
     const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
     const int l32 = lane % 32, half = lane / 32;
     int blk_j, bh_i;
-    if (!attn_work_item((p.Sk + 31) / 32, p.B * p.Hkv, blk_j, bh_i)) return;
-    const int b = bh_i / p.Hkv, kvh = bh_i % p.Hkv;
-    const int G = p.H / p.Hkv;
+    if (!attn_work_item((p.Sk + 31) / 32, p.B * (p.split_g ? p.H : p.Hkv), blk_j, bh_i)) return;
+    const int Gfull = p.H / p.Hkv;
+    const int b = bh_i / (p.split_g ? p.H : p.Hkv);
+    const int hsel = bh_i % (p.split_g ? p.H : p.Hkv);
+    const int kvh = p.split_g ? hsel / Gfull : hsel;
+    const int g0 = p.split_g ? hsel % Gfull : 0;   // first query head of this workgroup within the group
+    const int G = p.split_g ? 1 : Gfull;           // and how many it covers
     const int kb0 = blk_j * 32;  // key block 0 has the most items under the causal mask: first
     const int key = kb0 + l32;
     const bool k_ok = key < p.Sk;
@@ -631,7 +642,7 @@ __global__ __launch_bounds__(512) void attn_bwd_dkdv_lds_kernel(AttnArgs p) {
     auto fetch = [&](int item) {
         const int g = item / per_head;
         const int q0 = (qb_start + item % per_head) * 32;
-        const int h = kvh * G + g;
+        const int h = kvh * Gfull + g0 + g;
         int qr = q0 + l32;
         const bool ok = qr < p.Sq;
         qr = ok ? qr : p.Sq - 1;
@@ -736,6 +747,12 @@ __global__ __launch_bounds__(512) void attn_bwd_dkdv_lds_kernel(AttnArgs p) {
                 sv += red[w * PRIV + DP * 33 + d * 33 + kk];
             }
             const long o = (((long)b * p.Sk + krow) * p.Hkv + kvh) * DP + d;
+            if (p.split_g) {
+                const long n_all = (long)p.B * p.Sk * p.Hkv * DP;
+                p.part[(2 * g0) * n_all + o] = sk;
+                p.part[(2 * g0 + 1) * n_all + o] = sv;
+                continue;
+            }
             p.dv[o] = sv;
             if (DP == 64 && p.rope) {
                 // dK rotated back: this thread also sums the partner element (d +- 32)
@@ -750,6 +767,33 @@ __global__ __launch_bounds__(512) void attn_bwd_dkdv_lds_kernel(AttnArgs p) {
                 p.dk[o] = sk * p.scale;  // dK = scale * sum dS Q (Q is read unscaled)
             }
         }
+    }
+}
+
+// dk = scale * sum over the group's query heads of part[2g] (rotated back through RoPE when
+// asked), dv = sum of part[2g + 1]; heads added in order. One thread per element.
+__global__ __launch_bounds__(256) void attn_dkdv_combine_kernel(AttnArgs p, int DP) {
+    const long n_all = (long)p.B * p.Sk * p.Hkv * DP;
+    const long i = (long)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n_all) return;
+    const int G = p.H / p.Hkv;
+    float sk = 0.0f, sv = 0.0f;
+    for (int g = 0; g < G; g++) {
+        sk += p.part[(2 * g) * n_all + i];
+        sv += p.part[(2 * g + 1) * n_all + i];
+    }
+    p.dv[i] = sv;
+    if (DP == 64 && p.rope) {
+        const int d = (int)(i % DP);
+        const long ip = d < 32 ? i + 32 : i - 32;
+        float sp = 0.0f;
+        for (int g = 0; g < G; g++) sp += p.part[(2 * g) * n_all + ip];
+        const int krow = (int)((i / ((long)p.Hkv * DP)) % p.Sk);
+        const float2 cs = p.rope[(long)krow * 32 + (d & 31)];
+        const float x = sk * p.scale, y = sp * p.scale;
+        p.dk[i] = d < 32 ? x * cs.x + y * cs.y : x * cs.x - y * cs.y;
+    } else {
+        p.dk[i] = sk * p.scale;
     }
 }
 
@@ -915,11 +959,10 @@ __global__ __launch_bounds__(kKeySplit * 64) void attn_fwd_lds_kernel(AttnArgs p
         p.stats[2 * (((long)b * p.H + h) * p.Sq + qi) + 1] = l_run > 0.0f ? m_run + __logf(l_run) : kLseEmpty;
 }
 
-template <int DP>
-__global__ __launch_bounds__(kKeySplitDq * 64) void attn_bwd_dq_lds_kernel(AttnArgs p) {
+template <int DP, int NSPL>
+__global__ __launch_bounds__(NSPL * 64) void attn_bwd_dq_lds_kernel(AttnArgs p) {
     constexpr int NF = DP / 32;
     constexpr int NS = DP / 8;
-    constexpr int NSPL = kKeySplitDq;
     constexpr int TILE = 32 * DP;
     constexpr int MERGE = 64 * NF * 16;
     constexpr int PRIV = TILE > MERGE ? TILE : MERGE;
@@ -1114,7 +1157,13 @@ int launch_bwd(ft_context* ctx, const AttnArgs& a) {
         bool done = false;
         if constexpr (DP <= 64) {
             if (full) {
-                hipLaunchKernelGGL((attn_bwd_dq_lds_kernel<DP>), grid, dim3(kKeySplitDq * 64), 0, ctx->stream, a);
+                // Few workgroups (one or two sequences per pass): four waves share a query block's
+                // keys instead of two, so the chip is not left to a long serial key loop.
+                if ((size_t)grid.x <= (size_t)ctx->num_cus && a.Sk > 64)
+                    hipLaunchKernelGGL((attn_bwd_dq_lds_kernel<DP, 4>), grid, dim3(4 * 64), 0, ctx->stream, a);
+                else
+                    hipLaunchKernelGGL((attn_bwd_dq_lds_kernel<DP, kKeySplitDq>), grid, dim3(kKeySplitDq * 64), 0,
+                                       ctx->stream, a);
                 done = true;
             }
         }
@@ -1136,8 +1185,28 @@ int launch_bwd(ft_context* ctx, const AttnArgs& a) {
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem_lds));
                 attr_lds = true;
             }
-            const dim3 grid3(attn_grid(ft_div_up(a.Sk, 32), (size_t)a.B * a.Hkv));
+            const size_t items = ft_div_up(a.Sk, 32) * (size_t)a.B * a.Hkv;
+            const size_t G = (size_t)a.H / a.Hkv;
+            const size_t n_all = (size_t)a.B * a.Sk * a.Hkv * DP;
             ft_prof_scope prof(ctx, "attn_bwd_dkdv_kernel", 1.5 * fl, by * 0.5);
+            // Few items (one or two sequences per pass) and a GQA group to share them out:
+            // one workgroup per query head, then the ordered sum over the group.
+            if (G > 1 && items * 2 <= (size_t)ctx->num_cus && 2 * G * n_all <= kAttnScratchFloats) {
+                if (!ctx->attn_scratch) {
+                    FT_HIP(hipSetDevice(ctx->device));
+                    FT_HIP(hipMalloc((void**)&ctx->attn_scratch, kAttnScratchFloats * sizeof(float)));
+                }
+                AttnArgs s = a;
+                s.part = ctx->attn_scratch;
+                s.split_g = 1;
+                const dim3 grid_s(attn_grid(ft_div_up(a.Sk, 32), (size_t)a.B * a.H));
+                hipLaunchKernelGGL((attn_bwd_dkdv_lds_kernel<DP>), grid_s, dim3(512), smem_lds, ctx->stream, s);
+                FT_LAUNCH_CHECK();
+                hipLaunchKernelGGL(attn_dkdv_combine_kernel, dim3(ft_div_up(n_all, 256)), dim3(256), 0, ctx->stream, s, DP);
+                FT_LAUNCH_CHECK();
+                return FT_OK;
+            }
+            const dim3 grid3(attn_grid(ft_div_up(a.Sk, 32), (size_t)a.B * a.Hkv));
             hipLaunchKernelGGL((attn_bwd_dkdv_lds_kernel<DP>), grid3, dim3(512), smem_lds, ctx->stream, a);
             FT_LAUNCH_CHECK();
             return FT_OK;

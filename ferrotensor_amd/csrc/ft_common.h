@@ -29,6 +29,8 @@ struct ft_context {
     float* thin_scratch = nullptr;
     // Partial tiles of split-K GEMMs (few output tiles, long K); allocated on first use.
     float* gemm_scratch = nullptr;
+    // Per-query-head partial dK/dV of the attention backward at small batch; allocated on first use.
+    float* attn_scratch = nullptr;
 
     // Extra streams ("lanes") for work that can run beside the main stream:
     // lane 0 carries the LoRA factor gradients of a training step (only the

@@ -204,6 +204,7 @@ int ft_context_destroy(ft_context* ctx) {
     }
     if (ctx->thin_scratch) (void)hipFree(ctx->thin_scratch);
     if (ctx->gemm_scratch) (void)hipFree(ctx->gemm_scratch);
+    if (ctx->attn_scratch) (void)hipFree(ctx->attn_scratch);
     if (ctx->owns_stream) (void)hipStreamDestroy(ctx->stream);
     delete ctx;
     return FT_OK;

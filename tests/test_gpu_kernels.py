@@ -436,6 +436,7 @@ ATTN_CASES = [
     (2, 256, 256, 9, 3, 64, True, 0),       # SmolLM2-135M heads at seq 256
     (8, 256, 256, 9, 3, 64, True, 0),       # the kernel-microbench attention case, full size
     (2, 256, 256, 15, 5, 64, True, 0),      # SmolLM2-360M heads
+    (1, 256, 256, 15, 5, 64, True, 0),      # one sequence per pass: dK/dV per query head + ordered sum, dQ on 4 waves
     (1, 70, 70, 2, 1, 128, True, 0),
     (1, 33, 65, 2, 1, 32, True, 32),        # queries at positions 32.. against a longer key run
     (1, 5, 37, 4, 4, 24, False, 0),
