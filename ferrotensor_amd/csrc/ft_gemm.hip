@@ -637,8 +637,11 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(SplitReduceArgs a) {
     reinterpret_cast<float4*>(a.out[pi])[i] = v;
 }
 
-template <int BM, int BN, int WM, int WN, int LAYOUT, int NSEG, int EPI = kEpiPlain>
-__global__ __launch_bounds__(256) void gemm_async_kernel(AsyncBatch g) {
+// KW = 2: eight waves; a stage holds two consecutive K tiles and waves 4-7 multiply the second
+// one of every stage for the same 64x64 output tile (the two sums meet in LDS after the loop):
+// twice the waves per SIMD for products whose tiles leave a CU with at most two workgroups.
+template <int BM, int BN, int WM, int WN, int LAYOUT, int NSEG, int EPI = kEpiPlain, int KW = 1>
+__global__ __launch_bounds__(256 * KW) void gemm_async_kernel(AsyncBatch g) {
     static_assert(LAYOUT == 0 || LAYOUT == 1, "a is k-contiguous on this path");
     static_assert(NSEG == 1 || NSEG == kAsyncMaxSeg, "one segment, or the general case");
     static_assert(EPI == kEpiPlain || NSEG == 1, "fused epilogues take one segment");
@@ -649,7 +652,9 @@ __global__ __launch_bounds__(256) void gemm_async_kernel(AsyncBatch g) {
     static_assert((BM / WM) * (BN / WN) == 4, "4 waves per workgroup");
     constexpr int A_FLOATS = BM * 32;             // f32 tile
     constexpr int B_FLOATS = BN * 16;             // f16 tile, in float units
-    constexpr int STAGE = A_FLOATS + NB * B_FLOATS;
+    constexpr int SUB = A_FLOATS + NB * B_FLOATS;  // one K tile of 32
+    constexpr int STAGE = KW * SUB;
+    static_assert(KW == 1 || (KW == 2 && EPI == kEpiPlain && BM == 64 && BN == 64), "K-sharing waves: plain 64x64 tiles");
     constexpr int A_CH = BM / 8 / 4;              // 1 KiB chunks per wave
     constexpr int B_CH = BN / 16 / 4;
     constexpr int LPT = A_CH + NB * B_CH;         // load instructions per wave per tile
@@ -691,7 +696,8 @@ __global__ __launch_bounds__(256) void gemm_async_kernel(AsyncBatch g) {
     const int M = g.M;
     const int m0 = tm * BM;
     const int n0 = (tn - p.tile_begin) * BN;
-    const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
+    const int lane = threadIdx.x % 64, wave = (threadIdx.x / 64) % 4;
+    const int grp = KW == 1 ? 0 : __builtin_amdgcn_readfirstlane((int)(threadIdx.x / 256));  // wave-uniform
     const int wm0 = (wave / WAVES_N) * WM, wn0 = (wave % WAVES_N) * WN;
     const int l32 = lane % 32, half = lane / 32;
 
@@ -712,7 +718,7 @@ __global__ __launch_bounds__(256) void gemm_async_kernel(AsyncBatch g) {
     bool pre_add = false;
     if constexpr (PRE) {
         const float* s1 = EPI == kEpiSiluBwd ? p.e1 : p.add;
-        pre_add = EPI == kEpiSiluBwd || (p.add != nullptr && g.splits == 1 && p.rope == nullptr);
+        pre_add = grp == 0 && (EPI == kEpiSiluBwd || (p.add != nullptr && g.splits == 1 && p.rope == nullptr));
         if (pre_add) {
             const int col = n0 + wn0 + l32;
 #pragma unroll
@@ -750,11 +756,12 @@ __global__ __launch_bounds__(256) void gemm_async_kernel(AsyncBatch g) {
         lda_b[s] = sg.lda * 4;
         ldb_b[s] = sg.ldb * 2;
         tend[s] = (s > 0 ? tend[s - 1] : 0) + (s < p.nseg ? sg.nt : 0);
-        has_ext[s] = NB == 1 && s < p.nseg && sg.a2 != nullptr;
+        has_ext[s] = NB == 1 && grp == 0 && s < p.nseg && sg.a2 != nullptr;
     }
     const char* balt = reinterpret_cast<const char*>(p.b_alt);
     // This workgroup's share of the K tiles: [t0, nt).
-    const int nt_all = tend[NSEG - 1];
+    // (KW = 2: counted in pairs of tiles; the host only chooses it when every segment has an even number.)
+    const int nt_all = tend[NSEG - 1] / KW;
     const int split = (int)blockIdx.y;
     const int t0 = (int)(((long)nt_all * split) / g.splits);
     const int nt = (int)(((long)nt_all * (split + 1)) / g.splits);
@@ -817,6 +824,8 @@ __global__ __launch_bounds__(256) void gemm_async_kernel(AsyncBatch g) {
 
     auto issue = [&](int t, float* st) {
         t = t < nt ? t : nt - 1;  // past the end: re-read the last tile into a stage nobody reads
+        t = KW * t + grp;         // this wave group's tile of the pair
+        st += grp * SUB;
         if constexpr (NSEG > 1) {
             int s = 0;
             if (t >= tend[0]) s = 1;
@@ -876,7 +885,8 @@ __global__ __launch_bounds__(256) void gemm_async_kernel(AsyncBatch g) {
     };
     // One K tile: wait for it, let everybody leave the stage that is about to
     // be refilled, refill it (tile t + NST - 1), multiply tile t.
-    auto iter = [&](int t, const float* cur, float* refill) {
+    auto iter = [&](int t, const float* stage, float* refill) {
+        const float* cur = stage + grp * SUB;
         __builtin_amdgcn_s_waitcnt(0x0F70 | (WAIT & 15) | ((WAIT >> 4) << 14));
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
@@ -912,6 +922,20 @@ __global__ __launch_bounds__(256) void gemm_async_kernel(AsyncBatch g) {
         if (t + 2 < nt) iter(t + 2, St2, St1);
     }
 
+    if constexpr (KW == 2) {
+        // The second wave group hands its sums over through the second stage and retires.
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+        __syncthreads();  // loads landed, every wave has left the last stage
+        float* red = St1 + wave * 64 + lane;
+        if (grp == 1) {
+#pragma unroll
+            for (int r = 0; r < 16; r++) red[r * 256] = acc[0][0][r];
+        }
+        __syncthreads();
+        if (grp == 1) return;
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[0][0][r] += red[r * 256];
+    }
 #pragma unroll
     for (int s = 0; s < NSEG; s++) {
         if (has_ext[s]) {  // never with two b matrices
@@ -1406,6 +1430,35 @@ int launch_async(ft_context* ctx, AsyncBatch g, int layout, int epi = kEpiPlain)
             return FT_OK;
         } else {
             return ft_set_error(FT_ERR_INVALID, "fused epilogues use 64x64 tiles");
+        }
+    }
+    // Eight waves on a tile when the tiles alone leave at most two workgroups on a CU and the K
+    // loop can be shared in pairs of tiles.
+    bool pairs = BM == 64 && !any_rope && g.splits == 1 && (size_t)tiles <= 2 * (size_t)ctx->num_cus && min_kt >= 32;
+    for (int i = 0; i < g.count && pairs; i++)
+        for (int s = 0; s < g.p[i].nseg; s++) pairs = pairs && g.p[i].seg[s].nt % 2 == 0;
+    if constexpr (BM == 64) {
+        if (pairs) {
+            snprintf(name, sizeof(name), "gemm_async_kernel<%d, %d, %d, %d, %d, %d>", BM, BN, WM, WN, layout,
+                     max_seg > 1 ? kAsyncMaxSeg : 1);
+            ft_prof_scope prof(ctx, name, flops, bytes);
+            if (max_seg == 1) {
+                if (layout == 0)
+                    hipLaunchKernelGGL((gemm_async_kernel<64, 64, 32, 32, 0, 1, kEpiPlain, 2>), grid, dim3(512), 0,
+                                       ctx->stream, g);
+                else
+                    hipLaunchKernelGGL((gemm_async_kernel<64, 64, 32, 32, 1, 1, kEpiPlain, 2>), grid, dim3(512), 0,
+                                       ctx->stream, g);
+            } else {
+                if (layout == 0)
+                    hipLaunchKernelGGL((gemm_async_kernel<64, 64, 32, 32, 0, kAsyncMaxSeg, kEpiPlain, 2>), grid,
+                                       dim3(512), 0, ctx->stream, g);
+                else
+                    hipLaunchKernelGGL((gemm_async_kernel<64, 64, 32, 32, 1, kAsyncMaxSeg, kEpiPlain, 2>), grid,
+                                       dim3(512), 0, ctx->stream, g);
+            }
+            FT_LAUNCH_CHECK();
+            return FT_OK;
         }
     }
     snprintf(name, sizeof(name), "gemm_async_kernel<%d, %d, %d, %d, %d, %d>", BM, BN, WM, WN, layout,

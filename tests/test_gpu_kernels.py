@@ -90,6 +90,27 @@ def test_f16_weight_projections(g, name, K, N, M):
     assert_close(f"{name} matmul_bt_f16b", dx.to_numpy(), f64_mm(gy, wr.T), atol=2e-3, rtol=1e-4)
 
 
+@pytest.mark.parametrize("M,K,N", [(1536, 2560, 960), (2048, 1024, 960), (1472, 2048, 896)])
+def test_long_k_products_on_eight_waves(g, M, K, N):
+    """320 to 512 output tiles of 64x64 and K >= 1024: the workgroup's eight waves share the K loop
+    in pairs of tiles (both operand layouts; 1472 rows: a ragged last row block)."""
+    from ferrotensor_amd import UnifiedTensor
+    ctx, eng = g
+    a, w = rnd(K + N, M, K), rnd(K * 2 + N, K, N, scale=0.05)
+    w16 = UnifiedTensor.from_f32_as_f16(ctx, w, [K, N])
+    wr = cpu.round_f16(w)
+    out = empty(ctx, M, N)
+    eng.matmul_f16b(ctx, up(ctx, a), w16, out)
+    assert_close("matmul_f16b", out.to_numpy(), f64_mm(a, wr), atol=2e-3, rtol=1e-4)
+    # the other layout contracts over the weight's second dimension: w2 [N, K], g [M, K] -> [M, N]
+    w2 = rnd(K + 3 * N, N, K, scale=0.05)
+    w2_16 = UnifiedTensor.from_f32_as_f16(ctx, w2, [N, K])
+    gy = rnd(9, M, K)
+    dx = empty(ctx, M, N)
+    eng.matmul_bt_f16b(ctx, up(ctx, gy), w2_16, dx)
+    assert_close("matmul_bt_f16b", dx.to_numpy(), f64_mm(gy, cpu.round_f16(w2).T), atol=2e-3, rtol=1e-4)
+
+
 def test_f16_upload_is_bit_exact(g):
     from ferrotensor_amd import DType, UnifiedTensor
     ctx, _ = g
