@@ -1374,10 +1374,21 @@ int launch_async(ft_context* ctx, AsyncBatch g, int layout, int epi = kEpiPlain)
     // the extra pass over the output is then a fraction of a percent.
     const bool few_tiles = (size_t)tiles * 4 <= (size_t)ctx->num_cus * 5;
     const bool long_k = (size_t)tiles * 2 < 3 * (size_t)ctx->num_cus && min_kt >= 512;
+    // Eight waves on a tile (two K tiles per stage, see the kernel) need whole pairs of tiles in every segment.
+    bool pairs_ok = BM == 64 && epi == kEpiPlain && !any_rope && min_kt >= 8;
+    for (int i = 0; i < g.count && pairs_ok; i++)
+        for (int s = 0; s < g.p[i].nseg; s++) pairs_ok = pairs_ok && g.p[i].seg[s].nt % 2 == 0;
+    bool pairs = false;
     if (epi == kEpiPlain && mn4 && !any_rope && tiles > 0 && (few_tiles || long_k)) {
         int want = (int)((2 * (size_t)ctx->num_cus + tiles - 1) / tiles);
         if (want > 8) want = 8;
         if (want > min_kt / 4) want = min_kt / 4;
+        // Many shares (one sequence per pass): the second wave group takes half of them, which
+        // halves the partial tiles. (Two or three shares are faster as they are: measured.)
+        if (want >= 4 && pairs_ok) {
+            pairs = true;
+            want = (want + 1) / 2;
+        }
         if (want >= 2 && out_floats * want <= kSplitScratchFloats) {
             if (!ctx->gemm_scratch) {
                 FT_HIP(hipSetDevice(ctx->device));
@@ -1434,9 +1445,7 @@ int launch_async(ft_context* ctx, AsyncBatch g, int layout, int epi = kEpiPlain)
     }
     // Eight waves on a tile when the tiles alone leave at most two workgroups on a CU and the K
     // loop can be shared in pairs of tiles.
-    bool pairs = BM == 64 && !any_rope && g.splits == 1 && (size_t)tiles <= 2 * (size_t)ctx->num_cus && min_kt >= 32;
-    for (int i = 0; i < g.count && pairs; i++)
-        for (int s = 0; s < g.p[i].nseg; s++) pairs = pairs && g.p[i].seg[s].nt % 2 == 0;
+    pairs = pairs || (pairs_ok && g.splits == 1 && (size_t)tiles <= 2 * (size_t)ctx->num_cus && min_kt >= 32);
     if constexpr (BM == 64) {
         if (pairs) {
             snprintf(name, sizeof(name), "gemm_async_kernel<%d, %d, %d, %d, %d, %d>", BM, BN, WM, WN, layout,
@@ -1458,7 +1467,7 @@ int launch_async(ft_context* ctx, AsyncBatch g, int layout, int epi = kEpiPlain)
                                        dim3(512), 0, ctx->stream, g);
             }
             FT_LAUNCH_CHECK();
-            return FT_OK;
+            return reduce_shares();
         }
     }
     snprintf(name, sizeof(name), "gemm_async_kernel<%d, %d, %d, %d, %d, %d>", BM, BN, WM, WN, layout,
