@@ -654,7 +654,7 @@ __global__ __launch_bounds__(256 * KW) void gemm_async_kernel(AsyncBatch g) {
     constexpr int B_FLOATS = BN * 16;             // f16 tile, in float units
     constexpr int SUB = A_FLOATS + NB * B_FLOATS;  // one K tile of 32
     constexpr int STAGE = KW * SUB;
-    static_assert(KW == 1 || (KW == 2 && EPI == kEpiPlain && BM == 64 && BN == 64), "K-sharing waves: plain 64x64 tiles");
+    static_assert(KW == 1 || (KW == 2 && BM == 64 && BN == 64), "K-sharing waves: 64x64 tiles");
     constexpr int A_CH = BM / 8 / 4;              // 1 KiB chunks per wave
     constexpr int B_CH = BN / 16 / 4;
     constexpr int LPT = A_CH + NB * B_CH;         // load instructions per wave per tile
@@ -926,15 +926,20 @@ __global__ __launch_bounds__(256 * KW) void gemm_async_kernel(AsyncBatch g) {
         // The second wave group hands its sums over through the second stage and retires.
         __builtin_amdgcn_s_waitcnt(0x0F70);
         __syncthreads();  // loads landed, every wave has left the last stage
+        static_assert(KW == 1 || FN * NB * 16 * 256 <= STAGE, "the hand-over fits a stage");
         float* red = St1 + wave * 64 + lane;
         if (grp == 1) {
 #pragma unroll
-            for (int r = 0; r < 16; r++) red[r * 256] = acc[0][0][r];
+            for (int j = 0; j < FN * NB; j++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) red[(j * 16 + r) * 256] = acc[0][j][r];
         }
         __syncthreads();
         if (grp == 1) return;
 #pragma unroll
-        for (int r = 0; r < 16; r++) acc[0][0][r] += red[r * 256];
+        for (int j = 0; j < FN * NB; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[0][j][r] += red[(j * 16 + r) * 256];
     }
 #pragma unroll
     for (int s = 0; s < NSEG; s++) {
@@ -1384,8 +1389,8 @@ int launch_async(ft_context* ctx, AsyncBatch g, int layout, int epi = kEpiPlain)
         if (want > 8) want = 8;
         if (want > min_kt / 4) want = min_kt / 4;
         // Many shares (one sequence per pass): the second wave group takes half of them, which
-        // halves the partial tiles. (Two or three shares are faster as they are: measured.)
-        if (want >= 4 && pairs_ok) {
+        // halves the partial tiles. (Up to five shares are faster as they are: measured.)
+        if (want >= 6 && pairs_ok) {
             pairs = true;
             want = (want + 1) / 2;
         }
@@ -1431,8 +1436,16 @@ int launch_async(ft_context* ctx, AsyncBatch g, int layout, int epi = kEpiPlain)
             const double mn = (double)g.M * g.p[0].N;
             ft_prof_scope prof(ctx, name, gu ? 2.0 * flops : flops,
                                gu ? bytes + 64.0 * g.p[0].N * g.p[0].seg[0].nt + 8.0 * mn : bytes + 12.0 * mn);
-            if (gu)
+            // Fewer tiles than CUs (one sequence per pass): eight waves share the K loop of a tile.
+            const bool few = (size_t)tiles <= (size_t)ctx->num_cus && g.p[0].seg[0].nt % 2 == 0 && g.p[0].seg[0].nt >= 8;
+            if (gu && few)
+                hipLaunchKernelGGL((gemm_async_kernel<64, 64, 32, 32, 0, 1, kEpiGateUp, 2>), grid, dim3(512), 0,
+                                   ctx->stream, g);
+            else if (gu)
                 hipLaunchKernelGGL((gemm_async_kernel<64, 64, 32, 32, 0, 1, kEpiGateUp>), grid, dim3(256), 0,
+                                   ctx->stream, g);
+            else if (few)
+                hipLaunchKernelGGL((gemm_async_kernel<64, 64, 32, 32, 1, 1, kEpiSiluBwd, 2>), grid, dim3(512), 0,
                                    ctx->stream, g);
             else
                 hipLaunchKernelGGL((gemm_async_kernel<64, 64, 32, 32, 1, 1, kEpiSiluBwd>), grid, dim3(256), 0,
