@@ -180,11 +180,12 @@ def measured_traffic(kernel, workload):
     if workload != "360m":
         return None
     path = os.path.join(ROOT, "profiles", "lora_step_360m_hbm_traffic.md")
+    # profile names -> kernel symbols: <.., layout, segments[, epilogue[, wave groups]]>
     name = kernel
-    for tag, code in (("gate_up", "1"), ("silu_bwd", "2")):
+    for tag, code in (("gate_up", "1, 1"), ("silu_bwd", "2, 1")):
         name = name.replace(", %s>" % tag, ", %s>" % code)
-    if name == kernel:
-        name = kernel[:-1] + ", 0>"
+    if name == kernel and kernel.count(",") == 5:
+        name = kernel[:-1] + ", 0, 1>"
     try:
         for line in open(path):
             cells = [c.strip() for c in line.split("|")]

@@ -1461,7 +1461,7 @@ int launch_async(ft_context* ctx, AsyncBatch g, int layout, int epi = kEpiPlain)
     pairs = pairs || (pairs_ok && g.splits == 1 && (size_t)tiles <= 2 * (size_t)ctx->num_cus && min_kt >= 32);
     if constexpr (BM == 64) {
         if (pairs) {
-            snprintf(name, sizeof(name), "gemm_async_kernel<%d, %d, %d, %d, %d, %d>", BM, BN, WM, WN, layout,
+            snprintf(name, sizeof(name), "gemm_async_kernel<%d, %d, %d, %d, %d, %d, 0, 2>", BM, BN, WM, WN, layout,
                      max_seg > 1 ? kAsyncMaxSeg : 1);
             ft_prof_scope prof(ctx, name, flops, bytes);
             if (max_seg == 1) {
