@@ -175,7 +175,9 @@ def test_fused_lora_linear_forward_and_backward(g, M, K, N, r, f16):
 
 @pytest.mark.parametrize("M,K,Ns,r,f16", [(256, 960, (960, 320, 320), 8, True), (100, 64, (64, 32, 96), 4, True),
                                           (192, 128, (320, 256), 0, True), (64, 32, (48, 40), 8, False),
-                                          (130, 96, (40, 72, 8), 16, True)])
+                                          (130, 96, (40, 72, 8), 16, True),
+                                          # the step's own shapes: the summed input gradient runs its K segments on eight waves
+                                          (2048, 960, (960, 320, 320), 8, True), (2048, 960, (2560, 2560), 0, True)])
 def test_grouped_linears_match_single_calls(g, M, K, Ns, r, f16):
     """q/k/v (gate/up) of one input in one launch, and their summed input gradient in one launch."""
     from ferrotensor_amd import UnifiedTensor
