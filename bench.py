@@ -107,7 +107,7 @@ def lora_factors(model, w, seed=2):
 
 
 def step_flops(w, head_rows=None):
-    """Algorithmic flops of one step (SURVEY convention): fwd + dX GEMMs on the
+    """Algorithmic flops of one step: `2 M N K` for the forward and input-gradient GEMMs on the
     frozen base incl. the head, LoRA products, attention fwd + 2.5x bwd. The head
     (and its input gradient) runs on `head_rows` rows: the supervised positions."""
     T = w["B"] * w["S"]
