@@ -1,4 +1,5 @@
-"""The step at BASELINE.json's full headline size (SmolLM2-360M shape, 8 x 256, vocabulary 49152).
+"""The step at BASELINE.json's full sizes: the headline (SmolLM2-360M shape, 8 x 256, vocabulary 49152)
+and the 135M shape (576 hidden: the GEMM shapes that split K).
 
 The oracle finishes one 256-token sequence of this model in seconds, so one sequence is compared with
 it element by element (loss, gradient norm, every LoRA gradient); the full batch is checked through
@@ -14,12 +15,10 @@ from tests.gpu_util import assert_close
 
 pytestmark = pytest.mark.gpu
 
-W = bench.WORKLOADS["360m"]
-
-
-@pytest.fixture(scope="module")
-def world():
+@pytest.fixture(scope="module", params=["360m", "135m"])
+def world(request):
     from ferrotensor_amd import HipContext
+    W = bench.WORKLOADS[request.param]
     from ferrotensor_amd.trainer import Lfm2Model, ModelConfig
     ctx = HipContext(0)
     cfg = ModelConfig(vocab_size=W["vocab"], hidden_size=W["hidden"], intermediate_size=W["ffn"],
@@ -29,19 +28,19 @@ def world():
     model = Lfm2Model(ctx, cfg)
     model.load_tensors(tensors)
     factors = list(bench.lora_factors(model, W))
-    yield ctx, model, tensors, factors
+    yield ctx, model, tensors, factors, W
     model.close()
     ctx.close()
 
 
-def reset_adapters(model, factors):
+def reset_adapters(model, factors, W):
     for name, a, b in factors:
         model.set_lora(name, a, b, W["alpha"])
 
 
-def run_step(model, factors, rows, targets, masks, micro):
+def run_step(model, factors, W, rows, targets, masks, micro):
     from ferrotensor_amd.trainer import Trainer
-    reset_adapters(model, factors)
+    reset_adapters(model, factors, W)
     tr = Trainer(model, lr=2e-4, weight_decay=0.0, clip_grad_norm=1.0, grad_accum_steps=len(rows))
     per_seq = []
     st = None
@@ -54,17 +53,17 @@ def run_step(model, factors, rows, targets, masks, micro):
 
 
 def test_full_size_batch_properties(world):
-    ctx, model, _, factors = world
+    ctx, model, _, factors, W = world
     rows, targets, masks = bench.synthetic_batch(W)
-    st_a, _, g_a = run_step(model, factors, rows, targets, masks, micro=8)
-    st_b, _, g_b = run_step(model, factors, rows, targets, masks, micro=8)
+    st_a, _, g_a = run_step(model, factors, W, rows, targets, masks, micro=8)
+    st_b, _, g_b = run_step(model, factors, W, rows, targets, masks, micro=8)
     assert np.isfinite(st_a.loss) and st_a.tokens == int(masks.sum())
     # determinism at the real shape: every reduction of the step has a fixed order
     assert (st_a.loss, st_a.grad_norm) == (st_b.loss, st_b.grad_norm)
     for k in g_a:
         assert np.array_equal(g_a[k].view(np.uint32), g_b[k].view(np.uint32)), k
     # eight one-sequence passes (split-K GEMMs, accumulated factor gradients) add up to the batched step
-    st_c, per_seq, g_c = run_step(model, factors, rows, targets, masks, micro=1)
+    st_c, per_seq, g_c = run_step(model, factors, W, rows, targets, masks, micro=1)
     assert_close("sum of the per-sequence losses", [sum(per_seq)], [st_a.loss])
     assert_close("grad norm", [st_c.grad_norm], [st_a.grad_norm])
     scale = max(float(np.abs(g).max()) for g in g_a.values())
@@ -74,13 +73,13 @@ def test_full_size_batch_properties(world):
 
 
 def test_one_full_size_sequence_matches_the_oracle(world):
-    ctx, model, tensors, factors = world
+    ctx, model, tensors, factors, W = world
     cfg = rs.ModelConfig(W["vocab"], W["hidden"], W["ffn"], W["layers"], W["heads"], W["kv"], 1e-5, 100000.0, True)
     orc = rs.Model.from_hf_tensors(cfg, tensors, f16_linears=True)
     for name, a, b in factors:
         orc.set_lora(name, a, b, W["alpha"])
     rows, targets, masks = bench.synthetic_batch(W, B=1)
-    st, _, grads = run_step(model, factors, rows, targets, masks, micro=1)
+    st, _, grads = run_step(model, factors, W, rows, targets, masks, micro=1)
     want_stats, _, want_grads = rs.train_chunk(orc, rs.AdamW(lr=2e-4, weight_decay=0.0), rows, targets, masks,
                                                grad_accum_steps=1, clip_grad_norm=1.0, return_grads=True)
     clip = np.float32(want_stats.clip_scale or 1.0)   # the oracle hands back the clipped gradients
