@@ -1,5 +1,6 @@
 """The step at BASELINE.json's full sizes: the headline (SmolLM2-360M shape, 8 x 256, vocabulary 49152)
-and the 135M shape (576 hidden: the GEMM shapes that split K).
+the 135M shape (576 hidden: the GEMM shapes that split K), and two layers of the 1.7B shape (2048 hidden,
+32 heads without grouping, rank 16 on all seven projections, block checkpointing, 4 x 512 tokens).
 
 The oracle finishes one 256-token sequence of this model in seconds, so one sequence is compared with
 it element by element (loss, gradient norm, every LoRA gradient); the full batch is checked through
@@ -15,15 +16,20 @@ from tests.gpu_util import assert_close
 
 pytestmark = pytest.mark.gpu
 
-@pytest.fixture(scope="module", params=["360m", "135m"])
+SHAPES = {"360m": bench.WORKLOADS["360m"], "135m": bench.WORKLOADS["135m"],
+          "1.7b-two-layers": dict(bench.WORKLOADS["1.7b"], layers=2, B=4, S=512, prompt=(64, 256))}
+
+
+@pytest.fixture(scope="module", params=list(SHAPES))
 def world(request):
     from ferrotensor_amd import HipContext
-    W = bench.WORKLOADS[request.param]
+    W = SHAPES[request.param]
     from ferrotensor_amd.trainer import Lfm2Model, ModelConfig
     ctx = HipContext(0)
     cfg = ModelConfig(vocab_size=W["vocab"], hidden_size=W["hidden"], intermediate_size=W["ffn"],
                       num_hidden_layers=W["layers"], num_attention_heads=W["heads"], num_key_value_heads=W["kv"],
-                      rms_norm_eps=1e-5, rope_theta=100000.0, tie_word_embeddings=True, f16_linears=True)
+                      rms_norm_eps=1e-5, rope_theta=100000.0, tie_word_embeddings=True, f16_linears=True,
+                      checkpoint_blocks=bool(W.get("checkpoint", False)))
     tensors = dict(bench.synthetic_tensors(W))
     model = Lfm2Model(ctx, cfg)
     model.load_tensors(tensors)
@@ -55,8 +61,8 @@ def run_step(model, factors, W, rows, targets, masks, micro):
 def test_full_size_batch_properties(world):
     ctx, model, _, factors, W = world
     rows, targets, masks = bench.synthetic_batch(W)
-    st_a, _, g_a = run_step(model, factors, W, rows, targets, masks, micro=8)
-    st_b, _, g_b = run_step(model, factors, W, rows, targets, masks, micro=8)
+    st_a, _, g_a = run_step(model, factors, W, rows, targets, masks, micro=len(rows))
+    st_b, _, g_b = run_step(model, factors, W, rows, targets, masks, micro=len(rows))
     assert np.isfinite(st_a.loss) and st_a.tokens == int(masks.sum())
     # determinism at the real shape: every reduction of the step has a fixed order
     assert (st_a.loss, st_a.grad_norm) == (st_b.loss, st_b.grad_norm)
