@@ -105,6 +105,9 @@ struct ft_model {
     LinearW lm_head;
     std::vector<ParamRef> params;
     bool params_dirty = true;
+    // Bumped whenever an adapter's buffers are (re)allocated: a trainer holds raw pointers into
+    // them and sizes its moments from them, so it is only valid for the generation it was made in.
+    uint64_t param_generation = 0;
 
     // Step buffers, valid for (ws_B, ws_S).
     size_t ws_B = 0, ws_S = 0;
@@ -137,6 +140,8 @@ struct ft_model {
 struct ft_trainer {
     ft_model* model = nullptr;
     ft_trainer_config cfg{};
+    uint64_t generation = 0;        // the model's param_generation this trainer was built for
+    std::vector<size_t> numel;      // elements of m[i] / v[i]
     float t = 0.0f;                 // AdamW step counter (f32, as in the reference)
     size_t optimizer_steps = 0;     // steps taken = position of the LR schedule
     size_t step_in_accum = 0;
@@ -820,6 +825,7 @@ int ft_model_set_lora(ft_model* m, const char* prefix, const float* a, const flo
             FT_TRY(ft_zero(m->ctx, l->gb, rank * l->out * 4));
             l->r = rank;
             m->params_dirty = true;
+            m->param_generation++;
         }
         l->alpha = alpha;
         FT_TRY(ft_upload(m->ctx, l->a, a, l->in * rank * sizeof(float)));
@@ -934,9 +940,11 @@ int ft_trainer_create(ft_model* m, const ft_trainer_config* cfg, ft_trainer** ou
         auto t = std::make_unique<ft_trainer>();
         t->model = m;
         t->cfg = *cfg;
+        t->generation = m->param_generation;
         ft_context* ctx = m->ctx;
         std::vector<ft_segment> segs;
         for (auto& p : m->params) {
+            t->numel.push_back(p.n);
             float *pm = nullptr, *pv = nullptr;
             FT_TRY(alloc_f(ctx, p.n, &pm));
             FT_TRY(alloc_f(ctx, p.n, &pv));
@@ -1099,18 +1107,27 @@ int ft_trainer_optimizer_steps(ft_trainer* t, size_t* steps) {
     return FT_OK;
 }
 
+// A trainer built before an adapter was added or changed rank points into buffers the model has
+// freed since: refuse to use it.
+#define FT_CHECK_TRAINER_CURRENT(t, what)                                                                     \
+    FT_CHECK_ARG((t)->generation == (t)->model->param_generation,                                            \
+                 what ": the model's adapters changed (a rank, or a new adapter) after this trainer was "     \
+                      "created; create a new trainer")
+
 int ft_trainer_read_moments(ft_trainer* t, size_t index, float* m_host, float* v_host) {
     FT_CHECK_ARG(t && m_host && v_host, "ft_trainer_read_moments: NULL argument");
+    FT_CHECK_TRAINER_CURRENT(t, "ft_trainer_read_moments");
     FT_CHECK_ARG(index < t->m.size(), "ft_trainer_read_moments: index %zu of %zu", index, t->m.size());
-    const size_t bytes = t->model->params[index].n * sizeof(float);
+    const size_t bytes = t->numel[index] * sizeof(float);
     FT_TRY(ft_download(t->model->ctx, m_host, t->m[index], bytes));
     return ft_download(t->model->ctx, v_host, t->v[index], bytes);
 }
 
 int ft_trainer_write_moments(ft_trainer* t, size_t index, const float* m_host, const float* v_host) {
     FT_CHECK_ARG(t && m_host && v_host, "ft_trainer_write_moments: NULL argument");
+    FT_CHECK_TRAINER_CURRENT(t, "ft_trainer_write_moments");
     FT_CHECK_ARG(index < t->m.size(), "ft_trainer_write_moments: index %zu of %zu", index, t->m.size());
-    const size_t bytes = t->model->params[index].n * sizeof(float);
+    const size_t bytes = t->numel[index] * sizeof(float);
     FT_TRY(ft_upload(t->model->ctx, t->m[index], m_host, bytes));
     return ft_upload(t->model->ctx, t->v[index], v_host, bytes);
 }
@@ -1144,6 +1161,7 @@ int ft_trainer_train_chunk(ft_trainer* t, const uint32_t* rows, const uint32_t* 
     return guarded([&]() -> int {
         FT_CHECK_ARG(t && rows && targets && loss_mask && stats, "ft_trainer_train_chunk: NULL argument");
         FT_CHECK_ARG(B > 0 && S > 0, "ft_trainer_train_chunk: empty chunk");
+        FT_CHECK_TRAINER_CURRENT(t, "ft_trainer_train_chunk");
         ft_model* m = t->model;
         ft_context* ctx = m->ctx;
         const size_t T = B * S, V = m->cfg.vocab_size;

@@ -90,6 +90,10 @@ class HipContext:
         check(self._lib.ft_pool_stats(self.handle, C.byref(live), C.byref(idle)))
         return live.value, idle.value
 
+    def pool_trim(self):
+        """Returns every idle pooled buffer to the device (`BufferPool::clear`, pool.rs)."""
+        check(self._lib.ft_pool_trim(self.handle))
+
     def close(self):
         if self.handle is not None and self.handle.value:
             for child in list(self._children):
@@ -438,6 +442,13 @@ class ComputeEngine:
     def rope_theta_inverse(self, ctx, t, head_dim, pos, theta):
         b, s, h = self._rope_dims(t)
         check(self._lib.ft_rope_theta_inverse(ctx.handle, _p(t), b, s, h, head_dim, pos, theta))
+
+    def rope_theta_to(self, ctx, src, dst, head_dim, pos, theta, inverse=False):
+        """Out-of-place `rope_theta` / `rope_theta_inverse`: dst = rotation of src, src untouched."""
+        b, s, h = self._rope_dims(src)
+        assert dst.numel() == src.numel()
+        check(self._lib.ft_rope_theta_to(ctx.handle, _p(src), _p(dst), b, s, h, head_dim, pos, theta,
+                                         1 if inverse else 0))
 
     # -- attention (engine/attention.rs:165-177, 341-358) --
     @staticmethod

@@ -473,6 +473,34 @@ def pad_chunk(seqs, length_bucket=32):
     return (np.array(rows, np.uint32), np.array(targets, np.uint32), np.array(masks, np.uint8))
 
 
+def apply_gradients(params, grads, opt: AdamW, stats: "StepStats", clip_grad_norm: Optional[float] = None,
+                    scheduler=None):
+    """`Trainer::apply_gradients` (trainer/src/lib.rs:296-360): global norm; a non-finite norm
+    skips the step (neither the optimizer's t nor the schedule advances, :332-335); when the norm
+    exceeds `clip_grad_norm` every gradient is scaled in place by max / (norm + 1e-6), all in f32
+    (:336-343, `clip_grad_by_norm`, engine/training.rs:161-169); then the schedule steps and AdamW
+    applies. `grads` (name -> array) is updated with the clipped gradients."""
+    glist = [grads[n] for n, _ in params if n in grads]
+    if not glist:
+        return
+    norm = global_grad_norm(glist)
+    stats.grad_norm = float(norm)
+    if not np.isfinite(norm):
+        return
+    if clip_grad_norm is not None and norm > np.float32(clip_grad_norm):
+        s = np.float32(clip_grad_norm) / (norm + np.float32(1e-6))
+        stats.clip_scale = float(s)
+        for n, _ in params:
+            if n in grads:
+                grads[n] = cpu.scale(grads[n], float(s))
+    if scheduler is not None:   # step k (1-based) uses the schedule's value at k (:345-352)
+        scheduler.step()
+        opt.lr = scheduler.get_lr()
+        stats.lr = opt.lr
+    opt.step(params, grads)
+    stats.optimizer_step = True
+
+
 def train_chunk(model: Model, opt: AdamW, rows, targets, masks, grad_accum_steps=None,
                 clip_grad_norm: Optional[float] = None, trainable_base=False, return_grads=False, scheduler=None):
     """One forward + backward over equally long rows and one optimizer step
@@ -492,22 +520,8 @@ def train_chunk(model: Model, opt: AdamW, rows, targets, masks, grad_accum_steps
         grad_logits = cpu.scale(grad_logits, float(seed))
     grads = model.backward(grad_logits, cache)
     params = model.lora_params()
-    glist = [grads[n] for n, _ in params if n in grads]
-    norm = global_grad_norm(glist)
-    stats = StepStats(float(loss), [(float(a), b) for a, b in per_seq], float(norm), False)
-    if np.isfinite(norm):
-        if clip_grad_norm is not None and norm > clip_grad_norm:
-            s = np.float32(clip_grad_norm) / (norm + np.float32(1e-6))
-            stats.clip_scale = float(s)
-            for n, _ in params:
-                if n in grads:
-                    grads[n] = cpu.scale(grads[n], float(s))
-        if scheduler is not None:   # apply_gradients, trainer/src/lib.rs:345-352: step k uses the value at k
-            scheduler.step()
-            opt.lr = scheduler.get_lr()
-            stats.lr = opt.lr
-        opt.step(params, grads)
-        stats.optimizer_step = True
+    stats = StepStats(float(loss), [(float(a), b) for a, b in per_seq], None, False)
+    apply_gradients(params, grads, opt, stats, clip_grad_norm=clip_grad_norm, scheduler=scheduler)
     if return_grads:
         return stats, logits, grads
     return stats

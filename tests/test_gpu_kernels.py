@@ -338,6 +338,95 @@ def test_elementwise(g, n):
     np.testing.assert_array_equal(t.to_numpy(), a * np.float32(0.37) + b)
 
 
+@pytest.mark.parametrize("n", [1, 7, 4096 + 3, 1 << 20])
+def test_clip_grad_by_norm_scales_in_place(g, n):
+    """`clip_grad_by_norm` (engine/training.rs:161-169, WGSL grad_clip): x *= scale, one f32 product per
+    element, so bit-exact against numpy; together with `sum_squares_partial` it is the reference's clip."""
+    from ferrotensor_amd import UnifiedTensor
+    ctx, eng = g
+    x = rnd(n, n, scale=3.0)
+    parts = UnifiedTensor.zeros(ctx, [(n + 4095) // 4096])
+    t = up(ctx, x)
+    assert eng.sum_squares_partial(ctx, t, parts, 0) == (n + 4095) // 4096
+    norm = np.float32(np.sqrt(parts.to_numpy().astype(np.float64).sum()))
+    assert abs(float(norm) - float(rs.global_grad_norm([x]))) <= 1e-5 * float(norm)
+    scale = np.float32(1.0) / (norm + np.float32(1e-6))
+    eng.clip_grad_by_norm(ctx, t, float(scale))
+    np.testing.assert_array_equal(t.to_numpy(), cpu.scale(x, float(scale)))
+    np.testing.assert_array_equal(t.to_numpy(), x * scale)
+
+
+def test_copy_tensor_with_a_destination_offset(g):
+    """`copy_tensor(src, dst, dst_byte_offset)` (engine/mod.rs:399-415): device to device, bytes outside the
+    written range untouched; f16 buffers copy as raw bytes."""
+    from ferrotensor_amd import FtError, UnifiedTensor
+    ctx, eng = g
+    base, src = rnd(1, 1000), rnd(2, 300)
+    dst = up(ctx, base)
+    eng.copy_tensor(ctx, up(ctx, src), dst, dst_byte_offset=4 * 123)
+    want = base.copy()
+    want[123:423] = src
+    np.testing.assert_array_equal(dst.to_numpy(), want)
+    eng.copy_tensor(ctx, up(ctx, src), dst)
+    want[:300] = src
+    np.testing.assert_array_equal(dst.to_numpy(), want)
+    h = UnifiedTensor.from_f32_as_f16(ctx, src, [300])
+    d16 = UnifiedTensor.from_f32_as_f16(ctx, base, [1000])
+    eng.copy_tensor(ctx, h, d16, dst_byte_offset=2 * 400)
+    want16 = cpu.pack_f16(base)
+    want16[400:700] = cpu.pack_f16(src)
+    np.testing.assert_array_equal(d16.to_vec(ctx, np.uint16), want16)
+
+
+@pytest.mark.parametrize("B,S,heads,D,pos,theta", [(2, 9, 3, 8, 5, 10000.0), (2, 64, 5, 64, 0, 100000.0),
+                                                  (1, 33, 2, 6, 960, 500.0)])
+def test_rope_theta_out_of_place(g, B, S, heads, D, pos, theta):
+    """`ft_rope_theta_to`: the rotation written to a second buffer (what `Tensor::rope_theta` and
+    `RoPENode::backward` get by copying first, autograd/src/lib.rs:509-533, 1122-1139); the source keeps its bits
+    and both directions equal the in-place kernels bit for bit."""
+    ctx, eng = g
+    x = rnd(12, B, S, heads * D)
+    src, dst = up(ctx, x), empty(ctx, B, S, heads * D)
+    eng.rope_theta_to(ctx, src, dst, D, pos, theta)
+    np.testing.assert_array_equal(src.to_numpy(), x)
+    assert_close("rope_to", dst.to_numpy(), cpu.rope(x, D, pos, theta))
+    inplace = up(ctx, x)
+    eng.rope_theta(ctx, inplace, D, pos, theta)
+    np.testing.assert_array_equal(dst.to_numpy(), inplace.to_numpy())
+    back = empty(ctx, B, S, heads * D)
+    eng.rope_theta_to(ctx, dst, back, D, pos, theta, inverse=True)
+    assert_close("rope_to inverse", back.to_numpy(), x)
+    assert_close("rope_to inverse vs oracle", back.to_numpy(), cpu.rope(dst.to_numpy(), D, pos, theta, inverse=True))
+    eng.rope_theta_inverse(ctx, inplace, D, pos, theta)
+    np.testing.assert_array_equal(back.to_numpy(), inplace.to_numpy())
+
+
+def test_pool_reuses_exact_sizes_and_trims(g):
+    """The buffer pool (`pool.rs`): a freed buffer serves the next request of exactly its size; `ft_pool_trim`
+    hands the idle ones back to the device."""
+    ctx, _ = g
+    ctx.synchronize()
+    ctx.pool_trim()
+    live0, idle0 = ctx.pool_stats()
+    assert idle0 == 0
+    n, n2 = 12800, 12864                 # 51200 and 51456 bytes: two size classes (256-byte granularity)
+    a = empty(ctx, n)
+    ptr = a.ptr
+    live1, _ = ctx.pool_stats()
+    assert live1 == live0 + n * 4
+    del a
+    live2, idle2 = ctx.pool_stats()
+    assert live2 == live0 and idle2 == n * 4
+    b = empty(ctx, n)
+    assert b.ptr == ptr and ctx.pool_stats()[1] == 0
+    c = empty(ctx, n2)
+    assert c.ptr != ptr
+    del b, c
+    assert ctx.pool_stats()[1] == n * 4 + n2 * 4
+    ctx.pool_trim()
+    assert ctx.pool_stats() == (live0, 0)
+
+
 def test_embedding_gather_bit_exact(g):
     from ferrotensor_amd import UnifiedTensor
     ctx, eng = g

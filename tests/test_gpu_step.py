@@ -272,6 +272,210 @@ def test_tiny_llama_full_step_matches_oracle(ctx, f16, tied):
             assert_close(f"step {step} weight {n}", params[n], w, atol=1e-6, rtol=1e-4)
 
 
+def _moments(tr):
+    """{param name: (m, v)} of the trainer's AdamW state, keyed like `Lfm2Model.params()`."""
+    import ctypes as C
+    out = {}
+    for i, (name, numel) in enumerate(tr.model.named_params()):
+        m, v = np.empty(numel, np.float32), np.empty(numel, np.float32)
+        from ferrotensor_amd._lib import check
+        check(tr._lib.ft_trainer_read_moments(tr.handle, i, m.ctypes.data_as(C.c_void_p),
+                                              v.ctypes.data_as(C.c_void_p)))
+        out[name] = (m, v)
+    return out
+
+
+def _adam_t(tr):
+    import ctypes as C
+    t = C.c_float()
+    tr._lib.ft_trainer_get_adam_t(tr.handle, C.byref(t))
+    return t.value
+
+
+def _clip_case(ctx, seed=11):
+    cfg = tiny_config(True, True)
+    mods = ["q_proj", "k_proj", "v_proj", "o_proj", "gate_proj", "up_proj", "down_proj"]
+    hip, orc = build_pair(ctx, cfg, mods, rank=4, alpha=8.0, seed=seed)
+    rng = np.random.default_rng(5)
+    B, S = 2, 16
+    rows = rng.integers(0, 256, (B, S)).astype(np.uint32)
+    targets = np.concatenate([rows[:, 1:], rng.integers(0, 256, (B, 1)).astype(np.uint32)], axis=1)
+    masks = np.ones((B, S), np.uint8)
+    masks[:, :4] = 0
+    return hip, orc, rows, targets, masks, rng
+
+
+def test_gradient_clip_fires_against_oracle(ctx):
+    """`apply_gradients` with the clip active (trainer/src/lib.rs:336-343): the tiny config's gradient norm is
+    0.07-0.08, so a clip at 0.01 scales every gradient in every step. Norm, clip scale, the updated weights
+    and both AdamW moments against the oracle over three steps."""
+    from ferrotensor_amd.trainer import Trainer
+    hip, orc, rows, targets, masks, _ = _clip_case(ctx)
+    tr = Trainer(hip, lr=1e-3, weight_decay=0.01, clip_grad_norm=0.01)
+    opt = rs.AdamW(lr=1e-3, weight_decay=0.01)
+    for step in range(3):
+        want = rs.train_chunk(orc, opt, rows, targets, masks, clip_grad_norm=0.01)
+        st = tr.train_chunk(rows, targets, masks)
+        assert st.optimizer_step and want.optimizer_step
+        assert want.clip_scale is not None and want.clip_scale < 0.5, want
+        assert_close("loss", [st.loss], [want.loss])
+        assert_close("grad_norm", [st.grad_norm], [want.grad_norm])
+        assert_close("clip_scale", [st.clip_scale], [want.clip_scale], atol=1e-7, rtol=1e-3)
+        params, mom = hip.params(), _moments(tr)
+        for n, w in orc.lora_params():
+            assert_close(f"step {step} weight {n}", params[n], w, atol=1e-6, rtol=1e-4)
+            # the moments of clipped gradients are tiny (m ~1e-5, v ~1e-11): bars relative to their scale
+            m_bar, v_bar = 1e-3 * np.abs(opt.m[n]).max(), 2e-3 * np.abs(opt.v[n]).max()
+            assert_close(f"step {step} m {n}", mom[n][0], opt.m[n], atol=m_bar, rtol=1e-3)
+            assert_close(f"step {step} v {n}", mom[n][1], opt.v[n], atol=v_bar, rtol=2e-3)
+        assert _adam_t(tr) == opt.t == step + 1
+
+
+def test_gradient_clip_over_an_accumulation_window(ctx):
+    """A window of 4 sequences fed as two chunks of 2 (seed 1/4 each): the norm and the clip see the summed
+    gradients, once, when the window closes."""
+    from ferrotensor_amd.trainer import Trainer
+    hip, orc, rows, targets, masks, rng = _clip_case(ctx, seed=13)
+    B = rows.shape[0]
+    tr = Trainer(hip, lr=1e-3, weight_decay=0.0, clip_grad_norm=0.03, grad_accum_steps=4)
+    opt = rs.AdamW(lr=1e-3, weight_decay=0.0)
+    rows2 = rng.integers(0, 256, rows.shape).astype(np.uint32)
+    targets2 = np.concatenate([rows2[:, 1:], rows2[:, :1]], axis=1)
+    first = tr.train_chunk(rows, targets, masks)
+    assert not first.optimizer_step and first.clip_scale == 1.0
+    st = tr.train_chunk(rows2, targets2, masks)
+    assert st.optimizer_step
+    params_o = orc.lora_params()
+    total = {}
+    for r_, t_ in ((rows, targets), (rows2, targets2)):
+        logits, cache = orc.forward(r_)
+        _, _, gl = rs.masked_cross_entropy_batch(logits, t_, masks, B)
+        for n, gval in orc.backward(rs.cpu.scale(gl, 0.25), cache).items():
+            total[n] = gval if n not in total else rs.cpu.add(total[n], gval)
+    stats = rs.StepStats(0.0, [], None, False)
+    rs.apply_gradients(params_o, total, opt, stats, clip_grad_norm=0.03)
+    assert stats.clip_scale is not None and stats.clip_scale < 0.95, stats
+    assert_close("grad_norm", [st.grad_norm], [stats.grad_norm])
+    assert_close("clip_scale", [st.clip_scale], [stats.clip_scale], atol=1e-7, rtol=1e-3)
+    params = hip.params()
+    for n, w in params_o:
+        assert_close(f"weight {n}", params[n], w, atol=1e-6, rtol=1e-4)
+
+
+def test_fixture_model_step_with_the_clip_at_one(ctx, fx):
+    """The reference fixture's model has a gradient norm of about 4.4 on its `batch` case: with the CLI's
+    `clip_grad_norm = 1.0` the clip scale is about 0.22. Two optimizer steps against the oracle."""
+    from ferrotensor_amd.trainer import Trainer
+    rows, targets, masks, _, _ = fx.case("batch")
+    model = hip_model_from_fixture(ctx, fx)
+    orc = fx.oracle_model()
+    tr = Trainer(model, lr=1e-2, weight_decay=0.0, clip_grad_norm=1.0)
+    opt = rs.AdamW(lr=1e-2, weight_decay=0.0)
+    for step in range(2):
+        want = rs.train_chunk(orc, opt, rows, targets, masks, clip_grad_norm=1.0)
+        st = tr.train_chunk(rows, targets, masks)
+        assert want.clip_scale is not None and want.grad_norm > 1.0
+        assert_close("loss", [st.loss], [want.loss])
+        assert_close("grad_norm", [st.grad_norm], [want.grad_norm])
+        assert_close("clip_scale", [st.clip_scale], [want.clip_scale], atol=1e-7, rtol=1e-3)
+        params = model.params()
+        for n, w in orc.lora_params():
+            assert_close(f"step {step} weight {n}", params[n], w, atol=1e-6, rtol=1e-4)
+
+
+@pytest.mark.parametrize("bad", [np.nan, np.inf])
+def test_non_finite_gradient_norm_skips_the_step(ctx, bad):
+    """trainer/src/lib.rs:330-335: a NaN / Inf gradient norm skips the optimizer step. Weights, moments, AdamW's
+    t, the step counter and the LR schedule stay where they were, the window is closed (zero_grad), and the
+    next clean window overwrites the poisoned gradients and steps as if nothing had happened."""
+    from ferrotensor_amd.trainer import Trainer
+    cfg = tiny_config(True, True)
+    mods = ["q_proj", "k_proj", "v_proj", "o_proj"]
+    hip, orc = build_pair(ctx, cfg, mods, rank=4, alpha=8.0, seed=29)
+    rng = np.random.default_rng(15)
+    rows = rng.integers(0, 256, (2, 16)).astype(np.uint32)
+    targets = np.concatenate([rows[:, 1:], rows[:, :1]], axis=1)
+    masks = np.ones((2, 16), np.uint8)
+    kw = dict(lr=2e-3, weight_decay=0.01, clip_grad_norm=1.0, lr_schedule="warmup_cosine", warmup_steps=2,
+              total_steps=6, min_lr=2e-4)
+    tr = Trainer(hip, **kw)
+    opt = rs.AdamW(lr=2e-3, weight_decay=0.01)
+    sched = rs.WarmupCosineScheduler(2e-3, 2e-4, 2, 6)
+    want = rs.train_chunk(orc, opt, rows, targets, masks, clip_grad_norm=1.0, scheduler=sched)
+    st = tr.train_chunk(rows, targets, masks)
+    assert st.optimizer_step and tr.optimizer_steps == 1 and _adam_t(tr) == 1.0
+
+    # poison one element of one B factor (both models)
+    name = "model.layers.1.self_attn.v_proj"
+    clean = hip.params()
+    a = clean[name + ".lora_a"].reshape(cfg.hidden_size, 4)
+    b = clean[name + ".lora_b"].reshape(4, -1).copy()
+    b_bad = b.copy()
+    b_bad[2, 5] = bad
+    hip.set_lora(name, a, b_bad, 8.0)
+    before, mom_before = hip.params(), _moments(tr)
+    skipped = tr.train_chunk(rows, targets, masks)
+    assert not skipped.optimizer_step and skipped.lr is None
+    assert not np.isfinite(skipped.grad_norm)
+    assert tr.optimizer_steps == 1 and _adam_t(tr) == 1.0 and tr.step_in_accum == 0
+    after, mom_after = hip.params(), _moments(tr)
+    for n in before:
+        assert np.array_equal(before[n].view(np.uint32), after[n].view(np.uint32)), n
+        assert np.array_equal(mom_before[n][0], mom_after[n][0]) and np.array_equal(mom_before[n][1], mom_after[n][1]), n
+    # the oracle follows the same rule on the same poisoned factor
+    orc_lin = dict(orc.named_linears())[name]
+    orc_b_clean = orc_lin.lora_b.copy()
+    orc_lin.lora_b[2, 5] = bad
+    want_skip = rs.train_chunk(orc, opt, rows, targets, masks, clip_grad_norm=1.0, scheduler=sched)
+    assert not want_skip.optimizer_step and opt.t == 1.0 and sched.current == 1
+    orc_lin.lora_b[...] = orc_b_clean
+
+    # repaired: the next window steps with t = 2 and the schedule's second value
+    hip.set_lora(name, a, b, 8.0)
+    want2 = rs.train_chunk(orc, opt, rows, targets, masks, clip_grad_norm=1.0, scheduler=sched)
+    st2 = tr.train_chunk(rows, targets, masks)
+    assert st2.optimizer_step and tr.optimizer_steps == 2 and _adam_t(tr) == 2.0
+    assert abs(st2.lr - want2.lr) <= 2e-7 * 2e-3
+    assert_close("loss", [st2.loss], [want2.loss])
+    assert_close("grad_norm", [st2.grad_norm], [want2.grad_norm])
+    params = hip.params()
+    for n, w in orc.lora_params():
+        assert_close(f"weight {n}", params[n], w, atol=1e-6, rtol=1e-4)
+
+
+def test_a_trainer_is_refused_after_the_adapters_change(ctx):
+    """A trainer sizes its moments from, and points into, the adapters it was created over. Changing a rank or
+    adding an adapter afterwards reallocates them: the old trainer must report an error, not run through
+    freed buffers; a new trainer works, and re-setting an adapter at the same rank keeps the old one valid."""
+    from ferrotensor_amd import FtError
+    from ferrotensor_amd.trainer import Trainer
+    cfg = tiny_config()
+    hip, _ = build_pair(ctx, cfg, ["q_proj", "v_proj"], rank=4, alpha=8.0, seed=33)
+    rng = np.random.default_rng(1)
+    rows = rng.integers(0, 256, (2, 16)).astype(np.uint32)
+    targets = np.concatenate([rows[:, 1:], rows[:, :1]], axis=1)
+    masks = np.ones((2, 16), np.uint8)
+    tr = Trainer(hip, lr=1e-3)
+    assert tr.train_chunk(rows, targets, masks).optimizer_step
+    name = "model.layers.0.self_attn.q_proj"
+    i, o = hip.linear_dims(name)
+    same = hip.params()
+    hip.set_lora(name, same[name + ".lora_a"].reshape(i, 4), same[name + ".lora_b"].reshape(4, o), 8.0)
+    assert tr.train_chunk(rows, targets, masks).optimizer_step          # same rank: nothing was reallocated
+    hip.set_lora(name, np.zeros((i, 8), np.float32), np.zeros((8, o), np.float32), 16.0)
+    with pytest.raises(FtError, match="create a new trainer"):
+        tr.train_chunk(rows, targets, masks)
+    with pytest.raises(FtError, match="create a new trainer"):
+        _moments(tr)
+    assert tr.optimizer_steps == 2
+    tr2 = Trainer(hip, lr=1e-3)
+    assert tr2.train_chunk(rows, targets, masks).optimizer_step
+    hip.add_lora("model.layers.1.mlp.down_proj", 4, 8.0)                  # a new adapter: same rule
+    with pytest.raises(FtError, match="create a new trainer"):
+        tr2.train_chunk(rows, targets, masks)
+    assert Trainer(hip, lr=1e-3).train_chunk(rows, targets, masks).optimizer_step
+
+
 def test_warmup_cosine_schedule_drives_the_step(ctx):
     """Optimizer step k uses the schedule's value at k (trainer/src/lib.rs:345-352); a resumed
     trainer continues the curve where the counter says."""

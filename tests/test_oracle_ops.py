@@ -234,6 +234,66 @@ def test_adamw_against_torch_optim(wd):
         np.testing.assert_allclose(w, wt.detach().numpy(), rtol=1e-5, atol=1e-6)
 
 
+@pytest.mark.parametrize("max_norm,wd", [(0.5, 0.0), (1.0, 0.01), (1e9, 0.0)])
+def test_apply_gradients_clips_like_torch_clip_grad_norm(max_norm, wd):
+    """The clip of `apply_gradients` (max / (norm + 1e-6) when norm > max, trainer/src/lib.rs:336-343) is
+    the rule of `torch.nn.utils.clip_grad_norm_`; followed by AdamW it must track torch over several
+    steps, with tensors that span more than one 4096-element partial-sum chunk."""
+    shapes = [(5000,), (33, 7), (4096,), (3,)]
+    names = [f"p{i}" for i in range(len(shapes))]
+    w = {n: randn(*s) for n, s in zip(names, shapes)}
+    tw = [torch.nn.Parameter(torch.tensor(w[n], dtype=torch.float64)) for n in names]
+    topt = torch.optim.AdamW(tw, lr=1e-2, betas=(0.9, 0.999), eps=1e-8, weight_decay=wd)
+    opt = rs.AdamW(lr=1e-2, weight_decay=wd)
+    params = [(n, w[n]) for n in names]
+    for step in range(4):
+        grads = {n: randn(*s) * np.float32(0.02 * (step + 1)) for n, s in zip(names, shapes)}
+        for p, n in zip(tw, names):
+            p.grad = torch.tensor(grads[n], dtype=torch.float64)
+        total = float(torch.nn.utils.clip_grad_norm_(tw, max_norm))
+        topt.step()
+        stats = rs.StepStats(0.0, [], None, False)
+        rs.apply_gradients(params, grads, opt, stats, clip_grad_norm=max_norm)
+        assert stats.optimizer_step and opt.t == step + 1
+        assert abs(stats.grad_norm - total) <= 1e-5 * total
+        if total > max_norm:
+            assert abs(stats.clip_scale - max_norm / (total + 1e-6)) <= 1e-6 * stats.clip_scale
+            for p, n in zip(tw, names):      # the gradients are clipped in place
+                np.testing.assert_allclose(grads[n], p.grad.numpy(), rtol=1e-5, atol=1e-9)
+        else:
+            assert stats.clip_scale is None
+        for p, n in zip(tw, names):
+            np.testing.assert_allclose(w[n], p.detach().numpy(), rtol=2e-5, atol=2e-6)
+
+
+@pytest.mark.parametrize("bad", [np.nan, np.inf])
+def test_apply_gradients_skips_a_non_finite_norm(bad):
+    """trainer/src/lib.rs:330-335: a NaN / Inf norm returns before the clip, the schedule and the
+    optimizer: weights, moments, t and the schedule stay where they were; the next clean call steps."""
+    w = {"a": randn(300), "b": randn(17, 5)}
+    params = list(w.items())
+    opt = rs.AdamW(lr=1e-2, weight_decay=0.0)
+    sched = rs.WarmupCosineScheduler(1e-2, 1e-3, 2, 6)
+    stats = rs.StepStats(0.0, [], None, False)
+    rs.apply_gradients(params, {n: randn(*v.shape) for n, v in w.items()}, opt, stats, 1.0, sched)
+    assert stats.optimizer_step and opt.t == 1.0 and sched.current == 1
+    before = ({n: v.copy() for n, v in w.items()}, {n: v.copy() for n, v in opt.m.items()},
+              {n: v.copy() for n, v in opt.v.items()}, opt.lr)
+    grads = {n: randn(*v.shape) for n, v in w.items()}
+    grads["b"][3, 2] = bad
+    stats = rs.StepStats(0.0, [], None, False)
+    rs.apply_gradients(params, grads, opt, stats, 1.0, sched)
+    assert not stats.optimizer_step and not np.isfinite(stats.grad_norm) and stats.clip_scale is None
+    assert opt.t == 1.0 and sched.current == 1 and opt.lr == before[3] and stats.lr is None
+    for n in w:
+        np.testing.assert_array_equal(w[n], before[0][n])
+        np.testing.assert_array_equal(opt.m[n], before[1][n])
+        np.testing.assert_array_equal(opt.v[n], before[2][n])
+    stats = rs.StepStats(0.0, [], None, False)
+    rs.apply_gradients(params, {n: randn(*v.shape) for n, v in w.items()}, opt, stats, 1.0, sched)
+    assert stats.optimizer_step and opt.t == 2.0 and sched.current == 2
+
+
 def test_embedding_out_of_range_row_is_zero():
     table = randn(5, 3)
     out = cpu.embedding(table, np.array([[0, 4, 5, 1000]], np.uint32))
