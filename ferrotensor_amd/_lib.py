@@ -104,6 +104,7 @@ SIGNATURES = {
     "ft_lora_grad_a": [_P, _P, _P, _P, _SZ, _SZ, _SZ],
     "ft_rms_norm_eps": [_P, _P, _P, _P, _SZ, _SZ, _F],
     "ft_rms_norm_backward": [_P, _P, _P, _P, _P, _P, _SZ, _SZ, _F],
+    "ft_rms_norm_backward_noalloc": [_P, _P, _P, _P, _P, _P, _SZ, _SZ, _F],
     "ft_rope_theta": [_P, _P, _SZ, _SZ, _SZ, _SZ, _SZ, _F],
     "ft_rope_theta_inverse": [_P, _P, _SZ, _SZ, _SZ, _SZ, _SZ, _F],
     "ft_rope_theta_to": [_P, _P, _P, _SZ, _SZ, _SZ, _SZ, _SZ, _F, _I],

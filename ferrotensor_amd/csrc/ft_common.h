@@ -75,6 +75,10 @@ struct ft_prof_scope {
 
 int ft_set_error(int code, const char* fmt, ...);
 
+// Looks up, once per device, the device address of the fixed scratch array behind
+// ft_rms_norm_backward_noalloc (ft_rowops.hip). `device` must be the current device.
+int ft_internal_noalloc_init(int device);
+
 int ft_side_begin(ft_context* ctx, int lane = 0);
 int ft_side_end(ft_context* ctx);
 int ft_side_join(ft_context* ctx, int lane = -1);  // -1: every lane

@@ -5,6 +5,8 @@
 // wave reductions), so HBM traffic equals the algorithmic byte count.
 #include "ft_common.h"
 
+#include <mutex>
+
 namespace {
 
 constexpr int kWave = 64;
@@ -916,6 +918,38 @@ int ft_internal_multi_adamw(ft_context* ctx, const ft_segment* segs_dev, size_t 
     return FT_OK;
 }
 
+// ---------------------------------------------------------------------------
+// ft_rms_norm_backward_noalloc: the same two kernels as the norm-weight-gradient path of
+// ft_rms_norm_backward, with the partial rows (one per workgroup) in a fixed device array
+// instead of a pooled allocation, for callers that cannot allocate (HIP graph capture, tight
+// serving loops). Every device the library runs on holds its own copy of the array (2 MiB) at
+// its own address until the process ends; the array's name is only a host-side handle, the
+// address kernels take comes from hipGetSymbolAddress, looked up once per device.
+// ---------------------------------------------------------------------------
+namespace {
+constexpr int kNoAllocMaxParts = 256;    // partial rows = workgroups of the first kernel
+constexpr int kNoAllocMaxSize = 2048;    // floats per row the wave kernels hold in registers
+constexpr int kNoAllocMaxDevices = 64;
+}  // namespace
+
+static __device__ __align__(256) float scratch[kNoAllocMaxParts * kNoAllocMaxSize];
+
+static float* g_noalloc_scratch[kNoAllocMaxDevices] = {};
+static std::mutex g_noalloc_mutex;
+
+// Device address of `scratch` on `device`, which must be the current device.
+int ft_internal_noalloc_init(int device) {
+    FT_CHECK_ARG(device >= 0 && device < kNoAllocMaxDevices, "no-alloc scratch: device %d is outside 0..%d", device,
+                 kNoAllocMaxDevices - 1);
+    std::lock_guard<std::mutex> lock(g_noalloc_mutex);
+    if (g_noalloc_scratch[device]) return FT_OK;
+    float* ptr = nullptr;
+    FT_HIP(hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch)));
+    FT_CHECK_ARG(ptr != nullptr, "no-alloc scratch: hipGetSymbolAddress returned NULL on device %d", device);
+    g_noalloc_scratch[device] = ptr;
+    return FT_OK;
+}
+
 extern "C" {
 
 int ft_zero(ft_context* ctx, void* dev, size_t bytes) {
@@ -1062,6 +1096,45 @@ int ft_rms_norm_backward(ft_context* ctx, const float* x, const float* w, const 
         FT_LAUNCH_CHECK();
         FT_TRY(ft_free(ctx, partial));
     }
+    return FT_OK;
+}
+
+int ft_rms_norm_backward_noalloc(ft_context* ctx, const float* x, const float* w, const float* g, float* gx,
+                                 float* gw, size_t rows, size_t size, float eps) {
+    FT_CHECK_ARG(ctx && x && w && g && gx && gw, "ft_rms_norm_backward_noalloc: NULL argument");
+    FT_CHECK_ARG(size > 0 && size % 4 == 0 && size <= (size_t)kNoAllocMaxSize,
+                 "ft_rms_norm_backward_noalloc: size %zu must be a multiple of 4 and at most %d", size,
+                 kNoAllocMaxSize);
+    FT_CHECK_ARG(rows > 0 && rows < (1u << 30), "ft_rms_norm_backward_noalloc: rows %zu is outside 1..2^30-1", rows);
+    FT_CHECK_ARG(aligned16(x) && aligned16(w) && aligned16(g) && aligned16(gx),
+                 "ft_rms_norm_backward_noalloc: x, w, g and gx must be 16-byte aligned");
+    FT_CHECK_ARG(ctx->device >= 0 && ctx->device < kNoAllocMaxDevices, "ft_rms_norm_backward_noalloc: device %d",
+                 ctx->device);
+    float* partial = g_noalloc_scratch[ctx->device];
+    if (!partial) {
+        // A context normally looks the address up when it is created; this is the first call on a
+        // device whose contexts were made before the library knew the device.
+        FT_HIP(hipSetDevice(ctx->device));
+        FT_TRY(ft_internal_noalloc_init(ctx->device));
+        partial = g_noalloc_scratch[ctx->device];
+    }
+    // Same launch shape as ft_rms_norm_backward: one partial row per workgroup, every row of the
+    // array that the second kernel reads is written in full by the first (nothing to clear).
+    size_t wgs = (rows + 3) / 4;
+    size_t cap = (size_t)ctx->num_cus;
+    if (cap > (size_t)kNoAllocMaxParts) cap = kNoAllocMaxParts;
+    if (wgs > cap) wgs = cap;
+    const size_t lds = 3 * size * sizeof(float);
+    if (size <= 1024)
+        hipLaunchKernelGGL((rms_norm_backward_gw_wave_kernel<4>), dim3((unsigned)wgs), dim3(256), lds, ctx->stream, x, w,
+                           g, gx, partial, (int)rows, (int)size, eps);
+    else
+        hipLaunchKernelGGL((rms_norm_backward_gw_wave_kernel<8>), dim3((unsigned)wgs), dim3(256), lds, ctx->stream, x, w,
+                           g, gx, partial, (int)rows, (int)size, eps);
+    FT_LAUNCH_CHECK();
+    hipLaunchKernelGGL(column_sum_sliced_kernel, dim3(ft_div_up(size, 16)), dim3(256), 0, ctx->stream, partial, gw,
+                       (int)wgs, (int)size);
+    FT_LAUNCH_CHECK();
     return FT_OK;
 }
 

@@ -149,6 +149,9 @@ static int context_create(int device, void* stream, bool own, ft_context** out) 
     if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
         return ft_set_error(FT_ERR_INVALID, "ft_context_create: kernels are built for gfx950, device is %s",
                             prop.gcnArchName);
+    // Set-up that must not happen later, when a caller may be unable to allocate or load code:
+    // the device address of the fixed scratch array of ft_rms_norm_backward_noalloc.
+    FT_TRY(ft_internal_noalloc_init(device));
     ft_context* ctx = new ft_context();
     ctx->device = device;
     ctx->num_cus = prop.multiProcessorCount;

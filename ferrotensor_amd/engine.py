@@ -424,6 +424,14 @@ class ComputeEngine:
         check(self._lib.ft_rms_norm_backward(ctx.handle, _p(x), _p(w), _p(g), _p(gx), _p(gw),
                                              x.numel() // size, size, eps))
 
+    def rms_norm_backward_noalloc(self, ctx, x, w, g, gx, gw, eps):
+        """`rms_norm_backward` for callers that cannot allocate: partial sums in the library's fixed
+        device array (size <= 2048, a multiple of 4; gw required)."""
+        size = x.shape[-1]
+        assert g.numel() == x.numel() and gx.numel() == x.numel() and gw is not None and gw.numel() == size
+        check(self._lib.ft_rms_norm_backward_noalloc(ctx.handle, _p(x), _p(w), _p(g), _p(gx), _p(gw),
+                                                     x.numel() // size, size, eps))
+
     # -- rope (engine/attention.rs:15-83) --
     @staticmethod
     def _rope_dims(t):

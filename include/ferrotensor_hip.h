@@ -241,6 +241,17 @@ int ft_rms_norm_eps(ft_context* ctx, const float* x, const float* w, float* out,
  * NULL when the norm scale is frozen and nobody reads it. */
 int ft_rms_norm_backward(ft_context* ctx, const float* x, const float* w, const float* g, float* gx,
                          float* gw, size_t rows, size_t size, float eps);
+/* No counterpart in the reference. ft_rms_norm_backward with the norm-weight gradient keeps one
+ * partial row per workgroup in a buffer it takes from the context's pool, which may call
+ * hipMalloc. This variant is for callers that cannot allocate (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid it): same kernels, same results, but the partial
+ * rows live in a fixed device array of the library (2 MiB per GPU, held until the process ends)
+ * and the call makes no allocation of any kind. Limits, reported as FT_ERR_INVALID: gw must not
+ * be NULL, rows >= 1, size a multiple of 4 and <= 2048, x / w / g / gx 16-byte aligned. Every
+ * call on a GPU shares that GPU's array: calls that overlap on one GPU (two streams, two
+ * threads) race; calls on one stream are ordered and safe. */
+int ft_rms_norm_backward_noalloc(ft_context* ctx, const float* x, const float* w, const float* g,
+                                 float* gx, float* gw, size_t rows, size_t size, float eps);
 
 /* ---- RoPE (engine/attention.rs:21-83) ------------------------------------ */
 
