@@ -316,20 +316,29 @@ int ft_upload_f32_transposed(ft_context* ctx, void* dst_dev, const float* src_ho
     FT_CHECK_ARG(dtype == FT_DTYPE_F32 || dtype == FT_DTYPE_F16,
                  "ft_upload_f32_transposed: dtype %d is not supported", dtype);
     const size_t n = rows * cols;
+    // Transposed in 32 x 32 blocks so that both the strided side and the contiguous side stay in cache.
+    constexpr size_t kBlock = 32;
+    auto for_each_block = [&](auto&& put) {
+        for (size_t r0 = 0; r0 < rows; r0 += kBlock)
+            for (size_t c0 = 0; c0 < cols; c0 += kBlock) {
+                const size_t r1 = r0 + kBlock < rows ? r0 + kBlock : rows;
+                const size_t c1 = c0 + kBlock < cols ? c0 + kBlock : cols;
+                for (size_t c = c0; c < c1; c++)
+                    for (size_t r = r0; r < r1; r++) put(c * rows + r, src_host[r * cols + c]);
+            }
+    };
     if (dtype == FT_DTYPE_F32) {
         std::vector<float> t(n);
-        for (size_t c = 0; c < cols; c++)
-            for (size_t r = 0; r < rows; r++) t[c * rows + r] = src_host[r * cols + c];
+        for_each_block([&](size_t at, float v) { t[at] = v; });
         return ft_upload(ctx, dst_dev, t.data(), n * 4);
     }
     size_t bytes = ((n * 2 + 3) / 4) * 4;
     if (bytes < 4) bytes = 4;
     std::vector<uint16_t> t(bytes / 2, 0);
-    for (size_t c = 0; c < cols; c++)
-        for (size_t r = 0; r < rows; r++) {
-            const _Float16 h = (_Float16)src_host[r * cols + c];
-            std::memcpy(&t[c * rows + r], &h, 2);
-        }
+    for_each_block([&](size_t at, float v) {
+        const _Float16 h = (_Float16)v;   // round to nearest even, as half::f16::from_f32
+        std::memcpy(&t[at], &h, 2);
+    });
     return ft_upload(ctx, dst_dev, t.data(), bytes);
 }
 

@@ -39,7 +39,9 @@ def empty(ctx, *shape):
 MATMUL_SHAPES = [(1, 1, 1), (1, 7, 1), (3, 5, 7), (16, 16, 16), (17, 33, 9), (64, 64, 64), (65, 1, 130),
                  (127, 129, 65), (1, 512, 300), (300, 512, 1), (256, 384, 128), (130, 70, 200), (256, 96, 320),
                  # the DMA-fed f32 kernels: ragged last tiles, rows that are no multiple of 4, one and many K tiles
-                 (200, 128, 132), (132, 64, 260), (130, 64, 256), (260, 2048, 128), (129, 96, 131), (2048, 576, 1536), (256, 4096, 192)]
+                 (200, 128, 132), (132, 64, 260), (130, 64, 256), (260, 2048, 128), (129, 96, 131), (2048, 576, 1536), (256, 4096, 192),
+                 # the kernel microbenchmark's weight-gradient product x^T @ dY: M = in, K = rows, N = out
+                 (576, 2048, 1536)]
 
 # GEMM tolerance of the reference's f64 comparisons (gpu_kernels.rs:989-1084): 1e-3 + 1e-4*|want|
 # for N(0,1) operands; the oracle itself adds in f32, so compare against f64 here.
@@ -67,9 +69,12 @@ def test_matmul_layouts_match_cpu(g, M, K, N):
     assert_close(f"matmul vs oracle {M}x{K}x{N}", out.to_numpy(), cpu.matmul(a, b), atol=1e-3, rtol=1e-4)
 
 
-SMOLLM2_PROJECTIONS = [("135M q/o", 576, 576), ("135M k/v", 576, 192), ("135M gate/up", 576, 1536),
-                       ("135M down", 1536, 576), ("360M q/o", 960, 960), ("360M k/v", 960, 320),
-                       ("360M gate/up", 960, 2560), ("360M down", 2560, 960), ("1.7B q/k/v/o", 2048, 2048)]
+# every row of gpu_kernels.rs:966-982
+SMOLLM2_PROJECTIONS = [("135M q/o", 576, 576), ("135M k/v", 576, 192), ("135M fused qkv", 576, 960),
+                       ("135M gate/up", 576, 1536), ("135M down", 1536, 576), ("135M lm_head", 576, 49152),
+                       ("360M q/o", 960, 960), ("360M k/v", 960, 320), ("360M fused qkv", 960, 1600),
+                       ("360M gate/up", 960, 2560), ("360M down", 2560, 960), ("360M lm_head", 960, 49152),
+                       ("1.7B q/k/v/o", 2048, 2048), ("1.7B gate/up", 2048, 8192), ("1.7B down", 8192, 2048)]
 
 
 @pytest.mark.parametrize("name,K,N", SMOLLM2_PROJECTIONS)
@@ -88,6 +93,33 @@ def test_f16_weight_projections(g, name, K, N, M):
     dx = empty(ctx, M, K)
     eng.matmul_bt_f16b(ctx, up(ctx, gy), w16, dx)
     assert_close(f"{name} matmul_bt_f16b", dx.to_numpy(), f64_mm(gy, wr.T), atol=2e-3, rtol=1e-4)
+
+
+@pytest.mark.parametrize("name,M,K,N", [("1.7B gate/up, 8 x 1024 rows", 8192, 2048, 8192),
+                                        ("1.7B down, 8 x 1024 rows", 8192, 8192, 2048),
+                                        ("360M lm_head on the supervised rows of the headline batch", 1446, 960, 49152)])
+def test_projections_at_the_row_counts_of_the_full_batches(g, name, M, K, N):
+    """The GEMMs of the 1.7B-shaped step at its real row count (M = 8192: thousands of tiles per launch) and
+    the vocabulary head (the 128x128 tile): forward and input gradient, sampled rows against f64 (the full
+    f64 product of these shapes would take the CPU minutes; every row block and column panel is sampled)."""
+    from ferrotensor_amd import UnifiedTensor
+    ctx, eng = g
+    rng = np.random.default_rng(K + N)
+    a = rng.standard_normal((M, K), dtype=np.float32)
+    w = rng.standard_normal((K, N), dtype=np.float32) * np.float32(0.05)
+    w16 = UnifiedTensor.from_f32_as_f16(ctx, w, [K, N])
+    wr = cpu.round_f16(w)
+    del w
+    rows = np.unique(np.concatenate([np.arange(0, M, 61), [M - 1, M - 2, 63, 64, 127, 128]]))
+    out = empty(ctx, M, N)
+    eng.matmul_f16b(ctx, up(ctx, a), w16, out)
+    assert_close(f"{name} matmul_f16b", out.to_numpy()[rows], f64_mm(a[rows], wr), atol=2e-3, rtol=1e-4)
+    del out
+    gy = rng.standard_normal((M, N), dtype=np.float32)
+    dx = empty(ctx, M, K)
+    eng.matmul_bt_f16b(ctx, up(ctx, gy), w16, dx)
+    bar = 2e-3 * max(1.0, np.sqrt(N / 2048.0))     # sums of N products of N(0,1) x N(0,0.05): spread grows as sqrt(N)
+    assert_close(f"{name} matmul_bt_f16b", dx.to_numpy()[rows], f64_mm(gy[rows], wr.T), atol=bar, rtol=1e-4)
 
 
 @pytest.mark.parametrize("M,K,N", [(1536, 2560, 960), (2048, 1024, 960), (1472, 2048, 896)])
@@ -128,6 +160,8 @@ def test_f16_upload_is_bit_exact(g):
 
 
 @pytest.mark.parametrize("M,K,N,r", [(64, 32, 48, 4), (256, 576, 1536, 8), (100, 960, 320, 8), (96, 64, 40, 16),
+                                     # ranks the vector kernels do not take (not 4, 8 or 16): the general route
+                                     (96, 64, 40, 2), (256, 576, 1536, 32), (70, 96, 200, 1), (128, 192, 64, 12),
                                      (2048, 576, 1536, 8)])  # the last: the kernel-microbench GEMM, full size
 @pytest.mark.parametrize("f16", [False, True])
 def test_fused_lora_linear_forward_and_backward(g, M, K, N, r, f16):
@@ -549,6 +583,8 @@ ATTN_CASES = [
     (8, 256, 256, 9, 3, 64, True, 0),       # the kernel-microbench attention case, full size
     (2, 256, 256, 15, 5, 64, True, 0),      # SmolLM2-360M heads
     (1, 256, 256, 15, 5, 64, True, 0),      # one sequence per pass: dK/dV per query head + ordered sum, dQ on 4 waves
+    (1, 1024, 1024, 32, 32, 64, True, 0),   # SmolLM2-1.7B heads at seq 1024 (no grouping)
+    (2, 1024, 1024, 8, 2, 64, True, 0),     # grouped heads at seq 1024
     (1, 70, 70, 2, 1, 128, True, 0),
     (1, 33, 65, 2, 1, 32, True, 32),        # queries at positions 32.. against a longer key run
     (1, 5, 37, 4, 4, 24, False, 0),

@@ -476,6 +476,43 @@ def test_a_trainer_is_refused_after_the_adapters_change(ctx):
     assert Trainer(hip, lr=1e-3).train_chunk(rows, targets, masks).optimizer_step
 
 
+@pytest.mark.parametrize("rank", [2, 32])
+def test_other_ranks_step_with_accumulation_matches_oracle(ctx, rank):
+    """Ranks outside {4, 8, 16} take the general kernels for x@A, dT, dA, dB and the rank-r terms, and with
+    two micro-batches per window the accumulate branch of the factor gradients (temporary + add). Two
+    optimizer steps of a window of 4 sequences fed 2 + 2, against the oracle's summed gradients."""
+    from ferrotensor_amd.trainer import Trainer
+    cfg = tiny_config(True, True)
+    mods = ["q_proj", "k_proj", "v_proj", "o_proj", "gate_proj", "up_proj", "down_proj"]
+    hip, orc = build_pair(ctx, cfg, mods, rank=rank, alpha=2.0 * rank, seed=37)
+    rng = np.random.default_rng(7)
+    B, S = 4, 16
+    rows = rng.integers(0, 256, (B, S)).astype(np.uint32)
+    targets = np.concatenate([rows[:, 1:], rows[:, :1]], axis=1)
+    masks = (rng.random((B, S)) > 0.2).astype(np.uint8)
+    tr = Trainer(hip, lr=1e-3, weight_decay=0.0, clip_grad_norm=1.0, grad_accum_steps=B)
+    opt = rs.AdamW(lr=1e-3, weight_decay=0.0)
+    for step in range(2):
+        first = tr.train_chunk(rows[:2], targets[:2], masks[:2])
+        assert not first.optimizer_step
+        st = tr.train_chunk(rows[2:], targets[2:], masks[2:])
+        assert st.optimizer_step
+        # the oracle on all four sequences at once: the same window
+        want = rs.train_chunk(orc, opt, rows, targets, masks, clip_grad_norm=1.0)
+        assert_close("loss", [first.loss + st.loss], [want.loss])
+        assert_close("grad_norm", [st.grad_norm], [want.grad_norm])
+        params = hip.params()
+        for n, w in orc.lora_params():
+            assert_close(f"step {step} weight {n}", params[n], w, atol=1e-6, rtol=1e-4)
+    # and the gradients themselves, element by element, on one more window
+    tr.train_chunk(rows[:2], targets[:2], masks[:2], apply=False)
+    tr.train_chunk(rows[2:], targets[2:], masks[2:], apply=False)
+    grads = hip.grads()
+    want, _, want_grads = rs.train_chunk(orc, opt, rows, targets, masks, clip_grad_norm=None, return_grads=True)
+    for n in grads:
+        assert_close(f"grad {n}", grads[n], want_grads[n])
+
+
 def test_warmup_cosine_schedule_drives_the_step(ctx):
     """Optimizer step k uses the schedule's value at k (trainer/src/lib.rs:345-352); a resumed
     trainer continues the curve where the counter says."""
