@@ -1120,7 +1120,8 @@ __global__ __launch_bounds__(NSPL * 64) void attn_bwd_dq_lds_kernel(AttnArgs p) 
 // The unguarded vector loads need whole, aligned quads in every row.
 bool attn_full(const AttnArgs& a, int DP) {
     auto al = [](const void* q) { return q == nullptr || (((uintptr_t)q) & 15) == 0; };
-    return a.D == DP && al(a.q) && al(a.k) && al(a.v) && al(a.out) && al(a.d_out);
+    // o (forward) and dq / dk / dv (backward) are written as 16-byte groups; NULL in the other pass
+    return a.D == DP && al(a.q) && al(a.k) && al(a.v) && al(a.out) && al(a.d_out) && al(a.o) && al(a.dq) && al(a.dk) && al(a.dv);
 }
 
 template <int DP>

@@ -32,20 +32,6 @@ struct ft_context {
     // Per-query-head partial dK/dV of the attention backward at small batch; allocated on first use.
     float* attn_scratch = nullptr;
 
-    // Extra streams ("lanes") for work that can run beside the main stream:
-    // lane 0 carries the LoRA factor gradients of a training step (only the
-    // optimizer reads them); lane 1 is free. ft_side_begin makes a lane wait for
-    // everything enqueued on the main stream so far and redirects launches to
-    // it, ft_side_end switches back, ft_side_join makes the main stream wait for
-    // one lane or for all of them. Buffers a lane still reads must not be freed
-    // or rewritten on the main stream before the join.
-    static constexpr int kLanes = 2;
-    hipStream_t side_stream[kLanes] = {nullptr, nullptr};
-    hipEvent_t fork_event[kLanes] = {nullptr, nullptr}, join_event[kLanes] = {nullptr, nullptr};
-    bool side_pending[kLanes] = {false, false};
-    hipStream_t main_stream = nullptr;  // saved while launches are redirected
-    int side_active = -1;               // lane that launches are redirected to, or -1
-
     // Per-kernel timing with HIP events on the context's stream (off by default).
     struct ProfRecord {
         int key;
@@ -79,9 +65,6 @@ int ft_set_error(int code, const char* fmt, ...);
 // ft_rms_norm_backward_noalloc (ft_rowops.hip). `device` must be the current device.
 int ft_internal_noalloc_init(int device);
 
-int ft_side_begin(ft_context* ctx, int lane = 0);
-int ft_side_end(ft_context* ctx);
-int ft_side_join(ft_context* ctx, int lane = -1);  // -1: every lane
 
 #define FT_CHECK_ARG(cond, ...)                                  \
     do {                                                         \

@@ -1523,7 +1523,8 @@ bool async_eligible(int layout, const float* a, const void* b, const float* out,
     if (layout != 0 && layout != 1) return false;
     if (M == 0 || N == 0 || K < 32 || K % 32 != 0) return false;
     if (!aligned16p(a) || !aligned16p(b) || !aligned16p(out) || !out || !a || !b) return false;
-    (void)add;
+    // The residual is read in 16-byte groups (epilogue and split-K reduce kernel alike).
+    if (add && !aligned16p(add)) return false;
     if (layout == 0 && (N % 8 != 0 || N < 8)) return false;
     if (K2 > 0 && (K2 > 16 || K2 % 4 != 0 || !aligned16p(a2) || !aligned16p(b2))) return false;
     // Per-lane operand offsets are 32-bit byte offsets from a uniform base.

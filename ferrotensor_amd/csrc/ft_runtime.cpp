@@ -47,47 +47,8 @@ ft_prof_scope::~ft_prof_scope() {
     if (index >= 0) (void)hipEventRecord(ctx->prof_records[index].e1, ctx->stream);
 }
 
-int ft_side_begin(ft_context* ctx, int lane) {
-    FT_CHECK_ARG(ctx && ctx->side_active < 0, "ft_side_begin: already redirected");
-    FT_CHECK_ARG(lane >= 0 && lane < ft_context::kLanes, "ft_side_begin: lane %d", lane);
-    if (!ctx->side_stream[lane]) {
-        FT_HIP(hipSetDevice(ctx->device));
-        FT_HIP(hipStreamCreateWithFlags(&ctx->side_stream[lane], hipStreamNonBlocking));
-        FT_HIP(hipEventCreateWithFlags(&ctx->fork_event[lane], hipEventDisableTiming));
-        FT_HIP(hipEventCreateWithFlags(&ctx->join_event[lane], hipEventDisableTiming));
-    }
-    FT_HIP(hipEventRecord(ctx->fork_event[lane], ctx->stream));
-    FT_HIP(hipStreamWaitEvent(ctx->side_stream[lane], ctx->fork_event[lane], 0));
-    ctx->main_stream = ctx->stream;
-    ctx->stream = ctx->side_stream[lane];
-    ctx->side_active = lane;
-    return FT_OK;
-}
-
-int ft_side_end(ft_context* ctx) {
-    FT_CHECK_ARG(ctx && ctx->side_active >= 0, "ft_side_end: not redirected");
-    const int lane = ctx->side_active;
-    const hipError_t e = hipEventRecord(ctx->join_event[lane], ctx->side_stream[lane]);
-    ctx->stream = ctx->main_stream;
-    ctx->side_active = -1;
-    ctx->side_pending[lane] = true;
-    FT_HIP(e);
-    return FT_OK;
-}
-
-int ft_side_join(ft_context* ctx, int lane) {
-    FT_CHECK_ARG(ctx && ctx->side_active < 0, "ft_side_join: still redirected");
-    for (int l = 0; l < ft_context::kLanes; l++) {
-        if ((lane >= 0 && l != lane) || !ctx->side_pending[l]) continue;
-        ctx->side_pending[l] = false;
-        FT_HIP(hipStreamWaitEvent(ctx->stream, ctx->join_event[l], 0));
-    }
-    return FT_OK;
-}
-
 // Waits for the stream and folds the finished records into the totals.
 static int prof_collect(ft_context* ctx) {
-    FT_TRY(ft_side_join(ctx));
     FT_HIP(hipStreamSynchronize(ctx->stream));
     for (auto& r : ctx->prof_records) {
         float ms = 0.0f;
@@ -198,13 +159,6 @@ int ft_context_destroy(ft_context* ctx) {
         (void)hipEventDestroy(r.e1);
     }
     for (hipEvent_t e : ctx->prof_event_pool) (void)hipEventDestroy(e);
-    for (int l = 0; l < ft_context::kLanes; l++) {
-        if (!ctx->side_stream[l]) continue;
-        (void)hipStreamSynchronize(ctx->side_stream[l]);
-        (void)hipEventDestroy(ctx->fork_event[l]);
-        (void)hipEventDestroy(ctx->join_event[l]);
-        (void)hipStreamDestroy(ctx->side_stream[l]);
-    }
     if (ctx->thin_scratch) (void)hipFree(ctx->thin_scratch);
     if (ctx->gemm_scratch) (void)hipFree(ctx->gemm_scratch);
     if (ctx->attn_scratch) (void)hipFree(ctx->attn_scratch);
@@ -215,7 +169,6 @@ int ft_context_destroy(ft_context* ctx) {
 
 int ft_synchronize(ft_context* ctx) {
     FT_CHECK_ARG(ctx, "ft_synchronize: ctx is NULL");
-    FT_TRY(ft_side_join(ctx));
     FT_HIP(hipStreamSynchronize(ctx->stream));
     return FT_OK;
 }
@@ -292,7 +245,6 @@ int ft_upload(ft_context* ctx, void* dst_dev, const void* src_host, size_t bytes
 int ft_download(ft_context* ctx, void* dst_host, const void* src_dev, size_t bytes) {
     FT_CHECK_ARG(ctx && (bytes == 0 || (dst_host && src_dev)), "ft_download: NULL argument");
     if (bytes == 0) return FT_OK;
-    FT_TRY(ft_side_join(ctx));
     FT_HIP(hipMemcpyAsync(dst_host, src_dev, bytes, hipMemcpyDeviceToHost, ctx->stream));
     FT_HIP(hipStreamSynchronize(ctx->stream));
     return FT_OK;

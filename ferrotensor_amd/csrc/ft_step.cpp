@@ -126,9 +126,9 @@ struct ft_model {
     float *g0 = nullptr, *g1 = nullptr, *d_act = nullptr, *d_gate = nullptr, *d_up = nullptr, *d_h2 = nullptr,
           *d_attn = nullptr, *dq = nullptr, *dk = nullptr, *dv = nullptr, *d_h1 = nullptr, *dt = nullptr,
           *dt2 = nullptr, *dt3 = nullptr, *gtmp = nullptr, *rope_table = nullptr;
-    // Factor gradients (dA, dB) waiting for their launch on the side stream: the products of up to
-    // four linears go out together (one fork per block instead of one per linear). Each waiting
-    // linear keeps its own dT buffer from dt_pool until the main stream has joined the side stream.
+    // Factor gradients (dA, dB) waiting for their launch: the products of a block's adapted linears
+    // go out together in batched launches (flush_cols), before anything they read is rewritten.
+    // Each waiting linear keeps its own dT buffer from dt_pool until then.
     static constexpr int kDtPool = 8;
     float* dt_pool[kDtPool] = {};
     int dt_used = 0;
@@ -328,11 +328,9 @@ int linear_forward(ft_context* ctx, LinearW& l, const float* x, float* t, float*
     return linear_gemm(ctx, l, x, t, y, T, residual);
 }
 
-// Launches the waiting factor-gradient products on the side stream, in batches of equal rank.
+// Launches the waiting factor-gradient products in batches of equal rank; afterwards every dT
+// buffer is free again (launches of one stream run in order).
 int flush_cols(ft_model* m) {
-    if (m->pending_cols.empty()) return FT_OK;
-    ft_context* ctx = m->ctx;
-    FT_TRY(ft_side_begin(ctx));
     int rc = FT_OK;
     size_t i = 0;
     while (i < m->pending_cols.size() && rc == FT_OK) {
@@ -340,27 +338,17 @@ int flush_cols(ft_model* m) {
         while (i + n < m->pending_cols.size() && n < (size_t)FT_THIN_MAX_BATCH &&
                m->pending_cols[i + n].C == m->pending_cols[i].C)
             n++;
-        rc = ft_thin_colwise(ctx, &m->pending_cols[i], (int)n);
+        rc = ft_thin_colwise(m->ctx, &m->pending_cols[i], (int)n);
         i += n;
     }
     m->pending_cols.clear();
-    FT_TRY(ft_side_end(ctx));
+    m->dt_used = 0;
     return rc;
 }
 
-// The main stream waits for the side stream; afterwards every dT buffer is free again.
-int join_cols(ft_model* m) {
-    FT_TRY(ft_side_join(m->ctx, 0));
-    if (m->pending_cols.empty()) m->dt_used = 0;
-    return FT_OK;
-}
-
-// A dT buffer nobody on the side stream still reads.
+// A dT buffer no waiting product reads.
 int take_dt(ft_model* m, float** dt) {
-    if (m->dt_used == ft_model::kDtPool) {
-        FT_TRY(flush_cols(m));
-        FT_TRY(join_cols(m));
-    }
+    if (m->dt_used == ft_model::kDtPool) FT_TRY(flush_cols(m));
     *dt = m->dt_pool[m->dt_used++];
     return FT_OK;
 }
@@ -372,6 +360,8 @@ int linear_backward(ft_model* m, LinearW& l, const float* x, const float* t, con
     ft_context* ctx = m->ctx;
     if (l.has_lora()) {
         float* dt = nullptr;
+        // room for this linear's two products first: a flush frees every dT buffer
+        if (m->pending_cols.size() + 2 > (size_t)FT_THIN_MAX_BATCH) FT_TRY(flush_cols(m));
         FT_TRY(take_dt(m, &dt));
         FT_TRY(ft_lora_grad_down(ctx, dy, l.b, dt, T, l.out, l.r, l.scale()));
         // dB = t^T dy and dA = x^T dt in one sliced launch when possible (added to the
@@ -381,11 +371,9 @@ int linear_backward(ft_model* m, LinearW& l, const float* x, const float* t, con
             {dy, t, l.gb, (int)T, 0, (int)l.out, (int)l.r, (long)l.out, (long)l.r, (long)l.out, 1.0f, 0, 1, 0, acc},
             {x, dt, l.ga, (int)T, 0, (int)l.in, (int)l.r, (long)l.in, (long)l.r, (long)l.r, 1.0f, 0, 0, 0, acc}};
         if (ft_thin_colwise_ok(pb[0]) && ft_thin_colwise_ok(pb[1])) {
-            // Only the optimizer reads dA and dB: they wait for the next launch on the side stream,
-            // which runs beside an input-gradient GEMM.
+            // Only the optimizer reads dA and dB: they wait for the block's batched launch.
             m->pending_cols.push_back(pb[0]);
             m->pending_cols.push_back(pb[1]);
-            if (m->pending_cols.size() >= (size_t)FT_THIN_MAX_BATCH) FT_TRY(flush_cols(m));
         } else if (accumulate) {
             FT_TRY(ft_lora_grad_b(ctx, t, dy, m->gtmp, T, l.out, l.r));
             FT_TRY(ft_gradient_accumulate(ctx, l.gb, m->gtmp, l.r * l.out));
@@ -417,10 +405,9 @@ int linear_backward_group(ft_model* m, LinearW* const* ls, const float* const* t
     for (int i = 0; i < n; i++) batch = batch && ls[i]->has_lora() && ls[i]->r == ls[0]->r;
     float* dts[3] = {nullptr, nullptr, nullptr};
     if (batch) {
-        if (m->dt_used + n > ft_model::kDtPool) {
+        // room for this group's products and dT buffers first: a flush frees every dT buffer
+        if (m->dt_used + n > ft_model::kDtPool || m->pending_cols.size() + 2 * (size_t)n > (size_t)FT_THIN_MAX_BATCH)
             FT_TRY(flush_cols(m));
-            FT_TRY(join_cols(m));
-        }
         for (int i = 0; i < n; i++) FT_TRY(take_dt(m, &dts[i]));
     }
     const int acc = accumulate ? 1 : 0;
@@ -452,9 +439,8 @@ int linear_backward_group(ft_model* m, LinearW* const* ls, const float* const* t
         return ft_lora_linear_dx_group(ctx, d, (size_t)n, nullptr, dx, T, ls[0]->in);
     }
     FT_TRY(ft_thin_rowwise(ctx, rows, n));
-    if (m->pending_cols.size() + 2 * (size_t)n > (size_t)FT_THIN_MAX_BATCH) FT_TRY(flush_cols(m));
     for (int i = 0; i < 2 * n; i++) m->pending_cols.push_back(cols[i]);
-    if (flush || m->pending_cols.size() >= (size_t)FT_THIN_MAX_BATCH) FT_TRY(flush_cols(m));
+    if (flush) FT_TRY(flush_cols(m));
     if (dx) {
         ft_lora_dx_desc d[3];
         for (int i = 0; i < n; i++)
@@ -588,12 +574,9 @@ int model_backward(ft_model* m, size_t B, size_t S, bool accumulate) {
     for (size_t li = m->layers.size(); li-- > 0;) {
         Layer& L = m->layers[li];
         LayerActs& a = m->acts[li];
-        // The factor gradients of the block above (side stream) read its output gradients (g_other,
-        // dq/dk/dv; d_up/d_gate when the MLP has adapters) and, with checkpointing, the shared block
-        // buffers. All of those are rewritten below: wait for the side stream before the first such
-        // write, as late as possible so that short GEMMs (one sequence per pass) still hide it.
-        const bool join_at_top = c.checkpoint_blocks || L.up.has_lora() || L.gate.has_lora() || L.down.has_lora();
-        if (join_at_top) FT_TRY(join_cols(m));
+        // The factor gradients of a block read its activations, output gradients and dT buffers; they
+        // are launched (flush_cols) at the block's end, before g, the buffers of the next block's
+        // gradients and, with checkpointing, the shared block buffers are rewritten.
         if (c.checkpoint_blocks && li + 1 < m->layers.size()) {
             // Recompute this block's forward. (The last block's internals are still there from the
             // forward pass.)
@@ -614,7 +597,6 @@ int model_backward(ft_model* m, size_t B, size_t S, bool accumulate) {
             FT_TRY(linear_backward_group(m, ls, ts, dys, m->d_h2, 2, a.h2, T, accumulate, false));
         }
         // g_h = g + norm2_backward(d_h2) (into g_other)
-        if (!join_at_top) FT_TRY(join_cols(m));
         FT_TRY(ft_internal_rms_norm_backward_add(ctx, a.h, L.norm2, m->d_h2, g, g_other, T, H, c.rms_norm_eps));
         // h = x + o_proj(attn)
         FT_TRY(linear_backward(m, L.o, a.attn, a.to, g_other, m->d_attn, T, accumulate));
@@ -642,17 +624,14 @@ int model_backward(ft_model* m, size_t B, size_t S, bool accumulate) {
             const float* ts[3] = {a.tq, a.tk, a.tv};
             const float* dys[3] = {m->dq, m->dk, m->dv};
             // d_h1 = dx_q + dx_k + dx_v
-            // the block's last adapters: everything that waited goes to the side stream now
+            // the block's last adapters: everything that waited is launched now
             FT_TRY(linear_backward_group(m, ls, ts, dys, need_dx ? m->d_h1 : nullptr, 3, a.h1, T, accumulate, true));
         }
         if (!need_dx) break;
-        // g is rewritten next; the down projection's factor gradients read it
-        if (L.down.has_lora()) FT_TRY(join_cols(m));
         // g = g_h + norm1_backward(d_h1)
         FT_TRY(ft_internal_rms_norm_backward_add(ctx, a.x, L.norm1, m->d_h1, g_other, g, T, H, c.rms_norm_eps));
     }
-    FT_TRY(flush_cols(m));
-    return join_cols(m);
+    return flush_cols(m);
 }
 
 LinearW* find_linear(ft_model* m, const std::string& prefix) {

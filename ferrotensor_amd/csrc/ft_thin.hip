@@ -1,14 +1,14 @@
 // The rank-r products around a LoRA linear (r = 4, 8 or 16): bandwidth-bound
-// work with almost no flops, so they run on the vector ALUs with fully
-// coalesced loads, and several independent products go into one launch.
+// work with almost no flops: fully coalesced 16-byte loads, the small
+// contraction on the matrix unit, several independent products per launch.
 //
 //   row-wise   out[M, C] = scale * X[M, K] @ Y        (x@A,  dT = dY@B^T)
 //              16 rows per workgroup, K split over its 4 waves, 16x16x4 MFMA
 //              (the matrix unit does the K reduction, no cross-lane shuffles).
 //   col-wise   out[R, C] = X[M, R]^T @ Y[M, C]        (dA = x^T@dT, dB = T^T@dY)
-//              each thread owns 4 columns of X, the M rows are cut into
-//              slices; a second kernel adds the slices in order (deterministic,
-//              no atomics).
+//              64 columns of X per workgroup, the M rows cut into slices and
+//              contracted by the same MFMA; a second kernel adds the slices
+//              in order (deterministic, no atomics).
 #include "ft_common.h"
 #include "ft_thin.h"
 
@@ -90,87 +90,173 @@ __global__ __launch_bounds__(kRowWaves * 64) void thin_rowwise_kernel(ThinBatch 
 }
 
 // ---- col-wise ---------------------------------------------------------------
-// grid (ceil(Rmax / 256), count, slices); 256 threads = 4 waves. Every thread owns
-// 4 columns of X (a wave 256 of them); the rows of a slice are dealt to the four
-// waves in contiguous quarters and the four partial results are added in wave
-// order through LDS. partial[((slice * R) + n) * C + j] at p.scratch_offset.
-template <int C>
-__global__ __launch_bounds__(256) void thin_colwise_kernel(ThinBatch b, float* __restrict__ scratch, int slices) {
-    const ft_thin_problem& p = b.p[blockIdx.y];
-    if ((int)blockIdx.x * 256 >= p.R) return;  // whole workgroup past this problem's width
-    __shared__ float red[3][4 * C][kWave + 1];
-    const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
-    const int n = (blockIdx.x * 64 + lane) * 4;
-    const bool live = n < p.R;  // R is a multiple of 4 (checked on the host)
-    const int per = (p.M + slices - 1) / slices;
-    const int s_begin = blockIdx.z * per;
-    const int s_end = s_begin + per < p.M ? s_begin + per : p.M;
-    const int quarter = (per + 3) / 4;
-    const int m_begin = s_begin + wave * quarter;
-    const int m_end = m_begin + quarter < s_end ? m_begin + quarter : s_end;
-    float acc[4][C];
+// out_i[R, C] = X[M, R]^T @ Y_i[M, C] for up to three Y_i that share X (the dA of q/k/v all
+// contract the same norm output with their own dT): X is read once for all of them.
+//
+// The contraction over the M rows runs on the matrix unit: v_mfma_f32_16x16x4_f32 with the
+// factor columns as the 16 output rows (virtual column v = i * C + c of product i; 16 per "set",
+// up to 3 sets, unused ones fed zeros), 4 rows of M as k, and 16 columns of X as output columns.
+// A lane (j = lane % 16, kq = lane / 16) fetches X[m0 + kq][n0 + 4j .. 4j+3] as one 16-byte load:
+// a wave load covers four 256-byte row segments, and component e of the quad feeds MFMA e, whose
+// tile therefore holds the columns n0 + 4j + e. One load instruction pays for 4 * sets MFMAs and a
+// wave keeps eight of them in flight.
+//
+// grid (column tiles of 64 over all problems of the batch, M slices); 256 threads = 4 waves that
+// split the slice's rows; their tiles are added in wave order through LDS and the workgroup
+// writes one partial tile: partial[((slice * R) + n) * VC + v] at p.scratch_offset, VC = ny * C.
+// thin_colwise_finish_kernel adds the slices in order (deterministic, no atomics).
+struct ColProblem {
+    const float* x;
+    const float* y[3];
+    float* out[3];
+    int M, R, C, ny;
+    long ldx, ldy, ldo;
+    float scale;
+    int out_transposed, accumulate;
+    long scratch_offset;
+    int tile_begin;   // index of this problem's first column tile in grid.x
+    int slices;       // M slices of this problem (<= gridDim.y)
+};
+
+struct ColBatch {
+    ColProblem p[FT_THIN_MAX_BATCH];
+    int count;
+    int rows_per_wg;    // multiple of 4 * kColWaves
+    int rows_per_wave;  // rows_per_wg / kColWaves
+};
+
+constexpr int kColWaves = 4;
+constexpr int kColUnroll = 8;   // 4-row groups whose loads are issued together
+
+// The loads of one batch: kColUnroll groups of 4 rows from m0 (rows >= m_end read as zeros).
+template <int NSET>
+__device__ __forceinline__ void col_load(const float* xp, long ldx, const float* const (&yp)[NSET], long ldy, int nsets,
+                                         int m0, int m_end, int kq, bool live, float4 (&xv)[kColUnroll],
+                                         float (&yv)[kColUnroll][NSET]) {
 #pragma unroll
-    for (int e = 0; e < 4; e++)
+    for (int u = 0; u < kColUnroll; u++) {
+        const int m = m0 + 4 * u + kq;
+        const bool in = m < m_end;
+        xv[u] = (in && live) ? *reinterpret_cast<const float4*>(xp + (long)m * ldx) : make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
-        for (int j = 0; j < C; j++) acc[e][j] = 0.0f;
-    if (live) {
-        const float* xp = p.x + n;
-#pragma unroll 8
-        for (int m = m_begin; m < m_end; m++) {
-            const float4 xv = *reinterpret_cast<const float4*>(xp + (long)m * p.ldx);
-            const float* yr = p.y + (long)m * p.ldy;  // uniform across the wave
-#pragma unroll
-            for (int j = 0; j < C; j++) {
-                const float yv = yr[j];
-                acc[0][j] += xv.x * yv;
-                acc[1][j] += xv.y * yv;
-                acc[2][j] += xv.z * yv;
-                acc[3][j] += xv.w * yv;
-            }
+        for (int s = 0; s < NSET; s++) {
+            yv[u][s] = 0.0f;
+            if (s < nsets) yv[u][s] = (in && yp[s]) ? yp[s][(long)m * ldy] : 0.0f;
         }
-    }
-    if (wave > 0) {
-#pragma unroll
-        for (int e = 0; e < 4; e++)
-#pragma unroll
-            for (int j = 0; j < C; j++) red[wave - 1][e * C + j][lane] = acc[e][j];
-    }
-    __syncthreads();
-    if (wave == 0 && live) {
-#pragma unroll
-        for (int e = 0; e < 4; e++)
-#pragma unroll
-            for (int j = 0; j < C; j++)
-                acc[e][j] = ((acc[e][j] + red[0][e * C + j][lane]) + red[1][e * C + j][lane]) + red[2][e * C + j][lane];
-        float* dst = scratch + p.scratch_offset + ((long)blockIdx.z * p.R + n) * C;
-#pragma unroll
-        for (int e = 0; e < 4; e++)
-#pragma unroll
-            for (int j = 0; j < C; j += 4)
-                *reinterpret_cast<float4*>(dst + e * C + j) =
-                    make_float4(acc[e][j], acc[e][j + 1], acc[e][j + 2], acc[e][j + 3]);
     }
 }
 
-// out[n][j] (or out[j][n] when transposed) = scale * sum over slices, in slice order.
-__global__ __launch_bounds__(256) void thin_finish_kernel(ThinBatch b, const float* __restrict__ scratch, int slices) {
-    const ft_thin_problem& p = b.p[blockIdx.y];
+template <int NSET>
+__device__ __forceinline__ void col_mfma(thin_f4 (&acc)[NSET][4], int nsets, const float4 (&xv)[kColUnroll],
+                                         const float (&yv)[kColUnroll][NSET]) {
+#pragma unroll
+    for (int u = 0; u < kColUnroll; u++)
+#pragma unroll
+        for (int s = 0; s < NSET; s++) {
+            if (s >= nsets) continue;
+            acc[s][0] = __builtin_amdgcn_mfma_f32_16x16x4f32(yv[u][s], xv[u].x, acc[s][0], 0, 0, 0);
+            acc[s][1] = __builtin_amdgcn_mfma_f32_16x16x4f32(yv[u][s], xv[u].y, acc[s][1], 0, 0, 0);
+            acc[s][2] = __builtin_amdgcn_mfma_f32_16x16x4f32(yv[u][s], xv[u].z, acc[s][2], 0, 0, 0);
+            acc[s][3] = __builtin_amdgcn_mfma_f32_16x16x4f32(yv[u][s], xv[u].w, acc[s][3], 0, 0, 0);
+        }
+}
+
+template <int NSET>
+__global__ __launch_bounds__(kColWaves * 64) void thin_colwise_mfma_kernel(ColBatch b, float* __restrict__ scratch) {
+    int pi = 0;
+#pragma unroll
+    for (int i = 1; i < FT_THIN_MAX_BATCH; i++)
+        if (i < b.count && (int)blockIdx.x >= b.p[i].tile_begin) pi = i;
+    const ColProblem& p = b.p[pi];
+    const int wg_begin = blockIdx.y * b.rows_per_wg;
+    if (wg_begin >= p.M) return;   // uniform: this problem has fewer slices than the grid
+    __shared__ float red[kColWaves - 1][NSET * 16][kWave];
+    const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+    const int j = lane % 16, kq = lane / 16;
+    const int n = ((int)blockIdx.x - p.tile_begin) * 64 + 4 * j;
+    const bool live = n < p.R;   // R is a multiple of 4 (checked on the host)
+    const int wg_end = wg_begin + b.rows_per_wg < p.M ? wg_begin + b.rows_per_wg : p.M;
+    const int m_begin = wg_begin + wave * b.rows_per_wave;
+    const int m_end = m_begin + b.rows_per_wave < wg_end ? m_begin + b.rows_per_wave : wg_end;
+    // Where this lane's A operand (a factor column) of every set comes from.
+    const float* yp[NSET];
+#pragma unroll
+    for (int s = 0; s < NSET; s++) {
+        const int v = 16 * s + j;
+        const int yi = v / p.C, c = v % p.C;
+        const float* base = yi == 0 ? p.y[0] : (yi == 1 ? p.y[1] : p.y[2]);
+        yp[s] = yi < p.ny ? base + c : nullptr;
+    }
+    // Sets this problem fills (wave-uniform): a launch is compiled for the largest of its batch.
+    const int nsets = (p.ny * p.C + 15) / 16;
+    thin_f4 acc[NSET][4];
+#pragma unroll
+    for (int s = 0; s < NSET; s++)
+#pragma unroll
+        for (int e = 0; e < 4; e++) acc[s][e] = thin_f4{0.f, 0.f, 0.f, 0.f};
+    const float* xp = p.x + n;
+    // (Requesting the next batch of loads before multiplying the current one was measured: no gain.)
+    float4 xa[kColUnroll];
+    float ya[kColUnroll][NSET];
+    for (int m0 = m_begin; m0 < m_end; m0 += 4 * kColUnroll) {
+        col_load<NSET>(xp, p.ldx, yp, p.ldy, nsets, m0, m_end, kq, live, xa, ya);
+        col_mfma<NSET>(acc, nsets, xa, ya);
+    }
+    // acc[s][e][r] = sum over this wave's rows for virtual column 16s + 4kq + r, X column n + e
+    if (wave > 0) {
+#pragma unroll
+        for (int s = 0; s < NSET; s++)
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) red[wave - 1][(s * 4 + e) * 4 + r][lane] = acc[s][e][r];
+    }
+    __syncthreads();
+    if (wave == 0 && live) {
+        const int VC = p.ny * p.C;
+        float* dst = scratch + p.scratch_offset + ((long)blockIdx.y * p.R + n) * VC;
+#pragma unroll
+        for (int s = 0; s < NSET; s++) {
+            const int v = 16 * s + 4 * kq;
+            if (v >= VC) continue;   // VC is a multiple of 4: a quad of virtual columns is all in or all out
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                float o[4];
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    float t = acc[s][e][r];
+#pragma unroll
+                    for (int w = 0; w < kColWaves - 1; w++) t += red[w][(s * 4 + e) * 4 + r][lane];
+                    o[r] = t;
+                }
+                *reinterpret_cast<float4*>(dst + (long)e * VC + v) = make_float4(o[0], o[1], o[2], o[3]);
+            }
+        }
+    }
+}
+
+// out_i[n][c] (or out_i[c][n] when transposed) = scale * sum over slices, in slice order.
+__global__ __launch_bounds__(256) void thin_colwise_finish_kernel(ColBatch b, const float* __restrict__ scratch) {
+    const ColProblem& p = b.p[blockIdx.y];
     const int e = blockIdx.x * 256 + threadIdx.x;
-    const int total = p.R * p.C;
+    const int VC = p.ny * p.C;
+    const int total = p.R * VC;
     if (e >= total) return;
     const float* src = scratch + p.scratch_offset + e;
     float v = 0.0f;
     int s = 0;
-    for (; s + 8 <= slices; s += 8) {
+    for (; s + 8 <= p.slices; s += 8) {
         float t[8];
 #pragma unroll
         for (int u = 0; u < 8; u++) t[u] = src[(long)(s + u) * total];
 #pragma unroll
         for (int u = 0; u < 8; u++) v += t[u];
     }
-    for (; s < slices; s++) v += src[(long)s * total];
-    const int n = e / p.C, j = e % p.C;
-    float* o = p.out_transposed ? p.out + (long)j * p.ldo + n : p.out + (long)n * p.ldo + j;
+    for (; s < p.slices; s++) v += src[(long)s * total];
+    const int n = e / VC, vc = e % VC;
+    const int yi = vc / p.C, c = vc % p.C;
+    float* out = yi == 0 ? p.out[0] : (yi == 1 ? p.out[1] : p.out[2]);
+    float* o = p.out_transposed ? out + (long)c * p.ldo + n : out + (long)n * p.ldo + c;
     *o = p.accumulate ? *o + v * p.scale : v * p.scale;
 }
 
@@ -234,60 +320,93 @@ int ft_thin_rowwise(ft_context* ctx, const ft_thin_problem* probs, int count) {
 int ft_thin_colwise(ft_context* ctx, const ft_thin_problem* probs, int count) {
     FT_CHECK_ARG(ctx && probs && count >= 1 && count <= FT_THIN_MAX_BATCH, "thin colwise: bad batch");
     FT_TRY(ensure_scratch(ctx));
-    // The partial-sum buffer is shared: a call on the main stream must not overtake one on the side stream.
-    if (ctx->side_active < 0) FT_TRY(ft_side_join(ctx, 0));
-    ThinBatch b{};
-    b.count = count;
-    int rmax = 0, mmax = 0;
+    ColBatch b{};
+    int mmax = 0, vcmax = 0;
     double bytes = 0.0;
     for (int i = 0; i < count; i++) {
-        FT_CHECK_ARG(ft_thin_colwise_ok(probs[i]), "thin colwise: problem %d is not aligned for the vector kernel", i);
-        FT_CHECK_ARG(probs[i].C == probs[0].C, "thin colwise: a batch must share the rank");
-        if (probs[i].R > rmax) rmax = probs[i].R;
-        if (probs[i].M > mmax) mmax = probs[i].M;
+        const ft_thin_problem& q = probs[i];
+        FT_CHECK_ARG(ft_thin_colwise_ok(q), "thin colwise: problem %d is not aligned for the vector kernel", i);
+        FT_CHECK_ARG(q.C == probs[0].C, "thin colwise: a batch must share the rank");
+        if (q.R == 0) continue;   // an empty result; M == 0 gives zero slices: the finish kernel writes zeros
+        // Products that contract the same X (same rows, width and layout) share one problem.
+        int at = -1;
+        for (int k = 0; k < b.count && at < 0; k++) {
+            const ColProblem& c = b.p[k];
+            if (c.x == q.x && c.M == q.M && c.R == q.R && c.ldx == q.ldx && c.ldy == q.ldy && c.ldo == q.ldo &&
+                c.scale == q.scale && c.out_transposed == q.out_transposed && c.accumulate == q.accumulate &&
+                c.ny < 3)
+                at = k;
+        }
+        if (at < 0) {
+            at = b.count++;
+            ColProblem& c = b.p[at];
+            c.x = q.x;
+            c.M = q.M, c.R = q.R, c.C = q.C, c.ny = 0;
+            c.ldx = q.ldx, c.ldy = q.ldy, c.ldo = q.ldo;
+            c.scale = q.scale;
+            c.out_transposed = q.out_transposed, c.accumulate = q.accumulate;
+            bytes += 4.0 * (double)q.M * q.R;
+        }
+        ColProblem& c = b.p[at];
+        c.y[c.ny] = q.y;
+        c.out[c.ny] = q.out;
+        c.ny++;
+        bytes += 4.0 * ((double)q.M * q.C + (double)q.R * q.C);
+        if (q.M > mmax) mmax = q.M;
+        if (c.ny * c.C > vcmax) vcmax = c.ny * c.C;
     }
-    if (rmax == 0) return FT_OK;
-    // Rows per slice: enough slices to fill the chip, few enough that the
-    // partial sums stay a fraction of the input traffic.
-    int slices = mmax / 128;
-    if (slices > 16) slices = 16;
+    if (b.count == 0) return FT_OK;
+    int tiles = 0;
+    for (int i = 0; i < b.count; i++) {
+        b.p[i].tile_begin = tiles;
+        tiles += (b.p[i].R + 63) / 64;
+    }
+    // Rows per workgroup: enough workgroups to put several on every CU, few enough slices that the
+    // partial tiles stay a few percent of the input traffic; whole batches of loads per wave.
+    const int quantum = 4 * kColUnroll * kColWaves;   // 128 rows: one batch of loads per wave
+    const int want_wgs = 2 * ctx->num_cus;   // measured: 1x and 4x are both slower at the 360M shapes
+    int slices = want_wgs / tiles;
     if (slices < 1) slices = 1;
-    // A batch whose partial sums do not fit the scratch buffer goes out in pieces (the launches of
-    // one stream run in order, so the pieces may share the buffer).
-    {
-        size_t need = 0;
-        int fit = 0;
-        while (fit < count && need + (size_t)slices * probs[fit].R * probs[fit].C <= kScratchFloats) {
-            need += (size_t)slices * probs[fit].R * probs[fit].C;
-            fit++;
-        }
-        FT_CHECK_ARG(fit >= 1, "thin colwise: %zu partial sums of one product exceed the scratch buffer",
-                     (size_t)slices * probs[0].R * probs[0].C);
-        if (fit < count) {
-            FT_TRY(ft_thin_colwise(ctx, probs, fit));
-            return ft_thin_colwise(ctx, probs + fit, count - fit);
-        }
-    }
+    int rows_per_wg = ((mmax + slices - 1) / slices + quantum / 2) / quantum * quantum;
+    if (rows_per_wg < quantum) rows_per_wg = quantum;
+    b.rows_per_wg = rows_per_wg;
+    b.rows_per_wave = rows_per_wg / kColWaves;
     size_t off = 0;
-    for (int i = 0; i < count; i++) {
-        b.p[i] = probs[i];
-        b.p[i].scratch_offset = (long)off;
-        off += (size_t)slices * probs[i].R * probs[i].C;
-        bytes += 4.0 * ((double)probs[i].M * probs[i].R + (double)probs[i].M * probs[i].C +
-                        (double)probs[i].R * probs[i].C);
+    int smax = 1;
+    for (int i = 0; i < b.count; i++) {
+        ColProblem& c = b.p[i];
+        c.slices = (c.M + rows_per_wg - 1) / rows_per_wg;
+        if (c.slices > smax) smax = c.slices;
+        c.scratch_offset = (long)off;
+        off += (size_t)c.slices * c.R * c.ny * c.C;
     }
-    FT_CHECK_ARG(off <= kScratchFloats, "thin colwise: %zu partial sums exceed the scratch buffer", off);
-    const dim3 grid(ft_div_up(rmax, 256), (unsigned)count, (unsigned)slices);
-    const dim3 fgrid(ft_div_up((size_t)rmax * probs[0].C, 256), (unsigned)count);
+    if (off > kScratchFloats) {
+        // The partial tiles of the batch do not fit the buffer: one product at a time (launches of one
+        // stream run in order, so they may share it).
+        FT_CHECK_ARG(count > 1, "thin colwise: %zu partial sums of one product exceed the scratch buffer", off);
+        for (int i = 0; i < count; i++) FT_TRY(ft_thin_colwise(ctx, probs + i, 1));
+        return FT_OK;
+    }
+    const int nset = (vcmax + 15) / 16;
+    const dim3 grid((unsigned)tiles, (unsigned)smax);
+    size_t fmax = 0;
+    for (int i = 0; i < b.count; i++) {
+        const size_t t = (size_t)b.p[i].R * b.p[i].ny * b.p[i].C;
+        if (t > fmax) fmax = t;
+    }
+    const dim3 fgrid(ft_div_up(fmax, 256), (unsigned)b.count);
     ft_prof_scope prof(ctx, "thin_colwise+finish", 0.0, bytes);
-    if (probs[0].C == 4)
-        hipLaunchKernelGGL((thin_colwise_kernel<4>), grid, dim3(256), 0, ctx->stream, b, ctx->thin_scratch, slices);
-    else if (probs[0].C == 8)
-        hipLaunchKernelGGL((thin_colwise_kernel<8>), grid, dim3(256), 0, ctx->stream, b, ctx->thin_scratch, slices);
+    if (nset == 1)
+        hipLaunchKernelGGL((thin_colwise_mfma_kernel<1>), grid, dim3(kColWaves * 64), 0, ctx->stream, b,
+                           ctx->thin_scratch);
+    else if (nset == 2)
+        hipLaunchKernelGGL((thin_colwise_mfma_kernel<2>), grid, dim3(kColWaves * 64), 0, ctx->stream, b,
+                           ctx->thin_scratch);
     else
-        hipLaunchKernelGGL((thin_colwise_kernel<16>), grid, dim3(256), 0, ctx->stream, b, ctx->thin_scratch, slices);
+        hipLaunchKernelGGL((thin_colwise_mfma_kernel<3>), grid, dim3(kColWaves * 64), 0, ctx->stream, b,
+                           ctx->thin_scratch);
     FT_LAUNCH_CHECK();
-    hipLaunchKernelGGL(thin_finish_kernel, fgrid, dim3(256), 0, ctx->stream, b, ctx->thin_scratch, slices);
+    hipLaunchKernelGGL(thin_colwise_finish_kernel, fgrid, dim3(256), 0, ctx->stream, b, ctx->thin_scratch);
     FT_LAUNCH_CHECK();
     return FT_OK;
 }

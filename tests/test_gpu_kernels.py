@@ -644,3 +644,42 @@ def test_attention_rejects_unsupported_options(g):
         eng.flash_attention_v2_with(ctx, q, k, k, out, AttentionOptions(causal=True, window=2))
     with pytest.raises(FtError):
         eng.flash_attention_v2_with(ctx, q, k, k, out, AttentionOptions(causal=True, dropout_prob=0.1))
+
+
+def test_unaligned_residual_and_gradient_pointers_take_the_guarded_kernels(g):
+    """A residual, or attention gradient buffers, that are 4-byte but not 16-byte aligned (a view into the
+    middle of a buffer) must not reach the kernels that use 16-byte accesses: same results as aligned ones."""
+    import ctypes as C
+    from ferrotensor_amd import AttentionOptions, UnifiedTensor
+    from ferrotensor_amd._lib import check
+    ctx, eng = g
+    lib = ctx._lib
+    M, K, N = 256, 128, 192
+    x, w, res = rnd(1, M, K), rnd(2, K, N, scale=0.05), rnd(3, M * N + 1)
+    wt = UnifiedTensor.from_f32_as_f16(ctx, w, [K, N])
+    xt, rest, y = up(ctx, x), up(ctx, res), empty(ctx, M, N)
+    off = C.c_void_p(rest.ptr + 4)                       # element 1 of the residual buffer
+    check(lib.ft_lora_linear(ctx.handle, C.c_void_p(xt.ptr), C.c_void_p(wt.ptr), wt.dtype, None, None, off,
+                             C.c_void_p(y.ptr), M, K, N, 0))
+    want = f64_mm(x, cpu.round_f16(w)) + res[1:].reshape(M, N)
+    assert_close("residual at an odd offset", y.to_numpy(), want, atol=1e-3, rtol=1e-4)
+
+    B, S, H, D = 1, 64, 2, 64
+    q, k, v, do = rnd(4, B, S, H, D), rnd(5, B, S, H, D), rnd(6, B, S, H, D), rnd(7, B, S, H, D)
+    opts = AttentionOptions(causal=True)
+    tq, tk, tv, tdo = up(ctx, q), up(ctx, k), up(ctx, v), up(ctx, do)
+    out, stats = empty(ctx, B, S, H, D), UnifiedTensor.zeros(ctx, [B, H, S, 2])
+    eng.flash_attention_v2_with_stats(ctx, tq, tk, tv, out, stats, opts)
+    dq, dk, dv = empty(ctx, B, S, H, D), empty(ctx, B, S, H, D), empty(ctx, B, S, H, D)
+    eng.flash_attention_v2_backward_with_stats(ctx, tq, tk, tv, out, tdo, dq, dk, dv, stats, opts)
+    n = B * S * H * D
+    odd = [UnifiedTensor.zeros(ctx, [n + 1]) for _ in range(3)]
+    o = opts.c()
+    check(lib.ft_flash_attention_v2_backward_with_stats(
+        ctx.handle, C.c_void_p(tq.ptr), C.c_void_p(tk.ptr), C.c_void_p(tv.ptr), C.c_void_p(out.ptr),
+        C.c_void_p(tdo.ptr), C.c_void_p(odd[0].ptr + 4), C.c_void_p(odd[1].ptr + 4), C.c_void_p(odd[2].ptr + 4),
+        C.c_void_p(stats.ptr), B, S, S, H, H, D, C.byref(o)))
+    for name, a, b in (("dq", dq, odd[0]), ("dk", dk, odd[1]), ("dv", dv, odd[2])):
+        got = b.to_numpy()
+        assert got[0] == 0.0
+        assert_close(name + " at an odd offset", got[1:], a.to_numpy().reshape(-1), atol=2e-5)
