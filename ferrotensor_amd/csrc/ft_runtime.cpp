@@ -235,8 +235,9 @@ int ft_pool_stats(ft_context* ctx, size_t* live_bytes, size_t* idle_bytes) {
 int ft_upload(ft_context* ctx, void* dst_dev, const void* src_host, size_t bytes) {
     FT_CHECK_ARG(ctx && (bytes == 0 || (dst_dev && src_host)), "ft_upload: NULL argument");
     if (bytes == 0) return FT_OK;
-    // Pageable source: hipMemcpyAsync stages it before returning, so the
-    // caller may reuse src immediately (as with wgpu's write_buffer).
+    // Blocks until the copy is done, so the caller may reuse src at once (as with wgpu's
+    // write_buffer). The step driver does not come through here: it stages a chunk's arrays in
+    // pinned memory and sends them in one asynchronous copy.
     FT_HIP(hipMemcpyAsync(dst_dev, src_host, bytes, hipMemcpyHostToDevice, ctx->stream));
     FT_HIP(hipStreamSynchronize(ctx->stream));
     return FT_OK;

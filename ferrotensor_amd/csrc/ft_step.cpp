@@ -16,8 +16,9 @@
 //
 // The reference records a tape and walks it; the step's graph is static, so
 // forward and backward are written out here and every buffer is allocated once
-// per (batch, sequence) shape and kept. Nothing in the step waits for the GPU
-// until the per-row losses and the gradient norm are read back at its end.
+// per (batch, sequence) shape and kept. A chunk's host arrays go up in one copy
+// from pinned memory before the first kernel, and nothing waits for the GPU until
+// the per-row losses and the gradient norm come back in one copy at its end.
 #include "ft_common.h"
 #include "ft_thin.h"
 
@@ -114,8 +115,14 @@ struct ft_model {
     std::vector<void*> ws_allocs;
     std::vector<LayerActs> acts;
     float *x_final = nullptr, *hf = nullptr, *thead = nullptr, *logits = nullptr;
+    // Everything a chunk sends to the device (token ids, head row indices both ways, targets, row
+    // weights: 5 arrays of T words) is written into one pinned staging buffer and goes up in one
+    // copy before the first kernel; the per-row losses and the trainer's control block (3 words at
+    // step_out + T) come back in one copy into pinned memory at the end: the step's only wait.
+    uint32_t *io_host = nullptr, *io_dev = nullptr;
+    float *out_host = nullptr, *step_out = nullptr;
     uint32_t *ids_dev = nullptr, *targets_dev = nullptr;
-    float *weights_dev = nullptr, *row_loss = nullptr;
+    float *weights_dev = nullptr, *row_loss = nullptr, *control = nullptr;
     // Head on the supervised rows only: head_idx[k] = k-th supervised row, head_inv[row] = its k
     // (or head_rows for an unsupervised row, which gathers as a zero row), xc = those rows of x_final.
     uint32_t *head_idx_dev = nullptr, *head_inv_dev = nullptr;
@@ -150,7 +157,6 @@ struct ft_trainer {
     ft_segment* segs_dev = nullptr;
     size_t nseg = 0;
     float* partials = nullptr;
-    float* control = nullptr;       // {grad_norm, clip_scale, apply}
 };
 
 namespace {
@@ -166,6 +172,12 @@ int ws_alloc(ft_model* m, size_t n, float** out) {
 void ws_free(ft_model* m) {
     for (void* p : m->ws_allocs) (void)ft_free(m->ctx, p);
     m->ws_allocs.clear();
+    if (m->io_host) (void)hipHostFree(m->io_host);
+    if (m->out_host) (void)hipHostFree(m->out_host);
+    m->io_host = nullptr;
+    m->out_host = nullptr;
+    m->control = nullptr;
+    m->step_out = nullptr;
     m->acts.clear();
     m->ws_B = m->ws_S = 0;
 }
@@ -222,12 +234,17 @@ int ensure_workspace(ft_model* m, size_t B, size_t S) {
     m->thead = nullptr;
     if (m->lm_head.has_lora()) FT_TRY(ws_alloc(m, T * m->lm_head.r, &m->thead));
     FT_TRY(ws_alloc(m, T * V, &m->logits));
-    FT_TRY(ws_alloc(m, T, (float**)&m->ids_dev));
-    FT_TRY(ws_alloc(m, T, (float**)&m->targets_dev));
-    FT_TRY(ws_alloc(m, T, &m->weights_dev));
-    FT_TRY(ws_alloc(m, T, &m->row_loss));
-    FT_TRY(ws_alloc(m, T, (float**)&m->head_idx_dev));
-    FT_TRY(ws_alloc(m, T, (float**)&m->head_inv_dev));
+    FT_TRY(ws_alloc(m, 5 * T, (float**)&m->io_dev));
+    m->ids_dev = m->io_dev;
+    m->head_idx_dev = m->io_dev + T;
+    m->head_inv_dev = m->io_dev + 2 * T;
+    m->targets_dev = m->io_dev + 3 * T;
+    m->weights_dev = reinterpret_cast<float*>(m->io_dev + 4 * T);
+    FT_TRY(ws_alloc(m, T + 4, &m->step_out));
+    m->row_loss = m->step_out;
+    m->control = m->step_out + T;
+    FT_HIP(hipHostMalloc((void**)&m->io_host, 5 * T * sizeof(uint32_t), hipHostMallocDefault));
+    FT_HIP(hipHostMalloc((void**)&m->out_host, (T + 4) * sizeof(float), hipHostMallocDefault));
     FT_TRY(ws_alloc(m, T * H, &m->xc));
     FT_TRY(ws_alloc(m, T * H, &m->g0));
     FT_TRY(ws_alloc(m, T * H, &m->g1));
@@ -507,12 +524,15 @@ int layer_forward(ft_model* m, size_t l, size_t B, size_t S) {
     return FT_OK;
 }
 
-// `head` (optional): the rows whose logits are needed, ascending. The final norm and the
-// vocabulary head then run on those rows only (logits, row losses and d_logits are [head->size(), V]):
-// a row without a supervised target has zero loss and a zero logits gradient whatever its logits are
-// (masked_cross_entropy, kernels.wgsl:684-711), so leaving it out changes no bit of the result.
-int model_forward(ft_model* m, const uint32_t* rows_host, size_t B, size_t S,
-                  const std::vector<uint32_t>* head = nullptr) {
+// Stages a chunk's host arrays and sends them to the device in one copy.
+// `head` (optional): the rows whose logits are needed, ascending, with their targets and weights.
+// The final norm and the vocabulary head then run on those rows only (logits, row losses and
+// d_logits are [head->size(), V]): a row without a supervised target has zero loss and a zero
+// logits gradient whatever its logits are (masked_cross_entropy, kernels.wgsl:684-711), so leaving
+// it out changes no bit of the result. With `head_all_rows` (or no `head`) every row goes through
+// the head, unsupervised ones with MASKED_CE_SKIP and weight 0.
+int stage_chunk(ft_model* m, const uint32_t* rows_host, size_t B, size_t S, const std::vector<uint32_t>* head,
+                const std::vector<uint32_t>* tg, const std::vector<float>* wt) {
     ft_context* ctx = m->ctx;
     const ft_model_config& c = m->cfg;
     FT_CHECK_ARG(m->embed && m->norm_f && m->lm_head.w, "model is missing embed_tokens, norm or lm_head weights");
@@ -525,22 +545,50 @@ int model_forward(ft_model* m, const uint32_t* rows_host, size_t B, size_t S,
         ws_free(m);
     }
     FT_TRY(ensure_workspace(m, B, S));
-    const size_t T = B * S, H = c.hidden_size;
-    FT_TRY(ft_upload(ctx, m->ids_dev, rows_host, T * sizeof(uint32_t)));
-    FT_TRY(ft_embedding(ctx, m->embed, c.vocab_size, H, m->ids_dev, T, m->acts.empty() ? m->x_final : m->acts[0].x));
-    for (size_t l = 0; l < m->layers.size(); l++) FT_TRY(layer_forward(m, l, B, S));
-    const float* xf = m->x_final;
+    const size_t T = B * S;
+    uint32_t* ids = m->io_host;
+    uint32_t* idx = ids + T;
+    uint32_t* inv = ids + 2 * T;
+    uint32_t* tgs = ids + 3 * T;
+    float* wts = reinterpret_cast<float*>(ids + 4 * T);
+    std::memcpy(ids, rows_host, T * sizeof(uint32_t));
     m->head_rows = T;
     m->head_compact = head != nullptr && head->size() < T && !c.head_all_rows;
     if (m->head_compact) {
         m->head_rows = head->size();
-        std::vector<uint32_t> inv(T, (uint32_t)head->size());
+        for (size_t r = 0; r < T; r++) inv[r] = (uint32_t)head->size();
         for (size_t k = 0; k < head->size(); k++) {
             FT_CHECK_ARG((*head)[k] < T && (k == 0 || (*head)[k] > (*head)[k - 1]), "head rows must ascend within the chunk");
+            idx[k] = (*head)[k];
             inv[(*head)[k]] = (uint32_t)k;
+            tgs[k] = (*tg)[k];
+            wts[k] = (*wt)[k];
         }
-        FT_TRY(ft_upload(ctx, m->head_idx_dev, head->data(), head->size() * sizeof(uint32_t)));
-        FT_TRY(ft_upload(ctx, m->head_inv_dev, inv.data(), T * sizeof(uint32_t)));
+    } else {
+        for (size_t r = 0; r < T; r++) {
+            tgs[r] = FT_MASKED_CE_SKIP;
+            wts[r] = 0.0f;
+        }
+        if (head)
+            for (size_t k = 0; k < head->size(); k++) {
+                FT_CHECK_ARG((*head)[k] < T, "head rows must lie within the chunk");
+                tgs[(*head)[k]] = (*tg)[k];
+                wts[(*head)[k]] = (*wt)[k];
+            }
+    }
+    FT_HIP(hipMemcpyAsync(m->io_dev, m->io_host, 5 * T * sizeof(uint32_t), hipMemcpyHostToDevice, ctx->stream));
+    return FT_OK;
+}
+
+// Forward over the staged chunk: embedding, blocks, and the head on m->head_rows rows.
+int model_forward(ft_model* m, size_t B, size_t S) {
+    ft_context* ctx = m->ctx;
+    const ft_model_config& c = m->cfg;
+    const size_t T = B * S, H = c.hidden_size;
+    FT_TRY(ft_embedding(ctx, m->embed, c.vocab_size, H, m->ids_dev, T, m->acts.empty() ? m->x_final : m->acts[0].x));
+    for (size_t l = 0; l < m->layers.size(); l++) FT_TRY(layer_forward(m, l, B, S));
+    const float* xf = m->x_final;
+    if (m->head_compact) {
         // gather: row k of xc = row head[k] of x_final
         FT_TRY(ft_embedding(ctx, m->x_final, T, H, m->head_idx_dev, m->head_rows, m->xc));
         xf = m->xc;
@@ -548,6 +596,14 @@ int model_forward(ft_model* m, const uint32_t* rows_host, size_t B, size_t S,
     if (m->head_rows == 0) return FT_OK;
     FT_TRY(ft_rms_norm_eps(ctx, xf, m->norm_f, m->hf, m->head_rows, H, c.rms_norm_eps));
     FT_TRY(linear_forward(ctx, m->lm_head, m->hf, m->thead, m->logits, m->head_rows));
+    return FT_OK;
+}
+
+// Brings the row losses and the control block to the host (one copy, then the stream is idle).
+int fetch_step_out(ft_model* m) {
+    const size_t T = m->ws_B * m->ws_S;
+    FT_HIP(hipMemcpyAsync(m->out_host, m->step_out, (T + 4) * sizeof(float), hipMemcpyDeviceToHost, m->ctx->stream));
+    FT_HIP(hipStreamSynchronize(m->ctx->stream));
     return FT_OK;
 }
 
@@ -903,7 +959,8 @@ int ft_model_read_grad(ft_model* m, size_t index, float* out_host) {
 int ft_model_forward_logits(ft_model* m, const uint32_t* rows, size_t B, size_t S, float* logits_host) {
     return guarded([&]() -> int {
         FT_CHECK_ARG(m && rows && logits_host && B > 0 && S > 0, "ft_model_forward_logits: bad argument");
-        FT_TRY(model_forward(m, rows, B, S));
+        FT_TRY(stage_chunk(m, rows, B, S, nullptr, nullptr, nullptr));
+        FT_TRY(model_forward(m, B, S));
         return ft_download(m->ctx, logits_host, m->logits, B * S * m->cfg.vocab_size * sizeof(float));
     });
 }
@@ -940,7 +997,6 @@ int ft_trainer_create(ft_model* m, const ft_trainer_config* cfg, ft_trainer** ou
         FT_TRY(ft_alloc(ctx, segs.size() * sizeof(ft_segment), (void**)&t->segs_dev));
         FT_TRY(ft_upload(ctx, t->segs_dev, segs.data(), segs.size() * sizeof(ft_segment)));
         FT_TRY(alloc_f(ctx, segs.size(), &t->partials));
-        FT_TRY(alloc_f(ctx, 4, &t->control));
         *out = t.release();
         return FT_OK;
     });
@@ -953,7 +1009,6 @@ int ft_trainer_destroy(ft_trainer* t) {
     for (float* p : t->v) (void)ft_free(ctx, p);
     if (t->segs_dev) (void)ft_free(ctx, t->segs_dev);
     if (t->partials) (void)ft_free(ctx, t->partials);
-    if (t->control) (void)ft_free(ctx, t->control);
     delete t;
     return FT_OK;
 }
@@ -989,35 +1044,11 @@ size_t build_targets(const uint32_t* targets, const uint8_t* loss_mask, size_t B
     return total;
 }
 
-// Targets and weights of the rows the head ran on in the last forward (the supervised rows, or all
-// T rows with MASKED_CE_SKIP / 0 in between) to the device; returns how many rows that is.
-int upload_targets(ft_model* m, size_t T, const std::vector<uint32_t>& tg, const std::vector<float>& wt,
-                   const std::vector<uint32_t>& head, size_t* rows_out) {
-    if (m->head_compact) {
-        FT_TRY(ft_upload(m->ctx, m->targets_dev, tg.data(), tg.size() * sizeof(uint32_t)));
-        FT_TRY(ft_upload(m->ctx, m->weights_dev, wt.data(), wt.size() * sizeof(float)));
-        *rows_out = tg.size();
-        return FT_OK;
-    }
-    std::vector<uint32_t> tg_all(T, FT_MASKED_CE_SKIP);
-    std::vector<float> wt_all(T, 0.0f);
-    for (size_t k = 0; k < head.size(); k++) {
-        tg_all[head[k]] = tg[k];
-        wt_all[head[k]] = wt[k];
-    }
-    FT_TRY(ft_upload(m->ctx, m->targets_dev, tg_all.data(), T * sizeof(uint32_t)));
-    FT_TRY(ft_upload(m->ctx, m->weights_dev, wt_all.data(), T * sizeof(float)));
-    *rows_out = T;
-    return FT_OK;
-}
-
 // Per-sequence mean losses from the device row losses of the head rows (f64 sums in row order, as the
 // reference's host code; the rows left out are the ones that would add 0).
 int read_sequence_losses(ft_model* m, size_t B, size_t S, const std::vector<size_t>& tokens,
                          const std::vector<uint32_t>& head, float* per_sequence, float* total_out) {
-    const size_t rows = m->head_compact ? head.size() : B * S;
-    std::vector<float> losses(rows);
-    FT_TRY(ft_download(m->ctx, losses.data(), m->row_loss, rows * sizeof(float)));
+    const float* losses = m->out_host;   // filled by fetch_step_out
     std::vector<double> sums(B, 0.0);
     for (size_t k = 0; k < head.size(); k++) sums[head[k] / S] += (double)losses[m->head_compact ? k : head[k]];
     float total = 0.0f;
@@ -1051,12 +1082,12 @@ int ft_model_eval_chunk(ft_model* m, const uint32_t* rows, const uint32_t* targe
             per_sequence_loss[s] = 0.0f;
         }
         if (total == 0) return FT_OK;
-        FT_TRY(model_forward(m, rows, B, S, &head));
-        size_t ce_rows = 0;
-        FT_TRY(upload_targets(m, B * S, tg, wt, head, &ce_rows));
+        FT_TRY(stage_chunk(m, rows, B, S, &head, &tg, &wt));
+        FT_TRY(model_forward(m, B, S));
         // forward only: the gradient the kernel writes (in place of the logits) is discarded
         FT_TRY(ft_masked_cross_entropy_weighted(m->ctx, m->logits, m->targets_dev, m->weights_dev, m->logits,
-                                                m->row_loss, ce_rows, V, 1.0f));
+                                                m->row_loss, m->head_rows, V, 1.0f));
+        FT_TRY(fetch_step_out(m));
         return read_sequence_losses(m, B, S, tokens, head, per_sequence_loss, nullptr);
     });
 }
@@ -1160,15 +1191,14 @@ int ft_trainer_train_chunk(ft_trainer* t, const uint32_t* rows, const uint32_t* 
             if (per_sequence_loss)
                 for (size_t s = 0; s < B; s++) per_sequence_loss[s] = 0.0f;
         } else {
-            FT_TRY(model_forward(m, rows, B, S, &head));
-            size_t ce_rows = 0;
-            FT_TRY(upload_targets(m, T, tg, wt, head, &ce_rows));
+            FT_TRY(stage_chunk(m, rows, B, S, &head, &tg, &wt));
+            FT_TRY(model_forward(m, B, S));
             // Loss + d loss / d logits in place, with the backward seed
             // 1 / grad_accum_steps folded in (trainer/src/lib.rs:474-480, 553-572).
             const float seed = 1.0f / (float)accum;
             const float gscale = std::fabs(seed - 1.0f) > kF32Epsilon ? seed : 1.0f;
             FT_TRY(ft_masked_cross_entropy_weighted(ctx, m->logits, m->targets_dev, m->weights_dev, m->logits,
-                                                    m->row_loss, ce_rows, V, gscale));
+                                                    m->row_loss, m->head_rows, V, gscale));
             // The first backward of a window overwrites the gradient buffers (the reference's
             // zero_grad after every optimizer step); later ones add to them.
             FT_TRY(model_backward(m, B, S, t->window_has_grads));
@@ -1189,20 +1219,21 @@ int ft_trainer_train_chunk(ft_trainer* t, const uint32_t* rows, const uint32_t* 
             t->step_in_accum = 0;
             t->window_has_grads = false;
             if (have_grads) {
+                FT_CHECK_ARG(m->control, "ft_trainer_train_chunk: gradients without a workspace");
                 FT_TRY(ft_internal_multi_grad_norm(ctx, t->segs_dev, t->nseg, t->partials, t->cfg.clip_grad_norm,
-                                                   t->control));
+                                                   m->control));
                 if (apply) {
-                    FT_TRY(ft_internal_multi_adamw(ctx, t->segs_dev, t->nseg, &ap, 1.0f, t->control));
+                    FT_TRY(ft_internal_multi_adamw(ctx, t->segs_dev, t->nseg, &ap, 1.0f, m->control));
                     launched_update = true;
                 }
             }
         }
 
-        // The step's only wait: row losses and the control block.
+        // The step's only wait: row losses and the control block, in one copy.
+        if (total_tokens > 0 || (window_full && have_grads)) FT_TRY(fetch_step_out(m));
         if (total_tokens > 0) FT_TRY(read_sequence_losses(m, B, S, tokens, head, per_sequence_loss, &stats->loss));
         if (window_full && have_grads) {
-            float control[3];
-            FT_TRY(ft_download(ctx, control, t->control, sizeof(control)));
+            const float* control = m->out_host + m->ws_B * m->ws_S;
             int applied;
             std::memcpy(&applied, &control[2], 4);
             stats->grad_norm = control[0];
