@@ -107,16 +107,33 @@ def lora_factors(model, w, seed=2):
 
 
 def step_flops(w, head_rows=None):
-    """Algorithmic flops of one step: `2 M N K` for the forward and input-gradient GEMMs on the
-    frozen base incl. the head, LoRA products, attention fwd + 2.5x bwd. The head
-    (and its input gradient) runs on `head_rows` rows: the supervised positions."""
+    """Algorithmic flops of one step, exactly the products that run: `2 M N K` for every forward GEMM on the
+    frozen base and every input-gradient GEMM (the first block's q/k/v have none: their input is the frozen
+    embedding), the head and its input gradient on `head_rows` rows (the supervised positions), the rank-r
+    products of every adapter (forward x@A, t@B; backward dT, dT@A^T, dA, dB), attention forward + 2.5x
+    backward (causal: 2 B H S^2 D forward)."""
     T = w["B"] * w["S"]
-    H, F, V, L = w["hidden"], w["ffn"], w["vocab"], w["layers"]
+    H, F, V, L, r = w["hidden"], w["ffn"], w["vocab"], w["layers"], w["rank"]
     D = H // w["heads"]
-    p_layer = H * w["heads"] * D * 2 + H * w["kv"] * D * 2 + 3 * H * F
+    dims = {"q_proj": (H, w["heads"] * D), "k_proj": (H, w["kv"] * D), "v_proj": (H, w["kv"] * D),
+            "o_proj": (w["heads"] * D, H), "gate_proj": (H, F), "up_proj": (H, F), "down_proj": (F, H)}
     head_rows = T if head_rows is None else head_rows
-    attn = 2.0 * w["B"] * w["heads"] * w["S"] ** 2 * D * 3.5 * L
-    return 2 * (2.0 * T * L * p_layer + 2.0 * head_rows * H * V) + attn
+    total = 2 * 2.0 * head_rows * H * V
+    for layer in range(L):
+        for name, (i, o) in dims.items():
+            dx = not (layer == 0 and name in ("q_proj", "k_proj", "v_proj"))
+            total += 2.0 * T * i * o * (2 if dx else 1)
+            if name in w["targets"]:
+                total += 2.0 * T * r * (i + o) * (3 if dx else 2)
+                if not dx:
+                    total += 2.0 * T * r * o   # dT is still needed for dA
+    total += 2.0 * w["B"] * w["heads"] * w["S"] ** 2 * D * 3.5 * L
+    if w.get("checkpoint"):
+        # every block but the last is run forward a second time before its backward
+        for name, (i, o) in dims.items():
+            total += (L - 1) * (2.0 * T * i * o + (2.0 * T * r * (i + o) if name in w["targets"] else 0.0))
+        total += 2.0 * w["B"] * w["heads"] * w["S"] ** 2 * D * (L - 1)
+    return total
 
 
 def read_profile(ctx):
@@ -136,9 +153,10 @@ def read_profile(ctx):
     return sorted(out, key=lambda r: -r["ms"])
 
 
-def cpu_baseline(w, seconds_budget=30.0):
-    """The CPU oracle on this host, on ONE of the B sequences (full depth, full
-    vocabulary): a bounded sample of the same workload, scaled to tokens/s."""
+def cpu_baseline(w, seconds_budget=45.0):
+    """The CPU oracle on this host: the same step on the same batch. One sequence is timed first; when the
+    whole batch fits the budget it is timed too (median of up to 3 steps) and that is what is reported,
+    otherwise the one-sequence figure (a bounded sample of the same workload, stated in `sample`)."""
     from oracle import cpu
     from oracle import reference_step as rs
     cfg = rs.ModelConfig(w["vocab"], w["hidden"], w["ffn"], w["layers"], w["heads"], w["kv"], 1e-5, 100000.0, True)
@@ -151,20 +169,25 @@ def cpu_baseline(w, seconds_budget=30.0):
             i, o = lin.weight.shape
             model.set_lora(name, rng.standard_normal((i, w["rank"]), dtype=np.float32) * np.float32(0.02),
                            rng.standard_normal((w["rank"], o), dtype=np.float32) * np.float32(0.02), w["alpha"])
-    rows, targets, masks = synthetic_batch(w, B=1)
+    rows, targets, masks = synthetic_batch(w)
     opt = rs.AdamW(lr=2e-4, weight_decay=0.0)
-    times = []
-    t_all = time.perf_counter()
-    for _ in range(3):
+
+    def timed(n):
         t0 = time.perf_counter()
-        rs.train_chunk(model, opt, rows, targets, masks, grad_accum_steps=w["B"], clip_grad_norm=1.0)
-        times.append(time.perf_counter() - t0)
-        if time.perf_counter() - t_all > seconds_budget:
-            break
+        rs.train_chunk(model, opt, rows[:n], targets[:n], masks[:n], grad_accum_steps=w["B"], clip_grad_norm=1.0)
+        return time.perf_counter() - t0
+
+    t_all = time.perf_counter()
+    one = timed(1)
+    n, times = 1, [one]
+    if one * w["B"] * 1.2 < seconds_budget:
+        n, times = w["B"], []
+        while len(times) < 3 and (not times or time.perf_counter() - t_all + times[-1] < seconds_budget):
+            times.append(timed(n))
     t = float(np.median(times))
-    return {"value": w["S"] / t, "unit": "tokens/s", "cores": cpu.num_threads(), "kind": "port",
-            "sample": "1 of the %d sequences (%d tokens), all %d layers + head, fwd+bwd+AdamW, median of %d steps, "
-                      "%.2f s/step, %d OpenMP threads" % (w["B"], w["S"], w["layers"], len(times), t,
+    return {"value": n * w["S"] / t, "unit": "tokens/s", "cores": cpu.num_threads(), "kind": "port",
+            "sample": "%d of the %d sequences (%d tokens), all %d layers + head, fwd+bwd+AdamW, median of %d steps, "
+                      "%.2f s/step, %d OpenMP threads" % (n, w["B"], n * w["S"], w["layers"], len(times), t,
                                                           cpu.num_threads())}
 
 
@@ -174,12 +197,40 @@ FETCH_SIZE_FACTOR = 16384.0 / 8203.5
 WRITE_SIZE_FACTOR = 1.0
 
 
+def source_hash():
+    """Hash of the library's sources: names the build a stored profile was taken from."""
+    import hashlib
+    h = hashlib.sha256()
+    src = os.path.join(ROOT, "ferrotensor_amd", "csrc")
+    for name in sorted(os.listdir(src)) + ["../../include/ferrotensor_hip.h"]:
+        with open(os.path.join(src, name), "rb") as f:
+            h.update(name.encode() + b"\0" + f.read())
+    return h.hexdigest()[:16]
+
+
+TRAFFIC_PROFILE = os.path.join("profiles", "lora_step_360m_hbm_traffic.md")
+
+
+def traffic_source():
+    """Where `roofline.traffic` comes from: hardware counters cannot be read from inside this process, so the
+    figure is the one the rocprofv3 --pmc runs of this same command recorded under profiles/. The profile
+    names the source hash of the library it was taken from; `current` says whether that is this build."""
+    recorded = None
+    try:
+        for line in open(os.path.join(ROOT, TRAFFIC_PROFILE)):
+            if line.startswith("Library source hash:"):
+                recorded = line.split(":", 1)[1].strip().strip("`")
+    except OSError:
+        pass
+    return {"file": TRAFFIC_PROFILE, "library_source_hash": recorded, "current": recorded == source_hash()}
+
+
 def measured_traffic(kernel, workload):
     """HBM-side bytes per launch of `kernel` (calibrated FETCH_SIZE + WRITE_SIZE, KiB per dispatch) as recorded
     by the rocprofv3 --pmc runs summarised under profiles/; None when there is no record for this kernel."""
     if workload != "360m":
         return None
-    path = os.path.join(ROOT, "profiles", "lora_step_360m_hbm_traffic.md")
+    path = os.path.join(ROOT, TRAFFIC_PROFILE)
     # profile names -> kernel symbols: <.., layout, segments[, epilogue[, wave groups]]>
     name = kernel
     for tag, code in (("gate_up", "1, 1"), ("silu_bwd", "2, 1")):
@@ -386,6 +437,18 @@ def main():
     if not (np.isfinite(st.loss) and st.optimizer_step):
         sys.exit("bench.py: the step did not produce a finite loss / optimizer step: %r" % (st,))
 
+    # The same steps with the head on every position, as the reference runs it (same results, more work).
+    model.set_head_all_rows(True)
+    one_step()
+    ctx.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        one_step()
+    ctx.synchronize()
+    ms_all_rows = (time.perf_counter() - t0) / args.steps * 1e3
+    model.set_head_all_rows(False)
+    one_step()
+
     # Per-kernel HIP-event timing over the same number of identical steps.
     from ferrotensor_amd._lib import check
     check(ctx._lib.ft_profile_begin(ctx.handle))
@@ -418,12 +481,14 @@ def main():
                    "base_weights": "f16 storage, f32 arithmetic", "optimizer": "AdamW lr 2e-4 wd 0 clip 1.0",
                    "supervised_tokens": int(st.tokens), "loss": float(st.loss),
                    "head": "final norm, vocabulary head and loss on the %d supervised positions" % int(st.tokens)},
+        "ms_per_step_head_all_rows": ms_all_rows, "tokens_per_s_head_all_rows": tokens / (ms_all_rows * 1e-3),
         "supervised_tokens_per_s": int(st.tokens) / (elapsed / args.steps),
         "step_tflops": step_flops(w, int(st.tokens)) / (elapsed / args.steps) / 1e12,
         "step_mfma_frac": step_flops(w, int(st.tokens)) / (elapsed / args.steps) / 1e12 / FP32_MFMA_PEAK_TFLOPS,
         "roofline": {"bound": "mfma", "kernel": dom["name"], "achieved": achieved, "peak": FP32_MFMA_PEAK_TFLOPS,
                      "unit": "TFLOP/s", "frac": achieved / FP32_MFMA_PEAK_TFLOPS,
                      "traffic": measured_traffic(dom["name"], args.workload),
+                     "traffic_source": traffic_source() if args.workload == "360m" else None,
                      "launches_per_step": dom["launches"] // args.steps,
                      "avg_launch_us": dom["ms"] * 1e3 / dom["launches"],
                      "all_gemm_kernels_tflops": all_gemm_tf,

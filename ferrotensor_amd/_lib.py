@@ -41,7 +41,7 @@ class ModelConfigC(C.Structure):
                 ("num_hidden_layers", C.c_uint32), ("num_attention_heads", C.c_uint32),
                 ("num_key_value_heads", C.c_uint32), ("rms_norm_eps", C.c_float), ("rope_theta", C.c_float),
                 ("tie_word_embeddings", C.c_int32), ("f16_linears", C.c_int32), ("checkpoint_blocks", C.c_int32),
-                ("head_all_rows", C.c_int32)]
+                ("head_all_rows", C.c_int32), ("trainable_base", C.c_int32)]
 
 
 class TrainerConfigC(C.Structure):
@@ -147,6 +147,7 @@ SIGNATURES = {
     "ft_lora_seed": [C.c_uint64, C.c_char_p],
     "ft_lora_init_a": [_P, _SZ, _SZ, _SZ, C.c_uint64],
     "ft_model_add_lora": [_P, C.c_char_p, _SZ, _F],
+    "ft_model_set_head_all_rows": [_P, _I],
     "ft_lr_schedule": [C.c_uint32, _F, _F, C.c_uint32, C.c_uint32, C.c_uint32],
     "ft_trainer_train_chunk": [_P, _P, _P, _P, _SZ, _SZ, _I, C.POINTER(StepStatsC), _P],
 }

@@ -67,6 +67,7 @@ struct LinearW {
     float* b = nullptr;   // [r, out]
     float* ga = nullptr;
     float* gb = nullptr;
+    float* gw = nullptr;  // gradient of w [in, out] when the base trains
     bool has_lora() const { return r > 0; }
     // graph/src/lib.rs:119-122: the scale is alpha / rank, skipped when it is exactly 1.
     float scale() const {
@@ -78,6 +79,8 @@ struct LinearW {
 struct Layer {
     float* norm1 = nullptr;
     float* norm2 = nullptr;
+    float* gnorm1 = nullptr;  // gradients of the norm scales when the base trains
+    float* gnorm2 = nullptr;
     LinearW q, k, v, o, gate, up, down;
     LinearW* all[7] = {&q, &k, &v, &o, &gate, &up, &down};
 };
@@ -103,6 +106,7 @@ struct ft_model {
     float* embed = nullptr;
     std::vector<Layer> layers;
     float* norm_f = nullptr;
+    float* gnorm_f = nullptr;
     LinearW lm_head;
     std::vector<ParamRef> params;
     bool params_dirty = true;
@@ -277,17 +281,44 @@ int ensure_workspace(ft_model* m, size_t B, size_t S) {
     return FT_OK;
 }
 
-void rebuild_params(ft_model* m) {
+// The trainable tensors in reporting order. With a trainable base (model_builder.rs:353-357) the
+// linear weights and the norm scales are in it too, and their gradient buffers are made here.
+int rebuild_params(ft_model* m) {
     m->params.clear();
-    auto add = [&](LinearW& l) {
-        if (!l.has_lora()) return;
+    const bool base = m->cfg.trainable_base != 0;
+    const size_t H = m->cfg.hidden_size;
+    auto grad_buf = [&](float** g, size_t n) -> int {
+        if (*g) return FT_OK;
+        FT_TRY(alloc_f(m->ctx, n, g));
+        return ft_zero(m->ctx, *g, n * 4);
+    };
+    auto add_norm = [&](const std::string& name, float* w, float** g) -> int {
+        if (!base || !w) return FT_OK;
+        FT_TRY(grad_buf(g, H));
+        m->params.push_back({name, w, *g, H});
+        return FT_OK;
+    };
+    auto add = [&](LinearW& l) -> int {
+        if (base && l.w && l.dtype == FT_DTYPE_F32) {
+            FT_TRY(grad_buf(&l.gw, l.in * l.out));
+            m->params.push_back({l.prefix + ".weight", (float*)l.w, l.gw, l.in * l.out});
+        }
+        if (!l.has_lora()) return FT_OK;
         m->params.push_back({l.prefix + ".lora_a", l.a, l.ga, l.in * l.r});
         m->params.push_back({l.prefix + ".lora_b", l.b, l.gb, l.r * l.out});
+        return FT_OK;
     };
-    for (auto& L : m->layers)
-        for (auto* l : L.all) add(*l);
-    add(m->lm_head);
+    for (size_t li = 0; li < m->layers.size(); li++) {
+        Layer& L = m->layers[li];
+        const std::string p = "model.layers." + std::to_string(li);
+        FT_TRY(add_norm(p + ".input_layernorm.weight", L.norm1, &L.gnorm1));
+        for (auto* l : L.all) FT_TRY(add(*l));
+        FT_TRY(add_norm(p + ".post_attention_layernorm.weight", L.norm2, &L.gnorm2));
+    }
+    FT_TRY(add_norm("model.norm.weight", m->norm_f, &m->gnorm_f));
+    FT_TRY(add(m->lm_head));
     m->params_dirty = false;
+    return FT_OK;
 }
 
 // t_i = scale_i * x @ A_i for up to 3 linears that read the same x: one
@@ -375,6 +406,12 @@ int take_dt(ft_model* m, float** dt) {
 int linear_backward(ft_model* m, LinearW& l, const float* x, const float* t, const float* dy, float* dx, size_t T,
                     bool accumulate, bool dx_add = false) {
     ft_context* ctx = m->ctx;
+    if (l.gw) {
+        // trainable base: dW[in, out] = x^T @ dy (MatMulNode::backward, autograd/src/lib.rs:280-287)
+        float* dst = accumulate ? m->gtmp : l.gw;
+        FT_TRY(ft_matmul_at(ctx, x, dy, dst, l.in, T, l.out));
+        if (accumulate) FT_TRY(ft_gradient_accumulate(ctx, l.gw, m->gtmp, l.in * l.out));
+    }
     if (l.has_lora()) {
         float* dt = nullptr;
         // room for this linear's two products first: a flush frees every dT buffer
@@ -419,7 +456,11 @@ int linear_backward_group(ft_model* m, LinearW* const* ls, const float* const* t
                           float* dx, int n, const float* x, size_t T, bool accumulate, bool flush) {
     ft_context* ctx = m->ctx;
     bool batch = n <= 3;
-    for (int i = 0; i < n; i++) batch = batch && ls[i]->has_lora() && ls[i]->r == ls[0]->r;
+    bool any_gw = false;
+    for (int i = 0; i < n; i++) {
+        batch = batch && ls[i]->has_lora() && ls[i]->r == ls[0]->r && !ls[i]->gw;
+        any_gw = any_gw || ls[i]->gw != nullptr;
+    }
     float* dts[3] = {nullptr, nullptr, nullptr};
     if (batch) {
         // room for this group's products and dT buffers first: a flush frees every dT buffer
@@ -442,7 +483,7 @@ int linear_backward_group(ft_model* m, LinearW* const* ls, const float* const* t
     if (!batch) {
         bool any_lora = false;
         for (int i = 0; i < n; i++) any_lora = any_lora || ls[i]->has_lora();
-        if (any_lora || n > 3) {
+        if (any_lora || any_gw || n > 3) {
             for (int i = 0; i < n; i++)
                 FT_TRY(linear_backward(m, *ls[i], x, ts[i], dys[i], dx, T, accumulate, i > 0));
             if (flush) FT_TRY(flush_cols(m));
@@ -541,7 +582,7 @@ int stage_chunk(ft_model* m, const uint32_t* rows_host, size_t B, size_t S, cons
         for (auto* l : L.all) FT_CHECK_ARG(l->w, "linear %s has no weight", l->prefix.c_str());
     }
     if (m->params_dirty) {
-        rebuild_params(m);
+        FT_TRY(rebuild_params(m));
         ws_free(m);
     }
     FT_TRY(ensure_workspace(m, B, S));
@@ -607,7 +648,27 @@ int fetch_step_out(ft_model* m) {
     return FT_OK;
 }
 
-// Backward from d_logits (in m->logits) to every LoRA gradient.
+// gx = rms_norm_backward(x, w, g) (+ add). With a trainable norm scale (`gw`) its gradient is
+// computed too (RMSNormNode::backward, autograd/src/lib.rs:575-595), added to the earlier
+// micro-batches' when `accumulate`; `tmp` [rows, H] is scratch for that unfused form and must not
+// alias x, g or add.
+int norm_backward(ft_model* m, const float* x, const float* w, float* gw, const float* g, const float* add,
+                  float* gx, float* tmp, size_t rows, bool accumulate) {
+    ft_context* ctx = m->ctx;
+    const size_t H = m->cfg.hidden_size;
+    const float eps = m->cfg.rms_norm_eps;
+    if (!gw) {
+        if (add) return ft_internal_rms_norm_backward_add(ctx, x, w, g, add, gx, rows, H, eps);
+        return ft_rms_norm_backward(ctx, x, w, g, gx, nullptr, rows, H, eps);
+    }
+    float* out = add ? tmp : gx;
+    FT_TRY(ft_rms_norm_backward(ctx, x, w, g, out, accumulate ? m->gtmp : gw, rows, H, eps));
+    if (accumulate) FT_TRY(ft_gradient_accumulate(ctx, gw, m->gtmp, H));
+    if (add) FT_TRY(ft_add(ctx, add, tmp, gx, rows * H));
+    return FT_OK;
+}
+
+// Backward from d_logits (in m->logits) to the gradient of every trainable tensor.
 int model_backward(ft_model* m, size_t B, size_t S, bool accumulate) {
     ft_context* ctx = m->ctx;
     const ft_model_config& c = m->cfg;
@@ -621,11 +682,11 @@ int model_backward(ft_model* m, size_t B, size_t S, bool accumulate) {
     const size_t Th = m->head_rows;
     FT_TRY(linear_backward(m, m->lm_head, m->hf, m->thead, m->logits, m->d_h2, Th, accumulate));
     if (m->head_compact) {
-        FT_TRY(ft_rms_norm_backward(ctx, m->xc, m->norm_f, m->d_h2, g_other, nullptr, Th, H, c.rms_norm_eps));
+        FT_TRY(norm_backward(m, m->xc, m->norm_f, m->gnorm_f, m->d_h2, nullptr, g_other, nullptr, Th, accumulate));
         // scatter: row r of g = row head_inv[r] of the compact gradient, zero where the head did not run
         FT_TRY(ft_embedding(ctx, g_other, Th, H, m->head_inv_dev, T, g));
     } else {
-        FT_TRY(ft_rms_norm_backward(ctx, m->x_final, m->norm_f, m->d_h2, g, nullptr, T, H, c.rms_norm_eps));
+        FT_TRY(norm_backward(m, m->x_final, m->norm_f, m->gnorm_f, m->d_h2, nullptr, g, nullptr, T, accumulate));
     }
     for (size_t li = m->layers.size(); li-- > 0;) {
         Layer& L = m->layers[li];
@@ -639,7 +700,7 @@ int model_backward(ft_model* m, size_t B, size_t S, bool accumulate) {
             FT_TRY(layer_forward(m, li, B, S));
         }
         // x_next = h + down(silu(gate) * up)
-        if (!L.down.has_lora()) {
+        if (!L.down.has_lora() && !L.down.gw) {
             FT_TRY(ft_mlp_down_backward(ctx, g, L.down.w, L.down.dtype, a.gate, a.up, m->d_gate, m->d_up, m->d_act, T,
                                         F, H));
         } else {
@@ -653,7 +714,7 @@ int model_backward(ft_model* m, size_t B, size_t S, bool accumulate) {
             FT_TRY(linear_backward_group(m, ls, ts, dys, m->d_h2, 2, a.h2, T, accumulate, false));
         }
         // g_h = g + norm2_backward(d_h2) (into g_other)
-        FT_TRY(ft_internal_rms_norm_backward_add(ctx, a.h, L.norm2, m->d_h2, g, g_other, T, H, c.rms_norm_eps));
+        FT_TRY(norm_backward(m, a.h, L.norm2, L.gnorm2, m->d_h2, g, g_other, m->d_h1, T, accumulate));
         // h = x + o_proj(attn)
         FT_TRY(linear_backward(m, L.o, a.attn, a.to, g_other, m->d_attn, T, accumulate));
         if (m->rope_table &&
@@ -674,7 +735,8 @@ int model_backward(ft_model* m, size_t B, size_t S, bool accumulate) {
         // The first block's input is the frozen embedding: its norm output needs
         // no gradient, so the three input-gradient GEMMs are skipped
         // (MatMulNode::backward, autograd/src/lib.rs:268-287).
-        const bool need_dx = li > 0;
+        // A trainable input norm still needs its output's gradient for its own scale.
+        const bool need_dx = li > 0 || L.gnorm1 != nullptr;
         {
             LinearW* ls[3] = {&L.q, &L.k, &L.v};
             const float* ts[3] = {a.tq, a.tk, a.tv};
@@ -685,7 +747,7 @@ int model_backward(ft_model* m, size_t B, size_t S, bool accumulate) {
         }
         if (!need_dx) break;
         // g = g_h + norm1_backward(d_h1)
-        FT_TRY(ft_internal_rms_norm_backward_add(ctx, a.x, L.norm1, m->d_h1, g_other, g, T, H, c.rms_norm_eps));
+        FT_TRY(norm_backward(m, a.x, L.norm1, L.gnorm1, m->d_h1, g_other, g, m->d_h2, T, accumulate));
     }
     return flush_cols(m);
 }
@@ -701,8 +763,11 @@ LinearW* find_linear(ft_model* m, const std::string& prefix) {
 int set_linear_weight(ft_model* m, LinearW& l, const float* hf_out_in, size_t out, size_t in) {
     FT_CHECK_ARG(out == l.out && in == l.in, "%s.weight is [%zu, %zu], expected [%zu, %zu]", l.prefix.c_str(), out, in,
                  l.out, l.in);
-    const int dtype = m->cfg.f16_linears ? FT_DTYPE_F16 : FT_DTYPE_F32;
+    // upload_linear (model_builder.rs:325-340): f32 when the base trains, else f16 when asked
+    const int dtype = (m->cfg.f16_linears && !m->cfg.trainable_base) ? FT_DTYPE_F16 : FT_DTYPE_F32;
     if (!l.w) {
+        m->params_dirty = true;   // a new weight may be a new trainable tensor
+        m->param_generation++;
         size_t bytes = in * out * (dtype == FT_DTYPE_F16 ? 2 : 4);
         bytes = (bytes + 3) / 4 * 4;
         FT_TRY(ft_alloc(m->ctx, bytes, &l.w));
@@ -714,7 +779,11 @@ int set_linear_weight(ft_model* m, LinearW& l, const float* hf_out_in, size_t ou
 
 int set_vector(ft_model* m, float** slot, const float* data, size_t n, size_t want, const char* name) {
     FT_CHECK_ARG(n == want, "%s has %zu values, expected %zu", name, n, want);
-    if (!*slot) FT_TRY(alloc_f(m->ctx, n, slot));
+    if (!*slot) {
+        FT_TRY(alloc_f(m->ctx, n, slot));
+        m->params_dirty = true;   // with a trainable base a new norm scale is a new trainable tensor
+        m->param_generation++;
+    }
     return ft_upload(m->ctx, *slot, data, n * sizeof(float));
 }
 
@@ -787,12 +856,16 @@ int ft_model_destroy(ft_model* m) {
         rel(l.b);
         rel(l.ga);
         rel(l.gb);
+        rel(l.gw);
     };
     rel(m->embed);
     rel(m->norm_f);
+    rel(m->gnorm_f);
     for (auto& L : m->layers) {
         rel(L.norm1);
         rel(L.norm2);
+        rel(L.gnorm1);
+        rel(L.gnorm2);
         for (auto* l : L.all) rel_lin(*l);
     }
     rel_lin(m->lm_head);
@@ -920,11 +993,17 @@ int ft_model_add_lora(ft_model* m, const char* prefix, size_t rank, float alpha)
     });
 }
 
+int ft_model_set_head_all_rows(ft_model* m, int all_rows) {
+    FT_CHECK_ARG(m, "ft_model_set_head_all_rows: NULL argument");
+    m->cfg.head_all_rows = all_rows ? 1 : 0;
+    return FT_OK;
+}
+
 int ft_model_param_count(ft_model* m, size_t* count) {
     return guarded([&]() -> int {
         FT_CHECK_ARG(m && count, "ft_model_param_count: NULL argument");
         if (m->params_dirty) {
-            rebuild_params(m);
+            FT_TRY(rebuild_params(m));
             ws_free(m);
         }
         *count = m->params.size();
@@ -936,7 +1015,7 @@ int ft_model_param_info(ft_model* m, size_t index, const char** name, size_t* nu
     return guarded([&]() -> int {
         FT_CHECK_ARG(m, "ft_model_param_info: NULL argument");
         if (m->params_dirty) {
-            rebuild_params(m);
+            FT_TRY(rebuild_params(m));
             ws_free(m);
         }
         FT_CHECK_ARG(index < m->params.size(), "ft_model_param_info: index %zu of %zu", index, m->params.size());
@@ -969,7 +1048,7 @@ int ft_trainer_create(ft_model* m, const ft_trainer_config* cfg, ft_trainer** ou
     return guarded([&]() -> int {
         FT_CHECK_ARG(m && cfg && out, "ft_trainer_create: NULL argument");
         if (m->params_dirty) {
-            rebuild_params(m);
+            FT_TRY(rebuild_params(m));
             ws_free(m);
         }
         FT_CHECK_ARG(!m->params.empty(), "ft_trainer_create: the model has no LoRA adapter to train");

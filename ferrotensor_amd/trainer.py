@@ -33,12 +33,14 @@ class ModelConfig:
     f16_linears: bool = False
     checkpoint_blocks: bool = False
     head_all_rows: bool = False
+    trainable_base: bool = False
 
     def c(self):
         return _lib.ModelConfigC(self.vocab_size, self.hidden_size, self.intermediate_size, self.num_hidden_layers,
                                  self.num_attention_heads, self.num_key_value_heads, self.rms_norm_eps,
                                  self.rope_theta, 1 if self.tie_word_embeddings else 0, 1 if self.f16_linears else 0,
-                                 1 if self.checkpoint_blocks else 0, 1 if self.head_all_rows else 0)
+                                 1 if self.checkpoint_blocks else 0, 1 if self.head_all_rows else 0,
+                                 1 if self.trainable_base else 0)
 
 
 @dataclass
@@ -94,6 +96,12 @@ class Lfm2Model:
     def add_lora(self, prefix: str, rank: int, alpha: float):
         """`ModelBuilder::maybe_add_lora`: a fresh adapter, A seeded from (layer, module name), B zero."""
         check(self._lib.ft_model_add_lora(self.handle, prefix.encode(), rank, alpha))
+
+    def set_head_all_rows(self, all_rows: bool):
+        """True: final norm, vocabulary head and loss on every position (the reference's behaviour); False: on
+        the supervised positions only (same results, less work)."""
+        check(self._lib.ft_model_set_head_all_rows(self.handle, 1 if all_rows else 0))
+        self.config.head_all_rows = bool(all_rows)
 
     def linear_prefixes(self, targets: Sequence[str]) -> List[str]:
         out = []

@@ -375,6 +375,12 @@ typedef struct ft_model_config {
      * unless the row count moves the head's input-gradient GEMM across the tile count at which
      * it splits K (a different summation order: rounding-level differences). */
     int32_t head_all_rows;
+    /* Lfm2ModelBuilder::with_trainable_base (model_builder.rs:325-357): the linear weights are
+     * stored f32 whatever f16_linears says, and they and the norm scales receive gradients and are
+     * trained next to the adapters (`<prefix>.weight`, `...layernorm.weight`, `model.norm.weight`,
+     * `lm_head.weight` in the parameter list; weight gradients in the stored [in, out] layout). The
+     * embedding table stays frozen. 0 (default): LoRA factors only. */
+    int32_t trainable_base;
 } ft_model_config;
 
 typedef struct ft_model ft_model;
@@ -404,6 +410,9 @@ int ft_lora_init_a(float* a_host, size_t in_dim, size_t out_dim, size_t rank, ui
 /* ModelBuilder::maybe_add_lora (model_builder.rs:425-446): attaches a freshly
  * initialised adapter (seeded A, zero B) to the linear named `prefix`. */
 int ft_model_add_lora(ft_model* m, const char* prefix, size_t rank, float alpha);
+/* Switches ft_model_config.head_all_rows after creation: 1 = the head runs on every position, as
+ * Lfm2Model::forward_batch_with_dropout does (lfm.rs:597-623); 0 = on the supervised ones only. */
+int ft_model_set_head_all_rows(ft_model* m, int all_rows);
 /* Number of trainable tensors and their fixture names / sizes, in the order
  * gradients and parameters are reported (`<prefix>.lora_a`, `<prefix>.lora_b`). */
 int ft_model_param_count(ft_model* m, size_t* count);

@@ -27,12 +27,12 @@ def fx(golden_dir):
     return GradientParityFixture(golden_dir)
 
 
-def hip_model_from_fixture(ctx, fx):
+def hip_model_from_fixture(ctx, fx, trainable_base=False):
     from ferrotensor_amd.trainer import Lfm2Model, ModelConfig
     c = fx.config
     cfg = ModelConfig(c.vocab_size, c.hidden_size, c.intermediate_size, c.num_hidden_layers,
                       c.num_attention_heads, c.num_key_value_heads, c.rms_norm_eps, c.rope_theta,
-                      c.tie_word_embeddings, False)
+                      c.tie_word_embeddings, False, trainable_base=trainable_base)
     m = Lfm2Model(ctx, cfg)
     m.load_tensors(fx.model)
     for name in m.linear_prefixes(["q_proj", "k_proj", "v_proj", "o_proj", "gate_proj", "up_proj", "down_proj",
@@ -41,11 +41,13 @@ def hip_model_from_fixture(ctx, fx):
     return m
 
 
-@pytest.mark.parametrize("case", ["single", "batch", "masked"])
+@pytest.mark.parametrize("case", ["single", "batch", "masked", "full"])
 def test_lora_gradients_match_pytorch_fixture(ctx, fx, case):
+    """The four cases of gradient_parity.rs:416-444; `full` trains the base as well: the gradients of every
+    linear weight (in the stored [in, out] layout) and norm scale next to the 30 adapter gradients."""
     from ferrotensor_amd.trainer import Trainer
     rows, targets, masks, trainable_base, want_loss = fx.case(case)
-    model = hip_model_from_fixture(ctx, fx)
+    model = hip_model_from_fixture(ctx, fx, trainable_base)
     logits = model.forward_batch(rows)
     assert worst_ratio(logits, fx.expected[f"logits.{case}"]) <= 1.0
     # grad_accum_steps = 1 gives the backward seed 1 the fixture uses
@@ -54,10 +56,41 @@ def test_lora_gradients_match_pytorch_fixture(ctx, fx, case):
     assert worst_ratio([st.loss], [want_loss]) <= 1.0, (st.loss, want_loss)
     want = fx.expected_grads(case)
     grads = model.grads()
-    assert set(grads) == set(want) and len(want) == 30
+    assert set(grads) == set(want) and len(want) == (50 if trainable_base else 30)
     bad = {n: worst_ratio(grads[n], want[n]) for n in want if worst_ratio(grads[n], want[n]) > 1.0}
     assert not bad, bad
     assert not st.optimizer_step
+
+
+def test_trainable_base_accumulates_and_trains(ctx, fx):
+    """With a trainable base the weight and norm-scale gradients accumulate over micro-batches like the adapter
+    gradients (two one-sequence chunks == the two-sequence chunk), f16 storage is overridden by f32
+    (model_builder.rs:325-340), and an optimizer step moves base weights and norm scales."""
+    import dataclasses
+    from ferrotensor_amd.trainer import Lfm2Model, Trainer
+    rows, targets, masks, _, _ = fx.case("full")
+    model = hip_model_from_fixture(ctx, fx, True)
+    tr = Trainer(model, lr=1e-3, weight_decay=0.0, grad_accum_steps=2)
+    tr.train_chunk(rows, targets, masks, apply=False)
+    whole = model.grads()
+    model2 = hip_model_from_fixture(ctx, fx, True)
+    tr2 = Trainer(model2, lr=1e-3, weight_decay=0.0, grad_accum_steps=2)
+    assert not tr2.train_chunk(rows[:1], targets[:1], masks[:1]).optimizer_step
+    tr2.train_chunk(rows[1:], targets[1:], masks[1:], apply=False)
+    parts = model2.grads()
+    assert len(whole) == 50
+    for n in whole:
+        assert worst_ratio(parts[n], whole[n]) <= 1.0, n
+    before = model.params()
+    assert tr.train_chunk(rows, targets, masks).optimizer_step
+    after = model.params()
+    moved = [n for n in before if not np.array_equal(before[n], after[n])]
+    assert "model.layers.0.mlp.down_proj.weight" in moved and "model.norm.weight" in moved and len(moved) == 50
+    # f16 storage asked for, trainable base wins: the linears stay f32 and keep the fixture's logits
+    cfg16 = dataclasses.replace(model.config, f16_linears=True)
+    m16 = Lfm2Model(ctx, cfg16)
+    m16.load_tensors(fx.model)
+    assert worst_ratio(m16.forward_batch(fx.case("single")[0]), fx.expected["logits.base"], atol=1e-5, rtol=0.0) <= 1.0
 
 
 def test_base_logits_without_adapters(ctx, fx):
