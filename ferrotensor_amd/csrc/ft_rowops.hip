@@ -5,6 +5,7 @@
 // wave reductions), so HBM traffic equals the algorithmic byte count.
 #include "ft_common.h"
 
+#include <atomic>
 #include <mutex>
 
 namespace {
@@ -934,7 +935,7 @@ constexpr int kNoAllocMaxDevices = 64;
 
 static __device__ __align__(256) float scratch[kNoAllocMaxParts * kNoAllocMaxSize];
 
-static float* g_noalloc_scratch[kNoAllocMaxDevices] = {};
+static std::atomic<float*> g_noalloc_scratch[kNoAllocMaxDevices] = {};  // written once per device, under the mutex
 static std::mutex g_noalloc_mutex;
 
 // Device address of `scratch` on `device`, which must be the current device.
@@ -942,11 +943,11 @@ int ft_internal_noalloc_init(int device) {
     FT_CHECK_ARG(device >= 0 && device < kNoAllocMaxDevices, "no-alloc scratch: device %d is outside 0..%d", device,
                  kNoAllocMaxDevices - 1);
     std::lock_guard<std::mutex> lock(g_noalloc_mutex);
-    if (g_noalloc_scratch[device]) return FT_OK;
+    if (g_noalloc_scratch[device].load(std::memory_order_acquire)) return FT_OK;
     float* ptr = nullptr;
     FT_HIP(hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch)));
     FT_CHECK_ARG(ptr != nullptr, "no-alloc scratch: hipGetSymbolAddress returned NULL on device %d", device);
-    g_noalloc_scratch[device] = ptr;
+    g_noalloc_scratch[device].store(ptr, std::memory_order_release);
     return FT_OK;
 }
 
@@ -1110,13 +1111,13 @@ int ft_rms_norm_backward_noalloc(ft_context* ctx, const float* x, const float* w
                  "ft_rms_norm_backward_noalloc: x, w, g and gx must be 16-byte aligned");
     FT_CHECK_ARG(ctx->device >= 0 && ctx->device < kNoAllocMaxDevices, "ft_rms_norm_backward_noalloc: device %d",
                  ctx->device);
-    float* partial = g_noalloc_scratch[ctx->device];
+    float* partial = g_noalloc_scratch[ctx->device].load(std::memory_order_acquire);
     if (!partial) {
         // A context normally looks the address up when it is created; this is the first call on a
         // device whose contexts were made before the library knew the device.
         FT_HIP(hipSetDevice(ctx->device));
         FT_TRY(ft_internal_noalloc_init(ctx->device));
-        partial = g_noalloc_scratch[ctx->device];
+        partial = g_noalloc_scratch[ctx->device].load(std::memory_order_acquire);
     }
     // Same launch shape as ft_rms_norm_backward: one partial row per workgroup, every row of the
     // array that the second kernel reads is written in full by the first (nothing to clear).
