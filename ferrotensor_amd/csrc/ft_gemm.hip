@@ -1138,21 +1138,24 @@ __global__ __launch_bounds__(256) void gemm_f32_async_kernel(F32AsyncArgs g) {
     floatx16 acc;
 #pragma unroll
     for (int r = 0; r < 16; r++) acc[r] = 0.0f;
-    auto iter = [&](int t, const float* cur, float* refill) {
-        __builtin_amdgcn_s_waitcnt(0x0F70 | LPT);
-        __builtin_amdgcn_s_barrier();
-        __builtin_amdgcn_sched_barrier(0);
-        issue(t + NST - 1, refill);
-        __builtin_amdgcn_sched_barrier(0);
-        float4 af[2], bf[2];
-        af[0] = frag(cur, A_KM, 0, wm0 + l32);
-        bf[0] = frag(cur + TILE, B_KM, 0, wn0 + l32);
+    // Rotated like the loop of gemm_async_kernel: wait, barrier, refill and the first fragment
+    // reads of tile t + 1 come before the last MFMA group of tile t.
+    float4 af[2], bf[2];
+    auto iter = [&](int t, float* cur, const float* next) {
 #pragma unroll
         for (int s = 0; s < 4; s++) {
             const int c = s & 1, nx = c ^ 1;
             if (s + 1 < 4) {
                 af[nx] = frag(cur, A_KM, s + 1, wm0 + l32);
                 bf[nx] = frag(cur + TILE, B_KM, s + 1, wn0 + l32);
+            } else {
+                // own reads of the stage complete, tile t + 1 landed (tile t + 2 may be in flight)
+                __builtin_amdgcn_s_waitcnt(0x0070 | LPT);
+                __builtin_amdgcn_s_barrier();
+                __builtin_amdgcn_sched_barrier(0);
+                issue(t + NST, cur);
+                af[nx] = frag(next, A_KM, 0, wm0 + l32);
+                bf[nx] = frag(next + TILE, B_KM, 0, wn0 + l32);
             }
             __builtin_amdgcn_sched_barrier(0);
             acc = __builtin_amdgcn_mfma_f32_32x32x2f32(af[c].x, bf[c].x, acc, 0, 0, 0);
@@ -1164,10 +1167,17 @@ __global__ __launch_bounds__(256) void gemm_f32_async_kernel(F32AsyncArgs g) {
     };
     issue(t0, St0);
     issue(t0 + 1, St1);
+    __builtin_amdgcn_s_waitcnt(0x0F70 | LPT);
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+    issue(t0 + 2, St2);
+    af[0] = frag(St0, A_KM, 0, wm0 + l32);
+    bf[0] = frag(St0 + TILE, B_KM, 0, wn0 + l32);
+    __builtin_amdgcn_sched_barrier(0);
     for (int t = t0; t < nt; t += NST) {
-        iter(t, St0, St2);
-        if (t + 1 < nt) iter(t + 1, St1, St0);
-        if (t + 2 < nt) iter(t + 2, St2, St1);
+        iter(t, St0, St1);
+        if (t + 1 < nt) iter(t + 1, St1, St2);
+        if (t + 2 < nt) iter(t + 2, St2, St0);
     }
     __builtin_amdgcn_s_waitcnt(0x0F70);  // nothing may still be landing in LDS when the workgroup retires
     const int col = n0 + wn0 + l32;
