@@ -713,39 +713,73 @@ def test_micro_batches_accumulate_to_the_batched_step(ctx):
 
 
 def test_training_on_one_batch_halves_the_loss(ctx):
-    """`lora_training_reduces_loss_on_a_tiny_model` (ferrotensor-trainer/tests/gpu_training.rs:24-54): a tiny
-    model with weights of the reference test's scale (embedding 0.5, linears 0.2, tests/common/mod.rs:102-118),
-    freshly seeded rank-4 adapters on q/k/v/o, one memorisable sequence ((7i + 3) mod 64, common/mod.rs:370-372),
-    AdamW at 1e-2: 40 optimizer steps at least halve the loss."""
+    """`lora_training_reduces_loss_on_a_tiny_model` and `f16_base_weights_halve_memory_and_train_like_f32`
+    (ferrotensor-trainer/tests/gpu_training.rs:24-54, 56-95): a tiny model with weights of the reference test's
+    scale (embedding 0.5, linears 0.2, tests/common/mod.rs:102-118), freshly seeded rank-4 adapters on q/k/v/o,
+    one memorisable sequence ((7i + 3) mod 64, common/mod.rs:370-372), AdamW at 1e-2: 40 optimizer steps at
+    least halve the loss, with f32 and with f16 base weights, whose first loss is within 1 % of the f32 one."""
     from ferrotensor_amd.trainer import Lfm2Model, ModelConfig, Trainer
-    cfg = ModelConfig(vocab_size=64, hidden_size=32, intermediate_size=64, num_hidden_layers=2,
-                      num_attention_heads=4, num_key_value_heads=2, rms_norm_eps=1e-5, rope_theta=10000.0,
-                      tie_word_embeddings=False, f16_linears=False)
-    tensors = random_model_tensors(cfg, 3)
-    rng = np.random.default_rng(17)
-    for name, w in tensors.items():
-        if name.endswith("norm.weight") or name.endswith("layernorm.weight"):
-            continue
-        scale = 0.5 if "embed_tokens" in name else 0.2
-        tensors[name] = rng.uniform(-scale, scale, w.shape).astype(np.float32)
-    hip = Lfm2Model(ctx, cfg)
-    hip.load_tensors(tensors)
-    for prefix in hip.linear_prefixes(["q_proj", "k_proj", "v_proj", "o_proj"]):
-        hip.add_lora(prefix, 4, 8.0)
     seq = np.array([(i * 7 + 3) % 64 for i in range(24)], np.uint32)
     rows, targets = seq[None, :-1], seq[None, 1:]
     masks = np.ones_like(rows, dtype=np.uint8)
-    tr = Trainer(hip, lr=1e-2, grad_accum_steps=1)
-    losses = []
-    for _ in range(40):
-        st = tr.train_chunk(rows, targets, masks)
-        assert st.optimizer_step
-        losses.append(st.loss)
-    tr.close()
-    hip.close()
-    assert all(np.isfinite(losses))
-    assert losses[-1] < 0.5 * losses[0], losses
+    runs = {}
+    for f16 in (False, True):
+        cfg = ModelConfig(vocab_size=64, hidden_size=32, intermediate_size=64, num_hidden_layers=2,
+                          num_attention_heads=4, num_key_value_heads=2, rms_norm_eps=1e-5, rope_theta=10000.0,
+                          tie_word_embeddings=False, f16_linears=f16)
+        tensors = random_model_tensors(cfg, 3)
+        rng = np.random.default_rng(17)
+        for name, w in tensors.items():
+            if name.endswith("norm.weight") or name.endswith("layernorm.weight"):
+                continue
+            scale = 0.5 if "embed_tokens" in name else 0.2
+            tensors[name] = rng.uniform(-scale, scale, w.shape).astype(np.float32)
+        hip = Lfm2Model(ctx, cfg)
+        hip.load_tensors(tensors)
+        for prefix in hip.linear_prefixes(["q_proj", "k_proj", "v_proj", "o_proj"]):
+            hip.add_lora(prefix, 4, 8.0)
+        tr = Trainer(hip, lr=1e-2, grad_accum_steps=1)
+        losses = []
+        for _ in range(40):
+            st = tr.train_chunk(rows, targets, masks)
+            assert st.optimizer_step
+            losses.append(st.loss)
+        tr.close()
+        hip.close()
+        assert all(np.isfinite(losses))
+        assert losses[-1] < 0.5 * losses[0], (f16, losses)
+        runs[f16] = losses
+    assert abs(runs[True][0] - runs[False][0]) <= 1e-2 * runs[False][0], (runs[True][0], runs[False][0])
 
+
+def test_gradient_accumulation_defers_the_step_and_is_deterministic(ctx):
+    """gpu_training.rs:224-253: with grad_accum = 2 the first sequence only accumulates and the second applies
+    the update; repeating the run gives bit-identical adapters, stepping after every sequence different ones."""
+    from ferrotensor_amd.trainer import Trainer
+    seq = np.array([(i * 7 + 3) % 64 for i in range(24)], np.uint32)
+    a = (seq[None, :12], seq[None, 1:13])
+    b = (seq[None, 6:18], seq[None, 7:19])
+    ones = np.ones((1, 12), np.uint8)
+
+    def run(accum):
+        hip, _ = build_pair(ctx, tiny_config(False, False), ["q_proj", "k_proj", "v_proj", "o_proj"], rank=4,
+                            alpha=8.0, seed=29)
+        tr = Trainer(hip, lr=1e-2, grad_accum_steps=accum)
+        s1 = tr.train_chunk(a[0], a[1], ones)
+        s2 = tr.train_chunk(b[0], b[1], ones)
+        values = hip.params()
+        tr.close()
+        hip.close()
+        return s1, s2, values
+
+    s1, s2, accumulated = run(2)
+    assert not s1.optimizer_step and s2.optimizer_step
+    _, _, again = run(2)
+    for k in accumulated:
+        assert np.array_equal(accumulated[k].view(np.uint32), again[k].view(np.uint32)), k
+    p1, p2, sequential = run(1)
+    assert p1.optimizer_step and p2.optimizer_step
+    assert any(not np.array_equal(accumulated[k], sequential[k]) for k in accumulated)
 
 def test_the_step_is_deterministic_to_the_bit(ctx):
     """Two runs of the same three steps from the same state give the same bits in every gradient, weight and
