@@ -132,6 +132,7 @@ SIGNATURES = {
     "ft_model_param_count": [_P, C.POINTER(_SZ)],
     "ft_model_param_info": [_P, _SZ, C.POINTER(C.c_char_p), C.POINTER(_SZ)],
     "ft_model_read_param": [_P, _SZ, _P],
+    "ft_model_write_param": [_P, _SZ, _P],
     "ft_model_read_grad": [_P, _SZ, _P],
     "ft_model_forward_logits": [_P, _P, _SZ, _SZ, _P],
     "ft_model_eval_chunk": [_P, _P, _P, _P, _SZ, _SZ, _P, _P],
@@ -141,6 +142,7 @@ SIGNATURES = {
     "ft_trainer_write_moments": [_P, _SZ, _P, _P],
     "ft_trainer_get_adam_t": [_P, C.POINTER(_F)],
     "ft_trainer_set_adam_t": [_P, _F],
+    "ft_trainer_set_adam_hyper": [_P, _F, _F, _F, _F, _F],
     "ft_trainer_optimizer_steps": [_P, C.POINTER(_SZ)],
     "ft_trainer_step_in_accum": [_P, C.POINTER(_SZ)],
     "ft_trainer_set_optimizer_steps": [_P, _SZ],

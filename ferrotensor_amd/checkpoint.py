@@ -149,12 +149,19 @@ def file_name(param: str) -> str:
     return param
 
 
-def _param_shapes(model) -> Dict[str, Tuple[int, int]]:
+def _param_shapes(model) -> Dict[str, Tuple[int, ...]]:
+    """Shapes as the reference keeps them: A [in, r], B [r, out]; with a trainable base a linear weight in
+    its stored [in, out] layout and a norm scale as a vector."""
     shapes = {}
     for name, numel in model.named_params():
         prefix, kind = name.rsplit(".", 1)
-        i, o = model.linear_dims(prefix)
-        shapes[name] = (i, numel // i) if kind == "lora_a" else (numel // o, o)
+        if kind in ("lora_a", "lora_b"):
+            i, o = model.linear_dims(prefix)
+            shapes[name] = (i, numel // i) if kind == "lora_a" else (numel // o, o)
+        elif prefix.endswith("norm"):
+            shapes[name] = (numel,)
+        else:
+            shapes[name] = tuple(model.linear_dims(prefix))
     return shapes
 
 
@@ -191,6 +198,51 @@ def apply_lora_checkpoint(model, ckpt: LoraCheckpoint, alpha: Optional[float] = 
         model.set_lora(prefix, a, b, alpha)
         n += 1
     return n
+
+
+LLAMA_RENAMES = ((".input_layernorm.", ".operator_norm."), (".post_attention_layernorm.", ".ffn_norm."),
+                 (".mlp.", ".feed_forward."))
+
+
+def legacy_llama_name(name: str) -> Optional[str]:
+    """The name a Llama-block parameter had in older adapter files (graph/src/lfm.rs:232-255), or None."""
+    if not name.startswith("model.layers."):
+        return None
+    for new, old in LLAMA_RENAMES:
+        if new in name:
+            return name.replace(new, old, 1)
+    return None
+
+
+def apply_checkpoint(ckpt: LoraCheckpoint, model) -> int:
+    """`apply_checkpoint` (ferrotensor-trainer/src/checkpoint.rs:210-286): overwrites every trainable tensor of
+    `model` with the tensor of the same name (or of its old Llama name) in the file, in place. Strict both
+    ways: a tensor the file lacks, a shape that differs, or a tensor in the file that the model does not
+    have (a different rank, other LoRA targets) is an error and nothing is written. Returns the count."""
+    shapes = _param_shapes(model)
+    params = [(file_name(name), tuple(shapes[name])) for name, _ in model.named_params()]
+    sources = []
+    for index, (name, shape) in sorted(enumerate(params), key=lambda e: e[1][0]):
+        legacy = legacy_llama_name(name)
+        if legacy is not None and legacy not in ckpt.tensors:
+            legacy = None
+        if name in ckpt.tensors and legacy is not None:
+            raise ValueError("checkpoint has both %s and its old name %s" % (name, legacy))
+        key = name if name in ckpt.tensors else legacy
+        if key is None:
+            raise ValueError("checkpoint has no tensor %s" % name)
+        have = tuple(ckpt.tensors[key].shape)
+        if have != shape:
+            raise ValueError("tensor %s: checkpoint has shape %s, model expects %s" % (key, list(have), list(shape)))
+        sources.append((index, key))
+    used = {key for _, key in sources}
+    unused = sorted(k for k in ckpt.tensors if k not in used)
+    if unused:
+        raise ValueError("checkpoint has %d tensor(s) the model does not have, e.g. %s (a different rank, LoRA "
+                         "targets or --train-modules?)" % (len(unused), unused[0]))
+    for index, key in sources:
+        model.write_param(index, ckpt.tensors[key])
+    return len(sources)
 
 
 # ---------------------------------------------------------------------------
@@ -311,25 +363,60 @@ def load_training_checkpoint(path: str) -> Tuple[TrainingState, Optional[AdamWSt
     return state, adam
 
 
-def restore_optimizer(trainer, adam: AdamWState, step: int) -> int:
-    """`AdamW::load_state` + `Trainer::set_optimizer_steps`: parameters that have both saved moments
-    (of the right size) take them; returns how many did. The step counter `t` and the schedule
-    position are restored when at least one matched."""
-    lib, model = trainer._lib, trainer.model
-    matched = 0
-    for i, (name, numel) in enumerate(model.named_params()):
-        key = file_name(name)
-        m, v = adam.m_states.get(key), adam.v_states.get(key)
-        if m is None or v is None:
+@dataclass(frozen=True)
+class OptimizerLoad:
+    """autograd/src/lib.rs:1427-1442: parameters that took both saved moments, parameters left without,
+    and saved names no parameter has."""
+    matched: int
+    missing: int
+    unused: int
+
+    def is_complete(self) -> bool:
+        return self.missing == 0 and self.unused == 0
+
+
+def match_moments(shapes: Dict[str, Tuple[int, ...]], adam: AdamWState) -> Tuple[List[str], OptimizerLoad]:
+    """`match_moments` (autograd/src/lib.rs:1669-1703): which saved moments belong to which parameters, without
+    touching the device. A saved moment whose shape differs from its parameter's is an error that names it."""
+    saved = sorted(set(adam.m_states) | set(adam.v_states))
+    matched = []
+    for name in saved:
+        shape, m, v = shapes.get(name), adam.m_states.get(name), adam.v_states.get(name)
+        if shape is None or m is None or v is None:
             continue
-        if m.size != numel or v.size != numel:
-            raise ValueError("saved moments of %s hold %d / %d values, the parameter %d" % (key, m.size, v.size, numel))
-        m = np.ascontiguousarray(m, np.float32)
-        v = np.ascontiguousarray(v, np.float32)
+        for kind, moment in (("first", m), ("second", v)):
+            if tuple(moment.shape) != tuple(shape):
+                raise ValueError("saved %s moment of %s has shape %s (%d values), the parameter has shape %s"
+                                 % (kind, name, list(moment.shape), moment.size, list(shape)))
+        matched.append(name)
+    return matched, OptimizerLoad(len(matched), len(shapes) - len(matched), len(saved) - len(matched))
+
+
+def restore_optimizer(trainer, adam: AdamWState, step: Optional[int] = None) -> OptimizerLoad:
+    """`AdamW::load_state` (autograd/src/lib.rs:1630-1662) and, given `step`, `Trainer::set_optimizer_steps`:
+    every parameter with both saved moments of its shape takes them; a wrong shape raises before anything is
+    changed; when nothing matches the optimizer is left as it was; otherwise the saved hyperparameters and
+    step counter `t` come back too (parameters without saved moments start from zero moments)."""
+    lib, model = trainer._lib, trainer.model
+    names = [(file_name(name), numel) for name, numel in model.named_params()]
+    shapes = {file_name(n): s for n, s in _param_shapes(model).items()}
+    matched, report = match_moments(shapes, adam)
+    if not matched:
+        return report
+    taken = set(matched)
+    for i, (key, numel) in enumerate(names):
+        if key in taken:
+            m = np.ascontiguousarray(adam.m_states[key], np.float32)
+            v = np.ascontiguousarray(adam.v_states[key], np.float32)
+        else:
+            m = v = np.zeros(numel, np.float32)
         check(lib.ft_trainer_write_moments(trainer.handle, i, m.ctypes.data_as(C.c_void_p),
                                            v.ctypes.data_as(C.c_void_p)))
-        matched += 1
-    if matched:
-        check(lib.ft_trainer_set_adam_t(trainer.handle, float(adam.t)))
+    check(lib.ft_trainer_set_adam_hyper(trainer.handle, adam.lr, adam.beta1, adam.beta2, adam.eps, adam.weight_decay))
+    trainer.hyper.update(beta1=adam.beta1, beta2=adam.beta2, eps=adam.eps, weight_decay=adam.weight_decay)
+    if trainer.lr_schedule == "constant":
+        trainer.hyper["lr"] = adam.lr
+    check(lib.ft_trainer_set_adam_t(trainer.handle, float(adam.t)))
+    if step is not None:
         trainer.set_optimizer_steps(step)
-    return matched
+    return report

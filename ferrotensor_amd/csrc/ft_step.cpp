@@ -1030,6 +1030,12 @@ int ft_model_read_param(ft_model* m, size_t index, float* out_host) {
     return ft_download(m->ctx, out_host, m->params[index].w, m->params[index].n * sizeof(float));
 }
 
+int ft_model_write_param(ft_model* m, size_t index, const float* host) {
+    FT_CHECK_ARG(m && host && !m->params_dirty && index < m->params.size(), "ft_model_write_param: bad argument");
+    // The buffer keeps its address: optimizer moments and trainers built for it stay valid.
+    return ft_upload(m->ctx, m->params[index].w, host, m->params[index].n * sizeof(float));
+}
+
 int ft_model_read_grad(ft_model* m, size_t index, float* out_host) {
     FT_CHECK_ARG(m && out_host && !m->params_dirty && index < m->params.size(), "ft_model_read_grad: bad argument");
     return ft_download(m->ctx, out_host, m->params[index].g, m->params[index].n * sizeof(float));
@@ -1230,6 +1236,22 @@ int ft_trainer_get_adam_t(ft_trainer* t, float* steps) {
 int ft_trainer_set_adam_t(ft_trainer* t, float steps) {
     FT_CHECK_ARG(t && steps >= 0.0f, "ft_trainer_set_adam_t: bad argument");
     t->t = steps;
+    return FT_OK;
+}
+
+int ft_trainer_set_adam_hyper(ft_trainer* t, float lr, float beta1, float beta2, float eps, float weight_decay) {
+    FT_CHECK_ARG(t, "ft_trainer_set_adam_hyper: NULL argument");
+    FT_CHECK_ARG(std::isfinite(lr) && beta1 >= 0.0f && beta1 < 1.0f && beta2 >= 0.0f && beta2 < 1.0f && eps >= 0.0f &&
+                     std::isfinite(weight_decay),
+                 "ft_trainer_set_adam_hyper: lr %g, betas (%g, %g), eps %g, weight decay %g", lr, beta1, beta2, eps,
+                 weight_decay);
+    // With a schedule the optimizer's rate is overwritten before every step (LRScheduler::step), so a
+    // restored rate only lasts where there is none.
+    if (t->cfg.lr_schedule == FT_LR_CONSTANT) t->cfg.lr = lr;
+    t->cfg.beta1 = beta1;
+    t->cfg.beta2 = beta2;
+    t->cfg.eps = eps;
+    t->cfg.weight_decay = weight_decay;
     return FT_OK;
 }
 

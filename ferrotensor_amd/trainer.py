@@ -139,6 +139,13 @@ class Lfm2Model:
             out.append((name.value.decode(), numel.value))
         return out
 
+    def write_param(self, index: int, values):
+        """Overwrites trainable tensor `index` (the order of `named_params`) in place."""
+        numel = self.named_params()[index][1]
+        v = np.ascontiguousarray(values, np.float32).reshape(-1)
+        assert v.size == numel, "write_param: %d values for a parameter of %d" % (v.size, numel)
+        check(self._lib.ft_model_write_param(self.handle, index, v.ctypes.data_as(C.c_void_p)))
+
     def _read(self, fn, index, numel):
         out = np.empty(numel, np.float32)
         check(fn(self.handle, index, out.ctypes.data_as(C.c_void_p)))
@@ -243,6 +250,7 @@ class Trainer:
         self._lib = model._lib
         self.hyper = dict(lr=lr, beta1=beta1, beta2=beta2, eps=eps, weight_decay=weight_decay)
         kind = LR_SCHEDULES[lr_schedule]
+        self.lr_schedule = lr_schedule
         cfg = _lib.TrainerConfigC(lr, beta1, beta2, eps, weight_decay,
                                   clip_grad_norm if clip_grad_norm else 0.0, grad_accum_steps,
                                   kind, warmup_steps, total_steps, min_lr)

@@ -420,6 +420,9 @@ int ft_model_param_info(ft_model* m, size_t index, const char** name, size_t* nu
 /* Copies parameter / gradient `index` to the host (numel f32 values). The
  * gradient is the one the last step left (scaled by 1/grad_accum, unclipped). */
 int ft_model_read_param(ft_model* m, size_t index, float* out_host);
+/* Overwrites parameter `index` with numel f32 values from the host, in place: what
+ * apply_checkpoint does to an existing tensor (ferrotensor-trainer/src/checkpoint.rs:275-283). */
+int ft_model_write_param(ft_model* m, size_t index, const float* host);
 int ft_model_read_grad(ft_model* m, size_t index, float* out_host);
 /* Lfm2Model::forward_batch (lfm.rs:590-623): logits [B*S, vocab] to the host. */
 int ft_model_forward_logits(ft_model* m, const uint32_t* rows, size_t B, size_t S, float* logits_host);
@@ -480,6 +483,11 @@ int ft_trainer_read_moments(ft_trainer* t, size_t index, float* m_host, float* v
 int ft_trainer_write_moments(ft_trainer* t, size_t index, const float* m_host, const float* v_host);
 int ft_trainer_get_adam_t(ft_trainer* t, float* steps);
 int ft_trainer_set_adam_t(ft_trainer* t, float steps);
+/* The hyperparameters AdamW::load_state restores with the moments (autograd/src/lib.rs:1644-1649:
+ * lr, beta1, beta2, eps, weight_decay of the saved optimizer). With a schedule the rate is
+ * overwritten before every step (LRScheduler::step), so `lr` is only taken with FT_LR_CONSTANT. */
+int ft_trainer_set_adam_hyper(ft_trainer* t, float lr, float beta1, float beta2, float eps,
+                              float weight_decay);
 int ft_trainer_optimizer_steps(ft_trainer* t, size_t* steps);
 int ft_trainer_set_optimizer_steps(ft_trainer* t, size_t steps);
 /* Trainer::step_in_accum (trainer/src/lib.rs:463-466): sequences counted into the open

@@ -672,12 +672,92 @@ def test_resume_from_adapter_and_state_files_is_bit_identical(ctx, tmp_path):
     tr3 = Trainer(hip3, **kw)
     state, adam = ck.load_training_checkpoint(state_path)
     assert state.step == 2 and adam.t == 2.0
-    assert ck.restore_optimizer(tr3, adam, state.step) == 2 * 4 * cfg.num_hidden_layers
+    assert ck.restore_optimizer(tr3, adam, state.step) == ck.OptimizerLoad(2 * 4 * cfg.num_hidden_layers, 0, 0)
     st = tr3.train_chunk(rows, targets, masks)
     assert (st.loss, st.grad_norm, st.lr) == (straight[2].loss, straight[2].grad_norm, straight[2].lr)
     got = hip3.params()
     for n in want:
         np.testing.assert_array_equal(got[n], want[n])
+
+
+def test_optimizer_state_load_reports_what_it_matched(ctx):
+    """`optimizer_state_load_reports_what_it_matched` (ferrotensor-trainer/tests/gpu_training.rs:338-402): the same
+    parameters all take their moments back (and `t`, and the saved hyperparameters); disjoint names match
+    nothing, say so and leave the optimizer as it was; a moment of the wrong shape is an error that names the
+    parameter, and nothing is applied."""
+    import dataclasses
+    from ferrotensor_amd import checkpoint as ck
+    from ferrotensor_amd.trainer import Trainer
+    mods = ["q_proj", "k_proj", "v_proj", "o_proj"]
+    seq = np.array([(i * 7 + 3) % 64 for i in range(24)], np.uint32)
+    rows, targets, masks = seq[None, :-1], seq[None, 1:], np.ones((1, 23), np.uint8)
+    hip, _ = build_pair(ctx, tiny_config(), mods, rank=4, alpha=8.0, seed=31)
+    trained = Trainer(hip, lr=1e-2, beta1=0.8, weight_decay=0.05, grad_accum_steps=1)
+    for _ in range(2):
+        trained.train_chunk(rows, targets, masks)
+    state = ck.optimizer_state(trained)
+    n = len(hip.named_params())
+    assert n == 2 * 4 * 2 and state.t == 2.0
+
+    def moments(tr):
+        return ck.optimizer_state(tr)
+
+    same = Trainer(hip, lr=1e-3, grad_accum_steps=1)
+    assert ck.restore_optimizer(same, state) == ck.OptimizerLoad(n, 0, 0)
+    back = moments(same)
+    assert back.t == 2.0 and (back.lr, back.beta1, back.weight_decay) == (1e-2, 0.8, 0.05)
+    for k in state.m_states:
+        assert np.array_equal(back.m_states[k], state.m_states[k]) and np.array_equal(back.v_states[k], state.v_states[k])
+    # the restored optimizer continues exactly like the one that was saved: same adapters, same third step
+    before = hip.params()
+    third = trained.train_chunk(rows, targets, masks)
+    want = hip.params()
+    for i, (name, _) in enumerate(hip.named_params()):
+        hip.write_param(i, before[name])
+    again = same.train_chunk(rows, targets, masks)
+    assert (again.loss, again.grad_norm) == (third.loss, third.grad_norm)
+    got = hip.params()
+    for name in want:
+        assert np.array_equal(got[name].view(np.uint32), want[name].view(np.uint32)), name
+    same.close()
+
+    renamed = dataclasses.replace(state, m_states={"other." + k: v for k, v in state.m_states.items()},
+                                  v_states={"other." + k: v for k, v in state.v_states.items()})
+    other = Trainer(hip, lr=1e-3, grad_accum_steps=1)
+    assert ck.restore_optimizer(other, renamed) == ck.OptimizerLoad(0, n, n)
+    untouched = moments(other)
+    assert untouched.t == 0.0 and untouched.lr == 1e-3 and all(not m.any() for m in untouched.m_states.values())
+    other.close()
+
+    victim = min(state.v_states)
+    bad = dataclasses.replace(state, v_states={**state.v_states, victim: state.v_states[victim].reshape(-1)})
+    wrong = Trainer(hip, lr=1e-3, grad_accum_steps=1)
+    with pytest.raises(ValueError) as err:
+        ck.restore_optimizer(wrong, bad)
+    assert victim in str(err.value) and "shape" in str(err.value)
+    untouched = moments(wrong)
+    assert untouched.t == 0.0 and all(not m.any() for m in untouched.m_states.values())
+    wrong.close()
+    trained.close()
+    hip.close()
+
+
+def test_adapter_with_wrong_rank_is_rejected(ctx, tmp_path):
+    """`adapter_with_wrong_rank_is_rejected` (gpu_training.rs:404-443): a model built with rank-2 adapters cannot
+    take the rank-4 tensors of an adapter file saved without metadata; the error speaks of the shape."""
+    from ferrotensor_amd import checkpoint as ck
+    mods = ["q_proj", "k_proj", "v_proj", "o_proj"]
+    hip, _ = build_pair(ctx, tiny_config(), mods, rank=4, alpha=8.0, seed=33)
+    path = str(tmp_path / "a.safetensors")
+    ck.save_lora_checkpoint(hip, path)
+    hip.close()
+    loaded = ck.load_lora_checkpoint(path)
+    assert loaded.metadata is None
+    other, _ = build_pair(ctx, tiny_config(), mods, rank=2, alpha=8.0, seed=33)
+    with pytest.raises(ValueError) as err:
+        ck.apply_checkpoint(loaded, other)
+    assert "shape" in str(err.value)
+    other.close()
 
 
 def test_micro_batches_accumulate_to_the_batched_step(ctx):
