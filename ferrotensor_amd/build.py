@@ -14,7 +14,7 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ_DIR = os.path.join(HERE, "_build")
 LIB = os.path.join(HERE, "libferrotensor_hip.so")
 
-SOURCES = ["ft_runtime.cpp", "ft_rowops.hip", "ft_gemm.hip", "ft_thin.hip", "ft_attention.hip", "ft_step.cpp"]
+SOURCES = ["ft_runtime.cpp", "ft_rowops.hip", "ft_gemm.hip", "ft_thin.hip", "ft_attention.hip", "ft_attention16.hip", "ft_step.cpp"]
 
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
@@ -43,7 +43,7 @@ def _compile(src):
 
 def build(force=True, sources=None):
     srcs = [s for s in (sources or SOURCES) if os.path.exists(os.path.join(CSRC, s))]
-    headers = [os.path.join(CSRC, "ft_common.h"), os.path.join(CSRC, "ft_thin.h"), os.path.join(ROOT, "include", "ferrotensor_hip.h")]
+    headers = [os.path.join(CSRC, "ft_common.h"), os.path.join(CSRC, "ft_thin.h"), os.path.join(CSRC, "ft_attention.h"), os.path.join(ROOT, "include", "ferrotensor_hip.h")]
     deps = [os.path.join(CSRC, s) for s in srcs] + headers
     if not force and not _stale(LIB, deps):
         return LIB

@@ -11,43 +11,16 @@
 // shuffle finishes a row reduction), and the accumulator registers are already
 // in the operand layout of the next MFMA (P^T as the B operand of O^T = V^T P^T),
 // so P never leaves registers. K/V (or Q/dO) tiles of 32 rows are staged in LDS.
-#include "ft_common.h"
+#include "ft_attention.h"
 
 namespace {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
-constexpr float kMasked = -1.0e30f;   // scores at or below this are treated as -inf
-constexpr float kLseEmpty = 3.0e38f;  // log-sum-exp of a row with no visible key
-
-struct AttnArgs {
-    const float* q;
-    const float* k;
-    const float* v;
-    const float* out;
-    const float* d_out;
-    float* o;
-    float* dq;
-    float* dk;
-    float* dv;
-    float* stats;
-    int B, Sq, Sk, H, Hkv, D;
-    int causal, causal_offset;
-    float scale;
-    // Backward only, head_dim 64 on the LDS kernels: when set, dQ and dK leave the kernels already
-    // rotated back through RoPE (the inverse rotation by the (cos, sin) of their token position,
-    // table [Sq or Sk][32] float2), which is what RoPENode::backward does to them next.
-    const float2* rope;
-    // dK/dV on the LDS kernel with few (key block, kv head) items: one workgroup per query head
-    // instead of per kv head writes that head's unscaled sums to part[2 * g + {0: dK, 1: dV}]
-    // (each laid out like dk), and attn_dkdv_combine_kernel adds the group in head order.
-    float* part;
-    int split_g;
-};
+constexpr float kMasked = kAttnMasked;
+constexpr float kLseEmpty = kAttnLseEmpty;
 
 #define MFMA(a, b, c) __builtin_amdgcn_mfma_f32_32x32x2f32((a), (b), (c), 0, 0, 0)
-
-constexpr size_t kAttnScratchFloats = (size_t)8 << 20;  // 32 MiB of per-head partial dK/dV
 
 __device__ __forceinline__ floatx16 zero16() {
     floatx16 z;
@@ -1132,6 +1105,7 @@ int launch_fwd(ft_context* ctx, const AttnArgs& a) {
     const double by = 4.0 * a.B * ((double)a.Sq * a.H * a.D * 2 + (double)a.Sk * a.Hkv * a.D * 2);
     ft_prof_scope prof(ctx, "attn_fwd_kernel", fl, by);
     if constexpr (DP <= 64) {
+        if (DP == 64 && ft_attn16_usable(a) && ft_attn16_forward_pays(ctx, a)) return ft_attn16_forward(ctx, a);
         if (attn_full(a, DP)) {
             hipLaunchKernelGGL((attn_fwd_lds_kernel<DP>), grid, dim3(kKeySplit * 64), 0, ctx->stream, a);
             FT_LAUNCH_CHECK();
@@ -1160,7 +1134,9 @@ int launch_bwd(ft_context* ctx, const AttnArgs& a) {
             if (full) {
                 // Few workgroups (one or two sequences per pass): four waves share a query block's
                 // keys instead of two, so the chip is not left to a long serial key loop.
-                if ((size_t)grid.x <= (size_t)ctx->num_cus && a.Sk > 64)
+                if (DP == 64 && ft_attn16_usable(a) && ft_attn16_backward_dq_pays(ctx, a)) {
+                    FT_TRY(ft_attn16_backward_dq(ctx, a));
+                } else if ((size_t)grid.x <= (size_t)ctx->num_cus && a.Sk > 64)
                     hipLaunchKernelGGL((attn_bwd_dq_lds_kernel<DP, 4>), grid, dim3(4 * 64), 0, ctx->stream, a);
                 else
                     hipLaunchKernelGGL((attn_bwd_dq_lds_kernel<DP, kKeySplitDq>), grid, dim3(kKeySplitDq * 64), 0,
@@ -1190,6 +1166,7 @@ int launch_bwd(ft_context* ctx, const AttnArgs& a) {
             const size_t G = (size_t)a.H / a.Hkv;
             const size_t n_all = (size_t)a.B * a.Sk * a.Hkv * DP;
             ft_prof_scope prof(ctx, "attn_bwd_dkdv_kernel", 1.5 * fl, by * 0.5);
+            if (DP == 64 && ft_attn16_usable(a)) return ft_attn16_backward_dkdv(ctx, a);
             // Few items (one or two sequences per pass) and a GQA group to share them out:
             // one workgroup per query head, then the ordered sum over the group.
             if (G > 1 && items * 2 <= (size_t)ctx->num_cus && 2 * G * n_all <= kAttnScratchFloats) {
@@ -1256,6 +1233,13 @@ AttnArgs make_args(size_t B, size_t Sq, size_t Sk, size_t H, size_t Hkv, size_t 
 }
 
 }  // namespace
+
+int ft_attn_dkdv_combine(ft_context* ctx, const AttnArgs& a, int DP) {
+    const size_t n_all = (size_t)a.B * a.Sk * a.Hkv * DP;
+    hipLaunchKernelGGL(attn_dkdv_combine_kernel, dim3(ft_div_up(n_all, 256)), dim3(256), 0, ctx->stream, a, DP);
+    FT_LAUNCH_CHECK();
+    return FT_OK;
+}
 
 extern "C" {
 

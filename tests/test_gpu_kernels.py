@@ -588,6 +588,14 @@ ATTN_CASES = [
     (1, 70, 70, 2, 1, 128, True, 0),
     (1, 33, 65, 2, 1, 32, True, 32),        # queries at positions 32.. against a longer key run
     (1, 5, 37, 4, 4, 24, False, 0),
+    # the 16-row kernels (head_dim 64): the headline batch (64-row tiles, 16 waves), half of it (32-row tiles),
+    # ragged lengths, queries offset against a longer key run, no mask
+    (8, 256, 256, 15, 5, 64, True, 0),
+    (4, 256, 256, 15, 5, 64, True, 0),
+    (3, 70, 70, 4, 2, 64, True, 0),
+    (1, 33, 65, 2, 1, 64, True, 32),
+    (40, 50, 50, 4, 2, 64, True, 3),
+    (2, 130, 200, 4, 4, 64, False, 0),
 ]
 
 
