@@ -108,6 +108,11 @@ SIGNATURES = {
     "ft_rope_theta": [_P, _P, _SZ, _SZ, _SZ, _SZ, _SZ, _F],
     "ft_rope_theta_inverse": [_P, _P, _SZ, _SZ, _SZ, _SZ, _SZ, _F],
     "ft_rope_theta_to": [_P, _P, _P, _SZ, _SZ, _SZ, _SZ, _SZ, _F, _I],
+    "ft_train_batch_select": [_P, _P, _P, _P, _SZ, _SZ, C.POINTER(_SZ), C.POINTER(_SZ)],
+    "ft_train_batch_plan": [_SZ, _SZ, _SZ, C.POINTER(_SZ), C.POINTER(_SZ)],
+    "ft_chunk_padded_len": [C.POINTER(_SZ), C.POINTER(_SZ), _SZ, _SZ, C.POINTER(_SZ)],
+    "ft_pad_chunk": [C.POINTER(_P), C.POINTER(_P), C.POINTER(_P), C.POINTER(_SZ), C.POINTER(_SZ), C.POINTER(_SZ),
+                     _SZ, _SZ, _P, _P, _P],
     "ft_flash_attention_v2_with_stats": [_P, _P, _P, _P, _P, _P, _SZ, _SZ, _SZ, _SZ, _SZ, _SZ,
                                          C.POINTER(AttentionOptionsC)],
     "ft_flash_attention_v2_backward_with_stats": [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _SZ, _SZ, _SZ, _SZ,

@@ -404,6 +404,10 @@ def restore_optimizer(trainer, adam: AdamWState, step: Optional[int] = None) -> 
     if not matched:
         return report
     taken = set(matched)
+    # hyperparameters and the step counter first: a value the trainer refuses (beta >= 1, negative eps,
+    # a non-finite rate) raises here, before any moment on the device has been replaced
+    check(lib.ft_trainer_set_adam_hyper(trainer.handle, adam.lr, adam.beta1, adam.beta2, adam.eps, adam.weight_decay))
+    check(lib.ft_trainer_set_adam_t(trainer.handle, float(adam.t)))
     for i, (key, numel) in enumerate(names):
         if key in taken:
             m = np.ascontiguousarray(adam.m_states[key], np.float32)
@@ -412,11 +416,9 @@ def restore_optimizer(trainer, adam: AdamWState, step: Optional[int] = None) -> 
             m = v = np.zeros(numel, np.float32)
         check(lib.ft_trainer_write_moments(trainer.handle, i, m.ctypes.data_as(C.c_void_p),
                                            v.ctypes.data_as(C.c_void_p)))
-    check(lib.ft_trainer_set_adam_hyper(trainer.handle, adam.lr, adam.beta1, adam.beta2, adam.eps, adam.weight_decay))
     trainer.hyper.update(beta1=adam.beta1, beta2=adam.beta2, eps=adam.eps, weight_decay=adam.weight_decay)
     if trainer.lr_schedule == "constant":
         trainer.hyper["lr"] = adam.lr
-    check(lib.ft_trainer_set_adam_t(trainer.handle, float(adam.t)))
     if step is not None:
         trainer.set_optimizer_steps(step)
     return report

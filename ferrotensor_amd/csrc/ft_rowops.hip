@@ -1112,13 +1112,9 @@ int ft_rms_norm_backward_noalloc(ft_context* ctx, const float* x, const float* w
     FT_CHECK_ARG(ctx->device >= 0 && ctx->device < kNoAllocMaxDevices, "ft_rms_norm_backward_noalloc: device %d",
                  ctx->device);
     float* partial = g_noalloc_scratch[ctx->device].load(std::memory_order_acquire);
-    if (!partial) {
-        // A context normally looks the address up when it is created; this is the first call on a
-        // device whose contexts were made before the library knew the device.
-        FT_HIP(hipSetDevice(ctx->device));
-        FT_TRY(ft_internal_noalloc_init(ctx->device));
-        partial = g_noalloc_scratch[ctx->device].load(std::memory_order_acquire);
-    }
+    // Every context looks the address up when it is created (ft_internal_noalloc_init); looking it up
+    // here could load a code object and would change the caller's current device.
+    FT_CHECK_ARG(partial, "ft_rms_norm_backward_noalloc: scratch address not initialised for device %d", ctx->device);
     // Same launch shape as ft_rms_norm_backward: one partial row per workgroup, every row of the
     // array that the second kernel reads is written in full by the first (nothing to clear).
     size_t wgs = (rows + 3) / 4;

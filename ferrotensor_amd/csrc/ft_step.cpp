@@ -1255,6 +1255,93 @@ int ft_trainer_set_adam_hyper(ft_trainer* t, float lr, float beta1, float beta2,
     return FT_OK;
 }
 
+// ---- Trainer::train_batch / train_chunk, the host half (integer work, no device) ----
+
+int ft_train_batch_select(const uint32_t* input_ids, const uint32_t* target_ids, const uint8_t* attention_mask,
+                          const uint8_t* loss_mask, size_t batch, size_t padded_len, size_t* valid_len,
+                          size_t* kept) {
+    FT_CHECK_ARG(valid_len && kept && (batch == 0 || padded_len == 0 || (input_ids && target_ids && attention_mask && loss_mask)),
+                 "ft_train_batch_select: NULL argument");
+    (void)input_ids;
+    (void)target_ids;
+    size_t n = 0;
+    for (size_t b = 0; b < batch; b++) {
+        const uint8_t* attn = attention_mask + b * padded_len;
+        const uint8_t* mask = loss_mask + b * padded_len;
+        size_t len = 0;
+        while (len < padded_len && attn[len] == 1) len++;  // take_while(flag == 1)
+        bool supervised = false;
+        for (size_t i = 0; i < len && !supervised; i++) supervised = mask[i] != 0;
+        // fewer than two tokens, or no supervised position: the sequence does not train
+        if (len < 2 || !supervised) len = 0;
+        valid_len[b] = len;
+        if (len) n++;
+    }
+    *kept = n;
+    return FT_OK;
+}
+
+int ft_train_batch_plan(size_t sequences, size_t grad_accum_steps, size_t step_in_accum, size_t* chunk_sizes,
+                        size_t* chunks) {
+    FT_CHECK_ARG(chunks && (sequences == 0 || chunk_sizes), "ft_train_batch_plan: NULL argument");
+    size_t n = 0, rest = sequences;
+    while (rest > 0) {
+        size_t room = rest;  // grad_accum_steps 0: the whole batch is one window (ft_trainer_config)
+        if (grad_accum_steps) {
+            room = grad_accum_steps > step_in_accum ? grad_accum_steps - step_in_accum : 0;  // saturating_sub
+            if (room < 1) room = 1;
+            if (room > rest) room = rest;
+            step_in_accum += room;
+            if (step_in_accum >= grad_accum_steps) step_in_accum = 0;  // the chunk that fills the window steps
+        }
+        chunk_sizes[n++] = room;
+        rest -= room;
+    }
+    *chunks = n;
+    return FT_OK;
+}
+
+int ft_chunk_padded_len(const size_t* input_lens, const size_t* target_lens, size_t count, size_t length_bucket,
+                        size_t* padded_len) {
+    FT_CHECK_ARG(padded_len && (count == 0 || (input_lens && target_lens)), "ft_chunk_padded_len: NULL argument");
+    FT_CHECK_ARG(length_bucket >= 1, "ft_chunk_padded_len: length_bucket must be at least 1");
+    size_t longest = 0;
+    for (size_t i = 0; i < count; i++) {
+        const size_t len = input_lens[i] < target_lens[i] ? input_lens[i] : target_lens[i];
+        if (len > longest) longest = len;
+    }
+    *padded_len = (longest + length_bucket - 1) / length_bucket * length_bucket;
+    return FT_OK;
+}
+
+int ft_pad_chunk(const uint32_t* const* input_ids, const uint32_t* const* target_ids, const uint8_t* const* loss_masks,
+                 const size_t* input_lens, const size_t* target_lens, const size_t* mask_lens, size_t count,
+                 size_t padded_len, uint32_t* rows, uint32_t* targets, uint8_t* masks) {
+    FT_CHECK_ARG(count == 0 || (input_ids && target_ids && loss_masks && input_lens && target_lens && mask_lens),
+                 "ft_pad_chunk: NULL argument");
+    FT_CHECK_ARG(count == 0 || padded_len == 0 || (rows && targets && masks), "ft_pad_chunk: NULL output");
+    for (size_t s = 0; s < count; s++) {
+        const size_t len = input_lens[s] < target_lens[s] ? input_lens[s] : target_lens[s];
+        FT_CHECK_ARG(len <= padded_len, "ft_pad_chunk: sequence %zu has %zu tokens, the rows have %zu", s, len, padded_len);
+        FT_CHECK_ARG(len == 0 || (input_ids[s] && target_ids[s]), "ft_pad_chunk: sequence %zu is NULL", s);
+        const uint32_t pad = len ? input_ids[s][len - 1] : 0;  // the row's last token, for inputs and targets alike
+        uint32_t* r = rows + s * padded_len;
+        uint32_t* t = targets + s * padded_len;
+        uint8_t* m = masks + s * padded_len;
+        for (size_t i = 0; i < len; i++) {
+            r[i] = input_ids[s][i];
+            t[i] = target_ids[s][i];
+            m[i] = i < mask_lens[s] && loss_masks[s] ? loss_masks[s][i] : 0;  // loss_mask.get(i).unwrap_or(0)
+        }
+        for (size_t i = len; i < padded_len; i++) {
+            r[i] = pad;
+            t[i] = pad;
+            m[i] = 0;
+        }
+    }
+    return FT_OK;
+}
+
 int ft_trainer_step_in_accum(ft_trainer* t, size_t* sequences) {
     FT_CHECK_ARG(t && sequences, "ft_trainer_step_in_accum: NULL argument");
     *sequences = t->step_in_accum;

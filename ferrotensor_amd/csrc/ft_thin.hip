@@ -367,7 +367,8 @@ int ft_thin_colwise(ft_context* ctx, const ft_thin_problem* probs, int count) {
     const int want_wgs = 2 * ctx->num_cus;   // measured: 1x and 4x are both slower at the 360M shapes
     int slices = want_wgs / tiles;
     if (slices < 1) slices = 1;
-    int rows_per_wg = ((mmax + slices - 1) / slices + quantum / 2) / quantum * quantum;
+    // rounded up to whole batches, so that the last slice is never a sliver of rows
+    int rows_per_wg = ((mmax + slices - 1) / slices + quantum - 1) / quantum * quantum;
     if (rows_per_wg < quantum) rows_per_wg = quantum;
     b.rows_per_wg = rows_per_wg;
     b.rows_per_wave = rows_per_wg / kColWaves;

@@ -221,18 +221,46 @@ def lora_init_a(in_dim: int, out_dim: int, rank: int, seed: int) -> np.ndarray:
 
 
 def pad_chunk(seqs, length_bucket=32):
-    """`Trainer::train_chunk` padding (trainer/src/lib.rs:431-450): right-pad to a
-    multiple of `length_bucket` with each row's last token, loss mask 0."""
-    longest = max(min(len(i), len(t)) for i, t, _ in seqs)
-    padded = -(-longest // length_bucket) * length_bucket
-    rows, targets, masks = [], [], []
-    for ids, tg, mk in seqs:
-        n = min(len(ids), len(tg))
-        pad = ids[n - 1] if n else 0
-        rows.append(list(ids[:n]) + [pad] * (padded - n))
-        targets.append(list(tg[:n]) + [pad] * (padded - n))
-        masks.append([mk[i] if i < len(mk) else 0 for i in range(n)] + [0] * (padded - n))
-    return np.array(rows, np.uint32), np.array(targets, np.uint32), np.array(masks, np.uint8)
+    """`Trainer::train_chunk` padding (trainer/src/lib.rs:431-450) through `ft_chunk_padded_len` and
+    `ft_pad_chunk`: right-pad to a multiple of `length_bucket` with each row's last token, loss mask 0."""
+    lib = _lib.load()
+    n = len(seqs)
+    ids = [np.ascontiguousarray(i, np.uint32) for i, _, _ in seqs]
+    tgs = [np.ascontiguousarray(t, np.uint32) for _, t, _ in seqs]
+    mks = [np.ascontiguousarray(m, np.uint8) for _, _, m in seqs]
+    sizes = lambda arrs: (C.c_size_t * n)(*[a.size for a in arrs])
+    ptrs = lambda arrs: (C.c_void_p * n)(*[a.ctypes.data for a in arrs])
+    il, tl, ml = sizes(ids), sizes(tgs), sizes(mks)
+    padded = C.c_size_t()
+    check(lib.ft_chunk_padded_len(il, tl, n, length_bucket, C.byref(padded)))
+    S = padded.value
+    rows, targets, masks = np.empty((n, S), np.uint32), np.empty((n, S), np.uint32), np.empty((n, S), np.uint8)
+    check(lib.ft_pad_chunk(ptrs(ids), ptrs(tgs), ptrs(mks), il, tl, ml, n, S, rows.ctypes.data_as(C.c_void_p),
+                           targets.ctypes.data_as(C.c_void_p), masks.ctypes.data_as(C.c_void_p)))
+    return rows, targets, masks
+
+
+def select_sequences(input_ids, target_ids, attention_mask, loss_mask):
+    """`Trainer::train_batch`, which rows of a padded `Batch` train (trainer/src/lib.rs:377-395), through
+    `ft_train_batch_select`: the valid length of every row, 0 for a row that is dropped."""
+    a = [np.ascontiguousarray(x, t) for x, t in ((input_ids, np.uint32), (target_ids, np.uint32),
+                                                 (attention_mask, np.uint8), (loss_mask, np.uint8))]
+    B, S = a[0].shape
+    assert all(x.shape == (B, S) for x in a)
+    valid = (C.c_size_t * max(B, 1))()
+    kept = C.c_size_t()
+    check(_lib.load().ft_train_batch_select(*[x.ctypes.data_as(C.c_void_p) for x in a], B, S, valid, C.byref(kept)))
+    out = [valid[b] for b in range(B)]
+    assert sum(1 for v in out if v) == kept.value
+    return out
+
+
+def plan_chunks(sequences: int, grad_accum_steps: int, step_in_accum: int = 0):
+    """`Trainer::train_batch`, where the chunks end (trainer/src/lib.rs:408-421), through `ft_train_batch_plan`."""
+    sizes = (C.c_size_t * max(sequences, 1))()
+    n = C.c_size_t()
+    check(_lib.load().ft_train_batch_plan(sequences, grad_accum_steps, step_in_accum, sizes, C.byref(n)))
+    return [sizes[i] for i in range(n.value)]
 
 
 class Trainer:
@@ -299,13 +327,20 @@ class Trainer:
         they are trained one at a time. One StepStats per chunk; none when nothing is left."""
         kept = [(i, t, m) for i, t, m in seqs if min(len(i), len(t)) >= 2 and any(m[:min(len(i), len(t))])]
         out = []
-        accum = self.grad_accum_steps
-        while kept:
-            room = max(accum - self.step_in_accum, 1) if accum else len(kept)
+        for room in plan_chunks(len(kept), self.grad_accum_steps, self.step_in_accum):
             chunk, kept = kept[:room], kept[room:]
             rows, targets, masks = pad_chunk(chunk, self.length_bucket)
             out.append(self.train_chunk(rows, targets, masks, apply))
         return out
+
+    def train_padded_batch(self, input_ids, target_ids, attention_mask, loss_mask, apply: bool = True) -> List[StepStats]:
+        """`Trainer::train_batch` on a `Batch` as the data loader hands it over (trainer/src/lib.rs:371-423):
+        [batch, padded_len] ids, targets, attention mask and loss mask. Rows are cut at their attention mask,
+        rows that cannot train are dropped (`ft_train_batch_select`), the rest run as `train_batch`."""
+        valid = select_sequences(input_ids, target_ids, attention_mask, loss_mask)
+        seqs = [(np.asarray(input_ids[b])[:n], np.asarray(target_ids[b])[:n], np.asarray(loss_mask[b])[:n])
+                for b, n in enumerate(valid) if n]
+        return self.train_batch(seqs, apply)
 
     def close(self):
         if self.handle is not None and self.handle.value:

@@ -19,10 +19,8 @@
  *    `UnifiedTensor::from_f32_as_f16` (tensor.rs:258-269): element i at byte 2*i.
  *  - Ops only enqueue work on the context's stream and return
  *    (context.rs:291-317); order of execution = order of calls;
- *    `ft_synchronize` waits (context.rs:380-391). The training step also uses a
- *    second stream that the context owns (the LoRA factor gradients run there,
- *    beside the input-gradient GEMMs); it is joined before anything reads them
- *    and by `ft_synchronize` / `ft_download`.
+ *    `ft_synchronize` waits (context.rs:380-391). A context has exactly one
+ *    stream; the training step runs on it from its first kernel to its last.
  *  - Outputs are caller-allocated and written, never accumulated into, except
  *    the in-place ops (rope, gradient_scale, clip_grad_by_norm,
  *    gradient_accumulate, adamw_update), as in the reference.
@@ -490,12 +488,45 @@ int ft_trainer_set_adam_hyper(ft_trainer* t, float lr, float beta1, float beta2,
                               float weight_decay);
 int ft_trainer_optimizer_steps(ft_trainer* t, size_t* steps);
 int ft_trainer_set_optimizer_steps(ft_trainer* t, size_t steps);
+/* ---- Trainer::train_batch and the padding of train_chunk: host-side integer work ----
+ * No device is touched; every array is host memory. */
+
+/* Trainer::train_batch, which sequences of a Batch train (trainer/src/lib.rs:377-395). The batch is
+ * [batch, padded_len] row-major (padded_input_ids, padded_target_ids, attention_mask, loss_masks).
+ * A row is cut where its attention mask first differs from 1; it is dropped (valid_len[b] = 0)
+ * when fewer than 2 tokens remain or no position of the cut loss mask is non-zero. `kept` = rows
+ * with valid_len > 0. (The ids are not read; they are taken so the call mirrors the loop.) */
+int ft_train_batch_select(const uint32_t* input_ids, const uint32_t* target_ids,
+                          const uint8_t* attention_mask, const uint8_t* loss_mask, size_t batch,
+                          size_t padded_len, size_t* valid_len, size_t* kept);
+/* Trainer::train_batch, where the chunks end (trainer/src/lib.rs:408-421): chunk i takes
+ * chunk_sizes[i] of the kept sequences, in order; a chunk stops at the accumulation boundary
+ * (room = max(grad_accum_steps - step_in_accum, 1)), so the optimizer steps after the same
+ * sequence as in the one-at-a-time path. `step_in_accum` is ft_trainer_step_in_accum before the
+ * first chunk. grad_accum_steps 0 (the chunk's own size, ft_trainer_config) gives one chunk.
+ * chunk_sizes must hold `sequences` entries. */
+int ft_train_batch_plan(size_t sequences, size_t grad_accum_steps, size_t step_in_accum,
+                        size_t* chunk_sizes, size_t* chunks);
+/* Trainer::train_chunk, the common row length (trainer/src/lib.rs:431-436): the longest
+ * min(input, target) length rounded up to a multiple of length_bucket (Trainer::length_bucket,
+ * 32 by default, :132). */
+int ft_chunk_padded_len(const size_t* input_lens, const size_t* target_lens, size_t count,
+                        size_t length_bucket, size_t* padded_len);
+/* Trainer::train_chunk, the padding (trainer/src/lib.rs:437-450): sequence s is cut to
+ * min(input_lens[s], target_lens[s]) tokens and right-padded to padded_len with its last input
+ * token (inputs and targets alike), loss mask 0; a loss mask shorter than the sequence counts as 0
+ * past its end. rows / targets / masks are [count, padded_len], ready for ft_trainer_train_chunk. */
+int ft_pad_chunk(const uint32_t* const* input_ids, const uint32_t* const* target_ids,
+                 const uint8_t* const* loss_masks, const size_t* input_lens,
+                 const size_t* target_lens, const size_t* mask_lens, size_t count, size_t padded_len,
+                 uint32_t* rows, uint32_t* targets, uint8_t* masks);
+
 /* Trainer::step_in_accum (trainer/src/lib.rs:463-466): sequences counted into the open
  * accumulation window. train_batch cuts its chunks at grad_accum_steps minus this, so the
  * optimizer steps after the same sequence as in the one-at-a-time path (:413-423). */
 int ft_trainer_step_in_accum(ft_trainer* t, size_t* sequences);
 /* Trainer::train_chunk (trainer/src/lib.rs:426-502) for B equally long rows
- * (already padded; see ft_pad_chunk): forward, masked cross-entropy, backward
+ * (already padded: ft_pad_chunk): forward, masked cross-entropy, backward
  * with seed 1/grad_accum_steps, gradient norm, clip, AdamW. rows/targets are
  * [B,S] u32 and loss_mask [B,S] u8 in host memory; per_sequence_loss (B
  * values) may be NULL. `apply` = 0 stops after backward (gradients readable,

@@ -473,6 +473,36 @@ def pad_chunk(seqs, length_bucket=32):
     return (np.array(rows, np.uint32), np.array(targets, np.uint32), np.array(masks, np.uint8))
 
 
+def select_sequences(attention_mask, loss_mask):
+    """`Trainer::train_batch`, which rows of a `Batch` train (trainer/src/lib.rs:377-395): a row is cut
+    where its attention mask first differs from 1 and dropped when fewer than 2 tokens remain or the cut
+    loss mask has no non-zero entry. Returns the valid length per row (0 = dropped). Integer work."""
+    out = []
+    for attn, mask in zip(attention_mask, loss_mask):
+        n = 0
+        for flag in attn:
+            if flag != 1:
+                break
+            n += 1
+        out.append(n if n >= 2 and any(m != 0 for m in mask[:n]) else 0)
+    return out
+
+
+def plan_chunks(sequences: int, grad_accum_steps: int, step_in_accum: int = 0):
+    """`Trainer::train_batch`, where the chunks end (trainer/src/lib.rs:408-421 with the counter of
+    :486-489): room = max(grad_accum_steps - step_in_accum, 1); the chunk that fills the window resets
+    the counter. Integer work."""
+    sizes, rest = [], sequences
+    while rest > 0:
+        room = min(max(grad_accum_steps - step_in_accum, 1), rest)
+        sizes.append(room)
+        rest -= room
+        step_in_accum += room
+        if step_in_accum >= grad_accum_steps:
+            step_in_accum = 0
+    return sizes
+
+
 def apply_gradients(params, grads, opt: AdamW, stats: "StepStats", clip_grad_norm: Optional[float] = None,
                     scheduler=None):
     """`Trainer::apply_gradients` (trainer/src/lib.rs:296-360): global norm; a non-finite norm

@@ -335,21 +335,18 @@ def test_lora_seed_pinned_values():
 
 
 def test_lora_init_a_is_xorshift64star_uniform():
-    """The generator is the published xorshift64* (Vigna): from state 1 its first output is
-    0x2000001 * 0x2545F4914F6CDD1D mod 2^64 (the three shifts of 1 give 0x2000001). The matrix is
-    uniform in +-1/sqrt(in), differs between seeds and shapes, and is not rank-1."""
-    first_state = 0x2000001
-    first_bits = ((first_state * 0x2545F4914F6CDD1D) & ((1 << 64) - 1)) >> 40
-    # choose seed / dims so that the initial state is exactly 1: seed 0, in = out = rank = 0 is degenerate,
-    # so check through the recurrence instead: state0 = (0 + (in<<32 | out<<8 | rank)) | 1
-    a = rs.lora_init_a(1, 0, 1, 0)             # state0 = (1<<32 | 1) | 1
-    s = (1 << 32) | 1
-    s ^= s >> 12
-    s = (s ^ (s << 25)) & ((1 << 64) - 1)
-    s ^= s >> 27
-    bits = ((s * 0x2545F4914F6CDD1D) & ((1 << 64) - 1)) >> 40
-    assert a[0, 0] == np.float32((np.float32(bits) / np.float32(1 << 24)) * 2 - 1)   # bound = 1 for in_dim 1
-    assert first_bits == 0x47E4CE        # top 24 bits of the textbook first output 0x47E4CE4B896CDD1D
+    """`LoRAAdapter::new_seeded` (graph/src/lib.rs:59-92) at seed 7, in 4, out 3, rank 2. The expected values
+    were worked out apart from the oracle, in C with native wrapping 64-bit arithmetic typed from the Rust:
+    state0 = (7 * 0x9E3779B97F4A7C15 + (4 << 32 | 3 << 8 | 2)) | 1 = 0x538454167b096795, then per element
+    xorshift64* (shifts 12, 25, 27), bits = (state * 0x2545F4914F6CDD1D) >> 40, value = (bits / 2^24 * 2 - 1) / 2.
+    A seed other than 0 pins the golden-ratio mixing of the seed. Beyond that the matrix is uniform in
+    +-1/sqrt(in), differs between seeds and shapes, and is not rank-1."""
+    bits = [0x7b8ec6, 0xb151b4, 0x5238fe, 0x68cc18, 0xaaf8c4, 0xb4f168, 0xfd7741, 0xb72c0e]
+    want = np.array([(np.float32(b) / np.float32(1 << 24) * np.float32(2) - np.float32(1)) * np.float32(0.5)
+                     for b in bits], np.float32).reshape(4, 2)
+    np.testing.assert_array_equal(rs.lora_init_a(4, 3, 2, 7), want)
+    np.testing.assert_allclose(want.reshape(-1), [-0.0173527002, 0.192652941, -0.178817868, -0.0906357765,
+                                                  0.167858362, 0.206808567, 0.49010092, 0.215515971], rtol=1e-7)
     a = rs.lora_init_a(960, 320, 8, rs.lora_seed(3, "k_proj"))
     bound = 1.0 / math.sqrt(960)
     assert a.shape == (960, 8) and np.all(np.abs(a) <= bound) and abs(float(a.mean())) < 0.05 * bound
