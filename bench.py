@@ -374,6 +374,43 @@ def mfma_probe(args):
         "best_single_launch_tflops": best, "runs": runs}))
 
 
+def engine_ops_path(ctx, cfg, w, rows, targets, masks, args, fused_loss):
+    """The same workload through `ferrotensor_amd.engine_step`: every op of the step as its own call of the
+    1:1 ComputeEngine entry point, in the order the reference's autograd tape issues them (six calls per LoRA
+    linear, copy + scale, copy + RoPE, one sum-of-squares / clip / AdamW call per tensor). Same weights, batch
+    and optimizer settings as the fused path; the head runs on every position, as in the reference."""
+    from ferrotensor_amd.engine_step import EngineOpsModel, EngineOpsTrainer
+    eo = EngineOpsModel(ctx, cfg, dict(synthetic_tensors(w)))
+    rng = np.random.default_rng(2)
+    dims = {"q_proj": (w["hidden"], w["hidden"]), "k_proj": (w["hidden"], w["hidden"] // w["heads"] * w["kv"]),
+            "v_proj": (w["hidden"], w["hidden"] // w["heads"] * w["kv"]), "o_proj": (w["hidden"], w["hidden"]),
+            "gate_proj": (w["hidden"], w["ffn"]), "up_proj": (w["hidden"], w["ffn"]), "down_proj": (w["ffn"], w["hidden"])}
+    order = ["q_proj", "k_proj", "v_proj", "o_proj", "gate_proj", "up_proj", "down_proj"]
+    for layer in range(w["layers"]):          # the order lora_factors draws them in: layer by layer
+        for name in order:
+            if name in w["targets"]:
+                i, o = dims[name]
+                a = rng.standard_normal((i, w["rank"]), dtype=np.float32) * np.float32(0.02)
+                b = rng.standard_normal((w["rank"], o), dtype=np.float32) * np.float32(0.02)
+                eo.set_lora(layer, name, a, b, w["alpha"])
+    tr = EngineOpsTrainer(eo, lr=2e-4, weight_decay=0.0, clip_grad_norm=1.0)
+    steps = max(3, args.steps // 4)
+    first_loss = None
+    for _ in range(2):
+        loss, norm, clip = tr.train_chunk(rows, targets, masks)
+        first_loss = loss if first_loss is None else first_loss
+    ctx.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        loss, norm, clip = tr.train_chunk(rows, targets, masks)
+    ctx.synchronize()
+    ms = (time.perf_counter() - t0) / steps * 1e3
+    return {"ms_per_step": ms, "tokens_per_s": w["B"] * w["S"] / (ms * 1e-3), "steps": steps,
+            "engine_calls_per_step": tr.calls, "first_step_loss": first_loss,
+            "note": "1:1 ComputeEngine entry points in the reference's op order, driven from Python over ctypes; "
+                    "loss of its first step next to the fused path's current loss (%.4f, after its own steps)" % fused_loss}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -384,6 +421,10 @@ def main():
                     help="sequences per forward/backward pass (default: the whole batch); gradients accumulate "
                          "over the batch and one optimizer step follows, as `ferrotensor train --batch m --accum B/m`")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--path", default="fused", choices=["fused", "engine-ops"],
+                    help="engine-ops: additionally time the same step composed only of the 1:1 ComputeEngine entry "
+                         "points in the reference's op order (ferrotensor_amd.engine_step) and report it as "
+                         "`engine_ops_path` next to the fused number")
     ap.add_argument("--breakdown", action="store_true", help="print the per-kernel event-time table to stderr")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -495,6 +536,8 @@ def main():
                      "all_gemm_kernels_frac": all_gemm_tf / FP32_MFMA_PEAK_TFLOPS,
                      "gemm_ms_per_step": all_gemm_ms / args.steps, "kernel_ms_per_step": kernel_ms},
     }
+    if args.path == "engine-ops":
+        out["engine_ops_path"] = engine_ops_path(ctx, cfg, w, rows, targets, masks, args, float(st.loss))
     if not args.no_cpu_baseline:
         trainer.close()
         model.close()

@@ -11,9 +11,14 @@
 //! `to_vec` / `synchronize` are the synchronisation points; a tensor's buffer returns to an
 //! exact-size pool on its last drop (tensor.rs:106-115).
 //!
+//! The step driver (`Lfm2Model`, `Trainer`, `train_batch`) is in `step`.
+//!
 //! Not compiled in this repository's build image (it has no Rust toolchain): the signatures come
 //! from the generated `ferrotensor-hip-sys`, whose completeness against the header is tested.
 use ferrotensor_hip_sys as sys;
+
+pub mod step;
+pub use step::{AdamW, Batch, Lfm2Model, LrSchedule, ModelConfig, StepStats, TrainError, Trainer};
 use std::ffi::CStr;
 use std::os::raw::c_void;
 use std::sync::Arc;

@@ -1025,3 +1025,52 @@ def test_out_of_range_token_embeds_as_zero_row(ctx):
     rows = np.array([[1, 2, 999, 4, 5, 6, 7, 8]], np.uint32)
     want, _ = orc.forward(rows)
     assert_close("logits", hip.forward_batch(rows), want)
+
+
+# ---- the step composed of the 1:1 ComputeEngine entry points, in the reference's op order ----
+
+@pytest.mark.parametrize("f16", [False, True])
+def test_engine_ops_step_matches_the_oracle_and_the_fused_driver(ctx, f16):
+    """`ferrotensor_amd.engine_step`: the same step issued op by op as ferrotensor-autograd would (project_2d's
+    six calls per linear, copy + scale, copy + rope, one sum_squares / clip / adamw call per tensor) gives the
+    oracle's loss, gradient norm, clip and post-step weights, i.e. what the fused driver gives."""
+    from ferrotensor_amd.engine_step import EngineOpsModel, EngineOpsTrainer
+    from ferrotensor_amd.trainer import Trainer
+    cfg = tiny_config(f16, tied=True)
+    mods = ["q_proj", "k_proj", "v_proj", "o_proj"]
+    hip, orc = build_pair(ctx, cfg, mods, rank=4, alpha=8.0, seed=21)
+    eo = EngineOpsModel(ctx, cfg, random_model_tensors(cfg, 21))
+    frng = np.random.default_rng(22)          # the factors build_pair drew (seed + 1, same order)
+    prefixes = hip.linear_prefixes(mods)
+    for name in prefixes:
+        i, o = hip.linear_dims(name)
+        a = (frng.standard_normal((i, 4)) * 0.02).astype(np.float32)
+        b = (frng.standard_normal((4, o)) * 0.02).astype(np.float32)
+        parts = name.split(".")      # model.layers.N.self_attn.q_proj
+        eo.set_lora(int(parts[2]), parts[-1], a, b, 8.0)
+    rng = np.random.default_rng(6)
+    B, S = 2, 32
+    rows = rng.integers(0, 256, (B, S)).astype(np.uint32)
+    targets = np.concatenate([rows[:, 1:], rng.integers(0, 256, (B, 1)).astype(np.uint32)], axis=1)
+    masks = np.ones((B, S), np.uint8)
+    masks[0, :5] = 0
+    masks[1, :9] = 0
+    tr = Trainer(hip, lr=1e-3, weight_decay=0.01, clip_grad_norm=0.01)
+    et = EngineOpsTrainer(eo, lr=1e-3, weight_decay=0.01, clip_grad_norm=0.01)
+    opt = rs.AdamW(lr=1e-3, weight_decay=0.01)
+    for step in range(2):
+        want = rs.train_chunk(orc, opt, rows, targets, masks, clip_grad_norm=0.01)
+        st = tr.train_chunk(rows, targets, masks)
+        loss, norm, clip = et.train_chunk(rows, targets, masks)
+        assert want.clip_scale is not None and clip is not None
+        assert_close("loss", [loss], [want.loss])
+        assert_close("grad norm", [norm], [want.grad_norm])
+        assert_close("clip scale", [clip], [want.clip_scale], atol=1e-6)
+        assert_close("loss (fused)", [st.loss], [loss])
+        for n, w in orc.lora_params():
+            parts = n.split(".")     # model.layers.N.self_attn.q_proj.lora_a
+            lo = eo.layers[int(parts[2])][parts[4]].lora
+            got = (lo.a if parts[-1] == "lora_a" else lo.b).to_numpy()
+            assert_close(f"step {step} weight {n}", got.reshape(-1), w.reshape(-1), atol=1e-6, rtol=1e-4)
+    assert et.calls > 200     # op by op: hundreds of engine calls where the fused driver makes a few dozen launches
+

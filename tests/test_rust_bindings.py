@@ -8,7 +8,8 @@ import sys
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 SYS = os.path.join(ROOT, "rust", "ferrotensor-hip-sys")
-SAFE = os.path.join(ROOT, "rust", "ferrotensor-backend-hip", "src", "lib.rs")
+SAFE_DIR = os.path.join(ROOT, "rust", "ferrotensor-backend-hip", "src")
+SAFE = [os.path.join(SAFE_DIR, f) for f in ("lib.rs", "step.rs")]
 
 
 def header_functions():
@@ -37,9 +38,9 @@ def test_sys_crate_declares_every_entry_point():
 
 def test_safe_crate_calls_existing_entry_points_with_the_right_arity():
     want = header_functions()
-    text = open(SAFE).read()
+    text = "\n".join(open(f).read() for f in SAFE)
     calls = list(re.finditer(r"sys::(ft_\w+)\(", text))
-    assert len(calls) >= 40
+    assert len(calls) >= 70
     for m in calls:
         name = m.group(1)
         assert name in want, name
@@ -59,3 +60,21 @@ def test_safe_crate_calls_existing_entry_points_with_the_right_arity():
             i += 1
         n = commas + 1 if any_arg else 0
         assert n == want[name], (name, n, want[name])
+
+
+def test_step_driver_wrappers_cover_the_model_and_trainer_entry_points():
+    """`Lfm2Model` / `Trainer` of step.rs reach every ft_model_* / ft_trainer_* entry point and the host half
+    of train_batch, and carry the reference's method names (ferrotensor-trainer/src/lib.rs:154-213, 228, 371, 426)."""
+    text = open(SAFE[1]).read()
+    called = set(re.findall(r"sys::(ft_\w+)\(", text))
+    want = {n for n in header_functions() if n.startswith(("ft_model_", "ft_trainer_", "ft_train_batch_"))}
+    want |= {"ft_pad_chunk", "ft_chunk_padded_len"}
+    want -= {"ft_model_set_head_all_rows"}   # a benchmark switch, not part of the reference's surface
+    assert want <= called, sorted(want - called)
+    for name in ("with_grad_accum_steps", "with_clip_grad_norm", "with_lr_scheduler", "with_length_bucket",
+                 "train_step_masked", "train_batch", "train_chunk", "set_optimizer_steps", "optimizer_steps",
+                 "forward_batch", "named_params"):
+        assert re.search(r"pub fn %s\(" % name, text), name
+    fields = re.search(r"pub struct StepStats \{(.*?)\}", text, re.S).group(1)
+    for field in ("loss: f32", "tokens: usize", "optimizer_step: bool", "grad_norm: Option<f32>", "lr: Option<f32>"):
+        assert field in fields, field
