@@ -1412,6 +1412,8 @@ int launch_async(ft_context* ctx, AsyncBatch g, int layout, int epi = kEpiPlain)
     bool pairs = false;
     if (epi == kEpiPlain && mn4 && !any_rope && tiles > 0 && (few_tiles || long_k)) {
         int want = (int)((2 * (size_t)ctx->num_cus + tiles - 1) / tiles);
+        // 128x128 tiles hold two workgroups on a CU: the shares must fit one round of them
+        if (BM == 128) want = (int)(2 * (size_t)ctx->num_cus / tiles);
         if (want > 8) want = 8;
         if (want > min_kt / 4) want = min_kt / 4;
         // Many shares (one sequence per pass): the second wave group takes half of them, which
@@ -1538,6 +1540,19 @@ int launch_async_auto(ft_context* ctx, const AsyncBatch& g, int layout) {
     size_t tiles128 = 0;
     for (int i = 0; i < g.count; i++) tiles128 += (size_t)((g.M + 127) / 128) * (size_t)((g.p[i].N + 127) / 128);
     if (tiles128 >= 8 * (size_t)ctx->num_cus) return launch_async<128, 128, 64, 64>(ctx, g, layout);
+    // A very long K over few tiles (the head's input gradient: K = vocabulary): the large tile with its K
+    // tiles shared out runs at the rate of the many-tile case, and the extra pass over the partial tiles is
+    // a fraction of a percent of the product.
+    int min_kt = 1 << 30;
+    bool plain = true;
+    for (int i = 0; i < g.count; i++) {
+        int kt = 0;
+        for (int s = 0; s < g.p[i].nseg; s++) kt += g.p[i].seg[s].nt;
+        min_kt = kt < min_kt ? kt : min_kt;
+        plain = plain && g.p[i].rope == nullptr && ((size_t)g.M * g.p[i].N) % 4 == 0 && g.p[i].ldc == g.p[i].N;
+    }
+    if (plain && min_kt >= 512 && tiles128 * 2 <= 2 * (size_t)ctx->num_cus && tiles128 * 8 >= 2 * (size_t)ctx->num_cus)
+        return launch_async<128, 128, 64, 64>(ctx, g, layout);
     return launch_async<64, 64, 32, 32>(ctx, g, layout);
 }
 
