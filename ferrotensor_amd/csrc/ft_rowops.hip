@@ -5,6 +5,8 @@
 // wave reductions), so HBM traffic equals the algorithmic byte count.
 #include "ft_common.h"
 
+#include <algorithm>
+
 #include <atomic>
 #include <mutex>
 
@@ -839,6 +841,33 @@ __global__ __launch_bounds__(256) void multi_adamw_kernel(const ft_segment* __re
     }
 }
 
+// y[row, col] += bias[col]: the projection bias of `Linear::project_2d` (graph/src/lib.rs:128-139), which the
+// reference writes as ones[rows, 1] @ bias[1, out] added to the product.
+__global__ void __launch_bounds__(256) row_bias_add_kernel(float* __restrict__ y, const float* __restrict__ bias,
+                                                           size_t rows, int cols) {
+    const size_t n = rows * (size_t)cols;
+    for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x)
+        y[i] += bias[i % (size_t)cols];
+}
+
+// out[col] (+)= sum over rows of g[row, col]: ones^T @ g, the bias gradient. One workgroup per 64 columns,
+// four row lanes per column summed in a fixed order, so the result does not depend on the launch.
+__global__ void __launch_bounds__(256) col_sum_kernel(const float* __restrict__ g, float* __restrict__ out,
+                                                      size_t rows, int cols, int accumulate) {
+    __shared__ float part[4][64];
+    const int c = blockIdx.x * 64 + (threadIdx.x & 63);
+    const int lane_row = threadIdx.x >> 6;
+    float acc = 0.0f;
+    if (c < cols)
+        for (size_t r = lane_row; r < rows; r += 4) acc += g[r * (size_t)cols + c];
+    part[lane_row][threadIdx.x & 63] = acc;
+    __syncthreads();
+    if (lane_row == 0 && c < cols) {
+        const float s = (part[0][threadIdx.x] + part[1][threadIdx.x]) + (part[2][threadIdx.x] + part[3][threadIdx.x]);
+        out[c] = accumulate ? out[c] + s : s;
+    }
+}
+
 }  // namespace
 
 // Internal entry points used by the step driver (ft_step.cpp).
@@ -863,6 +892,30 @@ int ft_internal_rms_norm_backward_add(ft_context* ctx, const float* x, const flo
     else
         hipLaunchKernelGGL((rms_norm_backward_wave_kernel<8>), grid, dim3(256), 0, ctx->stream, x, w, g, add, gx,
                            (int)rows, (int)size, eps);
+    FT_LAUNCH_CHECK();
+    return FT_OK;
+}
+
+// y[rows, cols] += bias[cols] on every row.
+int ft_internal_row_bias_add(ft_context* ctx, float* y, const float* bias, size_t rows, size_t cols) {
+    FT_CHECK_ARG(ctx && y && bias, "row_bias_add: NULL argument");
+    FT_CHECK_ARG(cols > 0 && cols < (1u << 30), "row_bias_add: %zu columns", cols);
+    if (rows == 0) return FT_OK;
+    ft_prof_scope prof(ctx, "row_bias_add_kernel", 0.0, 8.0 * (double)rows * cols);
+    const size_t blocks = std::min<size_t>(ft_div_up(rows * cols, 256), 4096);
+    hipLaunchKernelGGL(row_bias_add_kernel, dim3((unsigned)blocks), dim3(256), 0, ctx->stream, y, bias, rows,
+                       (int)cols);
+    FT_LAUNCH_CHECK();
+    return FT_OK;
+}
+
+// out[cols] = (or +=, when `accumulate`) the sum of g[rows, cols] over its rows.
+int ft_internal_col_sum(ft_context* ctx, const float* g, float* out, size_t rows, size_t cols, int accumulate) {
+    FT_CHECK_ARG(ctx && g && out, "col_sum: NULL argument");
+    FT_CHECK_ARG(cols > 0 && cols < (1u << 30), "col_sum: %zu columns", cols);
+    ft_prof_scope prof(ctx, "col_sum_kernel", 0.0, 4.0 * (double)rows * cols);
+    hipLaunchKernelGGL(col_sum_kernel, dim3((unsigned)ft_div_up(cols, 64)), dim3(256), 0, ctx->stream, g, out, rows,
+                       (int)cols, accumulate);
     FT_LAUNCH_CHECK();
     return FT_OK;
 }

@@ -43,6 +43,8 @@ int ft_internal_rope_table(ft_context* ctx, float* table, size_t seq, size_t hea
 int ft_internal_rope_pair(ft_context* ctx, const float* a_src, float* a_dst, size_t heads_a, const float* b_src,
                           float* b_dst, size_t heads_b, const float* table, size_t batch, size_t seq,
                           size_t head_dim, int inverse);
+int ft_internal_row_bias_add(ft_context* ctx, float* y, const float* bias, size_t rows, size_t cols);
+int ft_internal_col_sum(ft_context* ctx, const float* g, float* out, size_t rows, size_t cols, int accumulate);
 bool ft_internal_attention_rope_fusable(const float* q, const float* k, const float* v, const float* out,
                                         const float* d_out, size_t Sq, size_t Sk, size_t D);
 int ft_internal_attention_backward_rope(ft_context* ctx, const float* q, const float* k, const float* v,
@@ -68,6 +70,8 @@ struct LinearW {
     float* ga = nullptr;
     float* gb = nullptr;
     float* gw = nullptr;  // gradient of w [in, out] when the base trains
+    float* bias = nullptr;   // [out], f32 (graph/src/lib.rs:105-106: Qwen2 query, key and value projections)
+    float* gbias = nullptr;  // its gradient when the base trains
     bool has_lora() const { return r > 0; }
     // graph/src/lib.rs:119-122: the scale is alpha / rank, skipped when it is exactly 1.
     float scale() const {
@@ -303,6 +307,11 @@ int rebuild_params(ft_model* m) {
             FT_TRY(grad_buf(&l.gw, l.in * l.out));
             m->params.push_back({l.prefix + ".weight", (float*)l.w, l.gw, l.in * l.out});
         }
+        // Linear::params (graph/src/lib.rs:180-188): weight, bias, then the adapter
+        if (base && l.bias) {
+            FT_TRY(grad_buf(&l.gbias, l.out));
+            m->params.push_back({l.prefix + ".bias", l.bias, l.gbias, l.out});
+        }
         if (!l.has_lora()) return FT_OK;
         m->params.push_back({l.prefix + ".lora_a", l.a, l.ga, l.in * l.r});
         m->params.push_back({l.prefix + ".lora_b", l.b, l.gb, l.r * l.out});
@@ -367,13 +376,24 @@ int linear_gemm_group(ft_context* ctx, LinearW* const* ls, const float* const* t
     return ft_lora_linear_group(ctx, x, d, (size_t)n, T, ls[0]->in);
 }
 
-// y = x @ W (+ (scale * x @ A) @ B) (+ residual), keeping t = scale * x @ A for backward.
+// y += bias on every row, for a linear that has one (graph/src/lib.rs:128-139: added after the adapter).
+int linear_bias(ft_context* ctx, const LinearW& l, float* y, size_t T) {
+    if (!l.bias) return FT_OK;
+    return ft_internal_row_bias_add(ctx, y, l.bias, T, l.out);
+}
+
+// y = x @ W (+ (scale * x @ A) @ B) (+ bias) (+ residual), keeping t = scale * x @ A for backward.
 int linear_forward(ft_context* ctx, LinearW& l, const float* x, float* t, float* y, size_t T,
                    const float* residual = nullptr) {
     LinearW* ls[1] = {&l};
     float* ts[1] = {t};
     FT_TRY(lora_down_group(ctx, ls, ts, 1, x, T));
-    return linear_gemm(ctx, l, x, t, y, T, residual);
+    if (!l.bias) return linear_gemm(ctx, l, x, t, y, T, residual);
+    // the bias belongs to the linear's output, the residual is added to that sum afterwards
+    FT_TRY(linear_gemm(ctx, l, x, t, y, T));
+    FT_TRY(linear_bias(ctx, l, y, T));
+    if (residual) FT_TRY(ft_add(ctx, residual, y, y, T * l.out));
+    return FT_OK;
 }
 
 // Launches the waiting factor-gradient products in batches of equal rank; afterwards every dT
@@ -406,6 +426,8 @@ int take_dt(ft_model* m, float** dt) {
 int linear_backward(ft_model* m, LinearW& l, const float* x, const float* t, const float* dy, float* dx, size_t T,
                     bool accumulate, bool dx_add = false) {
     ft_context* ctx = m->ctx;
+    // the bias gradient is ones^T @ dy, the output gradient summed over the rows
+    if (l.gbias) FT_TRY(ft_internal_col_sum(ctx, dy, l.gbias, T, l.out, accumulate ? 1 : 0));
     if (l.gw) {
         // trainable base: dW[in, out] = x^T @ dy (MatMulNode::backward, autograd/src/lib.rs:280-287)
         float* dst = accumulate ? m->gtmp : l.gw;
@@ -458,8 +480,8 @@ int linear_backward_group(ft_model* m, LinearW* const* ls, const float* const* t
     bool batch = n <= 3;
     bool any_gw = false;
     for (int i = 0; i < n; i++) {
-        batch = batch && ls[i]->has_lora() && ls[i]->r == ls[0]->r && !ls[i]->gw;
-        any_gw = any_gw || ls[i]->gw != nullptr;
+        batch = batch && ls[i]->has_lora() && ls[i]->r == ls[0]->r && !ls[i]->gw && !ls[i]->gbias;
+        any_gw = any_gw || ls[i]->gw != nullptr || ls[i]->gbias != nullptr;
     }
     float* dts[3] = {nullptr, nullptr, nullptr};
     if (batch) {
@@ -526,16 +548,19 @@ int layer_forward(ft_model* m, size_t l, size_t B, size_t S) {
             float* ts[3] = {a.tq, a.tk, a.tv};
             FT_TRY(lora_down_group(ctx, ls, ts, 3, a.h1, T));
         }
+        bool fused_rope = false;
         {
             LinearW* ls[3] = {&L.q, &L.k, &L.v};
             const float* ts[3] = {a.tq, a.tk, a.tv};
             float* ys[3] = {a.q, a.k, a.v};
-            // head_dim 64: q and k leave the GEMM already rotated
-            const bool fused_rope = m->rope_table && D == 64;
+            // head_dim 64: q and k leave the GEMM already rotated (a biased projection is rotated after
+            // its bias, so it takes the separate kernel)
+            fused_rope = m->rope_table && D == 64 && !L.q.bias && !L.k.bias;
             FT_TRY(linear_gemm_group(ctx, ls, ts, ys, 3, a.h1, T, fused_rope ? m->rope_table : nullptr, S,
                                      fused_rope ? 2 : 0));
+            for (int i = 0; i < 3; i++) FT_TRY(linear_bias(ctx, *ls[i], ys[i], T));
         }
-        if (m->rope_table && D == 64) {
+        if (fused_rope) {
         } else if (m->rope_table) {
             FT_TRY(ft_internal_rope_pair(ctx, a.q, a.q, nh, a.k, a.k, nkv, m->rope_table, B, S, D, 0));
         } else {
@@ -551,13 +576,14 @@ int layer_forward(ft_model* m, size_t l, size_t B, size_t S) {
             float* ts[2] = {a.tup, a.tgate};
             FT_TRY(lora_down_group(ctx, ls, ts, 2, a.h2, T));
         }
-        if (!L.up.has_lora() && !L.gate.has_lora() && L.up.dtype == L.gate.dtype) {
+        if (!L.up.has_lora() && !L.gate.has_lora() && L.up.dtype == L.gate.dtype && !L.up.bias && !L.gate.bias) {
             FT_TRY(ft_mlp_gate_up(ctx, a.h2, L.gate.w, L.up.w, L.up.dtype, a.gate, a.up, a.act, T, H, F));
         } else {
             LinearW* ls[2] = {&L.up, &L.gate};
             const float* ts[2] = {a.tup, a.tgate};
             float* ys[2] = {a.up, a.gate};
             FT_TRY(linear_gemm_group(ctx, ls, ts, ys, 2, a.h2, T));
+            for (int i = 0; i < 2; i++) FT_TRY(linear_bias(ctx, *ls[i], ys[i], T));
             FT_TRY(ft_silu_gate_fused(ctx, a.gate, a.up, a.act, T * F));
         }
         FT_TRY(linear_forward(ctx, L.down, a.act, a.tdown, x_next, T, a.h));
@@ -700,7 +726,7 @@ int model_backward(ft_model* m, size_t B, size_t S, bool accumulate) {
             FT_TRY(layer_forward(m, li, B, S));
         }
         // x_next = h + down(silu(gate) * up)
-        if (!L.down.has_lora() && !L.down.gw) {
+        if (!L.down.has_lora() && !L.down.gw && !L.down.gbias) {
             FT_TRY(ft_mlp_down_backward(ctx, g, L.down.w, L.down.dtype, a.gate, a.up, m->d_gate, m->d_up, m->d_act, T,
                                         F, H));
         } else {
@@ -857,6 +883,8 @@ int ft_model_destroy(ft_model* m) {
         rel(l.ga);
         rel(l.gb);
         rel(l.gw);
+        rel(l.bias);
+        rel(l.gbias);
     };
     rel(m->embed);
     rel(m->norm_f);
@@ -894,6 +922,15 @@ int ft_model_set_tensor(ft_model* m, const char* hf_name, const float* data, con
             if (c.tie_word_embeddings) return FT_OK;  // the tied head ignores a separate tensor
             return set_linear_weight(m, m->lm_head, data, shape[0], shape[1]);
         }
+        // build_linear (model_builder.rs:454-469): `<prefix>.bias` must be [out]
+        auto set_bias = [&](LinearW& l) -> int {
+            FT_CHECK_ARG(ndim == 1 && shape[0] == l.out, "%s must be [%zu]", hf_name, l.out);
+            return set_vector(m, &l.bias, data, n, l.out, hf_name);
+        };
+        if (name == "lm_head.bias") {
+            if (c.tie_word_embeddings) return FT_OK;  // the tied head is the embedding alone
+            return set_bias(m->lm_head);
+        }
         const std::string pre = "model.layers.";
         FT_CHECK_ARG(name.compare(0, pre.size(), pre) == 0, "unknown tensor %s", hf_name);
         const size_t dot = name.find('.', pre.size());
@@ -904,6 +941,13 @@ int ft_model_set_tensor(ft_model* m, const char* hf_name, const float* data, con
         const std::string rest = name.substr(dot);
         if (rest == ".input_layernorm.weight") return set_vector(m, &L.norm1, data, n, H, hf_name);
         if (rest == ".post_attention_layernorm.weight") return set_vector(m, &L.norm2, data, n, H, hf_name);
+        const std::string bias_suffix = ".bias";
+        if (rest.size() > bias_suffix.size() &&
+            rest.compare(rest.size() - bias_suffix.size(), bias_suffix.size(), bias_suffix) == 0) {
+            LinearW* l = find_linear(m, name.substr(0, name.size() - bias_suffix.size()));
+            FT_CHECK_ARG(l, "unknown tensor %s", hf_name);
+            return set_bias(*l);
+        }
         const std::string suffix = ".weight";
         FT_CHECK_ARG(rest.size() > suffix.size() && rest.compare(rest.size() - suffix.size(), suffix.size(), suffix) == 0,
                      "unknown tensor %s", hf_name);

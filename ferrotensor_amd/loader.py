@@ -184,13 +184,17 @@ def load_model(ctx, model_dir: str, f16_linears: bool = True, checkpoint_blocks:
     cfg = model_config(config, tied, f16_linears, checkpoint_blocks)
     for l in range(cfg.num_hidden_layers):
         p = "model.layers.%d.self_attn." % l
-        for unsupported in ("q_norm.weight", "k_norm.weight", "q_layernorm.weight", "q_proj.bias"):
+        for unsupported in ("q_norm.weight", "k_norm.weight", "q_layernorm.weight"):
             if weights.has(p + unsupported):
-                raise BuildError("%s%s: per-head norms and projection biases are not supported" % (p, unsupported))
+                raise BuildError("%s%s: per-head norms are not supported" % (p, unsupported))
     model = Lfm2Model(ctx, cfg)
     try:
         for name in expected_tensors(cfg, tied):
             model.set_tensor(name, weights.read(name))
+            # build_linear (model_builder.rs:454-469): a projection with a `<prefix>.bias` tensor gets it
+            bias = name[:-len(".weight")] + ".bias"
+            if ("_proj." in name or name == "lm_head.weight") and weights.has(bias):
+                model.set_tensor(bias, weights.read(bias))
     except Exception:
         model.close()
         raise

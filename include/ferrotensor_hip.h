@@ -392,7 +392,12 @@ int ft_model_destroy(ft_model* m);
  * `model.layers.N.self_attn.q_proj.weight` [out,in], `...input_layernorm.weight`,
  * `model.norm.weight`, `lm_head.weight`), applying the builder's rules
  * (model_builder.rs:400-424, 653-689): linears are transposed to [in,out] and
- * rounded to f16 when cfg.f16_linears; a tied head is the transposed embedding. */
+ * rounded to f16 when cfg.f16_linears; a tied head is the transposed embedding.
+ * `<linear>.bias` [out] (model_builder.rs:454-469, Qwen2's query, key and value projections) is
+ * kept f32 and added to every output row after the adapter's product, before RoPE and the
+ * residual (Linear::project_2d, graph/src/lib.rs:128-139); with cfg.trainable_base it is trained
+ * and listed after `<linear>.weight` (Linear::params, graph/src/lib.rs:180-188). A biased
+ * projection takes separate bias and RoPE kernels instead of the fused GEMM epilogues. */
 int ft_model_set_tensor(ft_model* m, const char* hf_name, const float* data, const size_t* shape, int ndim);
 /* Attaches a LoRA adapter (LoRAAdapter, graph/src/lib.rs:28-98) to the linear
  * named `prefix` (`model.layers.N.self_attn.q_proj`, `lm_head`, ...):

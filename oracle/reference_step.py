@@ -66,6 +66,7 @@ class Linear:
     lora_b: Optional[np.ndarray] = None  # [rank, out]
     alpha: float = 0.0
     rank: int = 0
+    bias: Optional[np.ndarray] = None    # [out] (Qwen2 query, key and value projections)
 
     @property
     def scale(self):
@@ -81,6 +82,10 @@ class Linear:
                 temp = cpu.scale(temp, float(s))
             cache["temp"] = temp
             out = cpu.add(out, cpu.matmul(temp, self.lora_b))
+        if self.bias is not None:
+            # graph/src/lib.rs:128-139: out + ones[rows, 1] @ bias[1, out], i.e. the bias on every row
+            ones = np.ones((x2d.shape[0], 1), np.float32)
+            out = cpu.add(out, cpu.matmul(ones, self.bias.reshape(1, -1)))
         cache["x"] = x2d
         return out
 
@@ -88,6 +93,10 @@ class Linear:
         """MatMulNode / ScaleNode / AddNode rules for the graph above."""
         x = cache["x"]
         dx = None
+        if self.bias is not None and trainable_base:
+            # backward of ones @ bias_row: ones^T @ g, the output gradient summed over the rows
+            ones = np.ones((g.shape[0], 1), np.float32)
+            _acc(grads, name + ".bias", cpu.matmul_at(ones, g).reshape(-1))
         if self.lora_a is not None:
             temp = cache["temp"]
             d_temp = cpu.matmul_bt(g, self.lora_b)          # [M, r]
@@ -139,7 +148,9 @@ class Model:
             w = cpu.transpose(tensors[key])
             if f16_linears:
                 w = cpu.round_f16(w)
-            return Linear(weight=w)
+            # build_linear (model_builder.rs:454-469): `<prefix>.bias` [out] when the checkpoint has it, kept f32
+            bias = tensors.get(key[:-len(".weight")] + ".bias")
+            return Linear(weight=w, bias=None if bias is None else np.ascontiguousarray(bias, np.float32))
 
         blocks = []
         for l in range(config.num_hidden_layers):

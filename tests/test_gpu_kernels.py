@@ -122,6 +122,53 @@ def test_projections_at_the_row_counts_of_the_full_batches(g, name, M, K, N):
     assert_close(f"{name} matmul_bt_f16b", dx.to_numpy()[rows], f64_mm(gy[rows], wr.T), atol=bar, rtol=1e-4)
 
 
+# K loops of one, two and three 32-wide tiles (the pipeline's prologue alone, with the clamped re-read after the
+# last tile), and the shortest shares split-K ever makes (a share holds at least 4 K tiles: K = 256 -> 4 + 4,
+# K = 288 -> 5 + 4, K = 512 -> four shares of 4; K = 832 -> three shares of 5 + 4 + 4 tile pairs on eight waves).
+SHORT_K = [32, 64, 96]
+SMALLEST_SHARES_K = [256, 288, 512, 832]
+
+
+@pytest.mark.parametrize("K", SHORT_K + SMALLEST_SHARES_K)
+@pytest.mark.parametrize("M,N", [(256, 192), (31, 960), (130, 128)])
+def test_f16_weight_products_with_short_k_and_smallest_split_shares(g, M, N, K):
+    """(256, 192) and (130, 128) are a dozen 64x64 tiles or fewer, so K >= 256 is split over workgroups;
+    (31, 960) is one ragged row block."""
+    from ferrotensor_amd import UnifiedTensor
+    ctx, eng = g
+    a, w = rnd(K + N + M, M, K), rnd(K * 2 + N, K, N, scale=0.05)
+    w16 = UnifiedTensor.from_f32_as_f16(ctx, w, [K, N])
+    wr = cpu.round_f16(w)
+    out = empty(ctx, M, N)
+    eng.matmul_f16b(ctx, up(ctx, a), w16, out)
+    assert_close(f"matmul_f16b {M}x{K}x{N}", out.to_numpy(), f64_mm(a, wr), atol=1e-3, rtol=1e-4)
+    # the other operand layout: g[M, N'] @ w[K', N']^T with the short loop over N' = K
+    w2 = rnd(K * 3 + N, N, K, scale=0.05)
+    w2_16 = UnifiedTensor.from_f32_as_f16(ctx, w2, [N, K])
+    dx = empty(ctx, M, N)
+    eng.matmul_bt_f16b(ctx, up(ctx, a), w2_16, dx)
+    assert_close(f"matmul_bt_f16b {M}x{K}x{N}", dx.to_numpy(), f64_mm(a, cpu.round_f16(w2).T), atol=1e-3, rtol=1e-4)
+
+
+@pytest.mark.parametrize("K", [64, 96, 256, 288, 512])
+@pytest.mark.parametrize("M,N", [(256, 128), (132, 260)])
+def test_f32_products_with_short_k_and_smallest_split_shares(g, M, N, K):
+    """The DMA-fed f32 kernel takes K >= 64 (two tiles); (256, 128) is 8 tiles of 64x64, so K >= 256 is split
+    into shares of 4 and 5 tiles; (132, 260) has ragged last tiles both ways. All three operand layouts."""
+    ctx, eng = g
+    a, b = rnd(M * 7 + K, M, K), rnd(N * 3 + K, K, N)
+    want = f64_mm(a, b)
+    out = empty(ctx, M, N)
+    eng.matmul(ctx, up(ctx, a), up(ctx, b), out)
+    assert_close(f"matmul {M}x{K}x{N}", out.to_numpy(), want, atol=1e-3, rtol=1e-4)
+    out = empty(ctx, M, N)
+    eng.matmul_bt(ctx, up(ctx, a), up(ctx, np.ascontiguousarray(b.T)), out)
+    assert_close(f"matmul_bt {M}x{K}x{N}", out.to_numpy(), want, atol=1e-3, rtol=1e-4)
+    out = empty(ctx, M, N)
+    eng.matmul_at(ctx, up(ctx, np.ascontiguousarray(a.T)), up(ctx, b), out)
+    assert_close(f"matmul_at {M}x{K}x{N}", out.to_numpy(), want, atol=1e-3, rtol=1e-4)
+
+
 @pytest.mark.parametrize("M,K,N", [(1536, 2560, 960), (2048, 1024, 960), (1472, 2048, 896)])
 def test_long_k_products_on_eight_waves(g, M, K, N):
     """320 to 512 output tiles of 64x64 and K >= 1024: the workgroup's eight waves share the K loop

@@ -995,6 +995,155 @@ def test_head_dim_64_step_matches_oracle(ctx, checkpoint):
             assert_close(f"step {step} weight {n}", params[n], w, atol=1e-6, rtol=1e-4)
 
 
+def _with_biases(tensors, which, seed):
+    rng = np.random.default_rng(seed)
+    out = dict(tensors)
+    for name, w in tensors.items():
+        if any(name.endswith(m + ".weight") for m in which):
+            out[name[:-len(".weight")] + ".bias"] = (rng.standard_normal(w.shape[0]) * 0.1).astype(np.float32)
+    return out
+
+
+@pytest.mark.parametrize("head_dim_64", [False, True])
+def test_biased_projections_step_matches_oracle(ctx, head_dim_64):
+    """Qwen2-style `q/k/v_proj.bias` (Linear::project_2d, graph/src/lib.rs:128-139): logits, adapter gradients
+    and two optimizer steps against the oracle. With head dim 64 the unbiased model rotates q and k in the
+    GEMM epilogue; the biased one must add the bias first and rotate afterwards."""
+    from ferrotensor_amd.trainer import Lfm2Model, ModelConfig, Trainer
+    if head_dim_64:
+        cfg = ModelConfig(vocab_size=256, hidden_size=192, intermediate_size=256, num_hidden_layers=2,
+                          num_attention_heads=3, num_key_value_heads=1, rms_norm_eps=1e-5, rope_theta=100000.0,
+                          tie_word_embeddings=True, f16_linears=True)
+    else:
+        cfg = tiny_config(False, False)
+    tensors = _with_biases(random_model_tensors(cfg, 41), ("q_proj", "k_proj", "v_proj"), 42)
+    assert sum(k.endswith(".bias") for k in tensors) == 3 * cfg.num_hidden_layers
+    hip = Lfm2Model(ctx, cfg)
+    hip.load_tensors(tensors)
+    ocfg = rs.ModelConfig(cfg.vocab_size, cfg.hidden_size, cfg.intermediate_size, cfg.num_hidden_layers,
+                          cfg.num_attention_heads, cfg.num_key_value_heads, cfg.rms_norm_eps, cfg.rope_theta,
+                          cfg.tie_word_embeddings)
+    orc = rs.Model.from_hf_tensors(ocfg, tensors, f16_linears=cfg.f16_linears)
+    plain = rs.Model.from_hf_tensors(ocfg, {k: v for k, v in tensors.items() if not k.endswith(".bias")},
+                                     f16_linears=cfg.f16_linears)
+    rng = np.random.default_rng(43)
+    for name in hip.linear_prefixes(["q_proj", "k_proj", "v_proj", "o_proj"]):
+        i, o = hip.linear_dims(name)
+        a = (rng.standard_normal((i, 8)) * 0.02).astype(np.float32)
+        b = (rng.standard_normal((8, o)) * 0.02).astype(np.float32)
+        hip.set_lora(name, a, b, 16.0)
+        orc.set_lora(name, a, b, 16.0)
+        plain.set_lora(name, a, b, 16.0)
+    B, S = 2, 64
+    rows = rng.integers(0, 256, (B, S)).astype(np.uint32)
+    targets = np.concatenate([rows[:, 1:], rows[:, :1]], axis=1)
+    masks = np.ones((B, S), np.uint8)
+    masks[:, :5] = 0
+    want_logits, _ = orc.forward(rows)
+    got_logits = hip.forward_batch(rows)
+    assert_close("logits", got_logits, want_logits)
+    # the biases matter at this tolerance: the same model without them is far off
+    assert np.abs(plain.forward(rows)[0] - want_logits).max() > 100 * 1e-4
+    tr = Trainer(hip, lr=1e-3, weight_decay=0.0, clip_grad_norm=1.0)
+    opt = rs.AdamW(lr=1e-3, weight_decay=0.0)
+    for step in range(2):
+        tr.train_chunk(rows, targets, masks, apply=False)
+        grads = hip.grads()
+        assert not any(n.endswith(".bias") for n in grads)   # frozen with the base
+        want_stats, _, want_grads = rs.train_chunk(orc, opt, rows, targets, masks, clip_grad_norm=1.0,
+                                                   return_grads=True)
+        cs = want_stats.clip_scale or 1.0
+        for n in grads:
+            assert_close(f"step {step} grad {n}", grads[n], want_grads[n] / np.float32(cs))
+        st = tr.train_chunk(rows, targets, masks)
+        assert_close("loss", [st.loss], [want_stats.loss])
+        assert_close("grad_norm", [st.grad_norm], [want_stats.grad_norm])
+        params = hip.params()
+        for n, w in orc.lora_params():
+            assert_close(f"step {step} weight {n}", params[n], w, atol=1e-6, rtol=1e-4)
+
+
+def test_model_directory_with_biases_loads_them(ctx, fx, golden_dir, tmp_path):
+    """`load_model` on a directory whose q/k/v projections have `.bias` tensors (build_linear,
+    model_builder.rs:454-469): the logits are the oracle's for the biased model; a bias of the wrong length
+    is refused."""
+    import os
+    import shutil
+    from ferrotensor_amd import checkpoint as ck
+    from ferrotensor_amd import loader
+    from ferrotensor_amd._lib import FtError
+    tensors = _with_biases(fx.model, ("q_proj", "k_proj", "v_proj"), 9)
+    d = tmp_path / "biased"
+    d.mkdir()
+    shutil.copy(os.path.join(golden_dir, "gradient_parity", "config.json"), d / "config.json")
+    ck.write_safetensors(str(d / "model.safetensors"), tensors, {})
+    model = loader.load_model(ctx, str(d), f16_linears=False)
+    rows = fx.case("batch")[0]
+    want, _ = rs.Model.from_hf_tensors(fx.config, tensors).forward(rows)
+    assert worst_ratio(model.forward_batch(rows), want) <= 1.0
+    plain, _ = rs.Model.from_hf_tensors(fx.config, fx.model).forward(rows)
+    assert worst_ratio(plain, want) > 10.0
+    bad = dict(tensors)
+    bad["model.layers.0.self_attn.k_proj.bias"] = np.zeros(7, np.float32)
+    d2 = tmp_path / "bad"
+    d2.mkdir()
+    shutil.copy(os.path.join(golden_dir, "gradient_parity", "config.json"), d2 / "config.json")
+    ck.write_safetensors(str(d2 / "model.safetensors"), bad, {})
+    with pytest.raises(FtError, match="k_proj.bias must be"):
+        loader.load_model(ctx, str(d2), f16_linears=False)
+
+
+def test_trainable_biases_on_every_linear_match_oracle(ctx, fx):
+    """Every linear biased (lm_head too) and the base trainable: the bias gradients (ones^T @ dy) and all the
+    others against the oracle, accumulated over two micro-batches, then one optimizer step moves the biases.
+    Parameter order within a linear is weight, bias, adapter (Linear::params, graph/src/lib.rs:180-188)."""
+    from ferrotensor_amd.trainer import Lfm2Model, ModelConfig, Trainer
+    c = fx.config
+    every = ("q_proj", "k_proj", "v_proj", "o_proj", "gate_proj", "up_proj", "down_proj", "lm_head")
+    tensors = _with_biases(fx.model, every, 3)
+    cfg = ModelConfig(c.vocab_size, c.hidden_size, c.intermediate_size, c.num_hidden_layers,
+                      c.num_attention_heads, c.num_key_value_heads, c.rms_norm_eps, c.rope_theta,
+                      c.tie_word_embeddings, False, trainable_base=True)
+    hip = Lfm2Model(ctx, cfg)
+    hip.load_tensors(tensors)
+    orc = rs.Model.from_hf_tensors(c, tensors)
+    for name in hip.linear_prefixes(list(every)):
+        hip.set_lora(name, fx.adapters[name + ".lora_a"], fx.adapters[name + ".lora_b"], fx.meta["lora_alpha"])
+        orc.set_lora(name, fx.adapters[name + ".lora_a"], fx.adapters[name + ".lora_b"], fx.meta["lora_alpha"])
+    rows, targets, masks, _, _ = fx.case("full")
+    logits, cache = orc.forward(rows, trainable_base=True)
+    loss, _, grad_logits = rs.masked_cross_entropy_batch(logits, targets, masks, rows.shape[0])
+    want = orc.backward(grad_logits, cache)
+    assert len(want) == 65
+    tr = Trainer(hip, lr=1e-3, weight_decay=0.0, grad_accum_steps=1)
+    st = tr.train_chunk(rows, targets, masks, apply=False)
+    grads = hip.grads()
+    assert set(grads) == set(want)
+    names = list(grads)
+    i = names.index("model.layers.0.self_attn.q_proj.weight")
+    assert names[i + 1:i + 4] == ["model.layers.0.self_attn.q_proj.bias", "model.layers.0.self_attn.q_proj.lora_a",
+                                  "model.layers.0.self_attn.q_proj.lora_b"]
+    assert worst_ratio([st.loss], [loss]) <= 1.0
+    for n in want:
+        assert worst_ratio(grads[n], want[n]) <= 1.0, n
+    # two one-sequence micro-batches accumulate to half the two-sequence gradients (seed 1/2 each)
+    hip2 = Lfm2Model(ctx, cfg)
+    hip2.load_tensors(tensors)
+    for name in hip2.linear_prefixes(list(every)):
+        hip2.set_lora(name, fx.adapters[name + ".lora_a"], fx.adapters[name + ".lora_b"], fx.meta["lora_alpha"])
+    tr2 = Trainer(hip2, lr=1e-3, weight_decay=0.0, grad_accum_steps=2)
+    assert not tr2.train_chunk(rows[:1], targets[:1], masks[:1]).optimizer_step
+    tr2.train_chunk(rows[1:], targets[1:], masks[1:], apply=False)
+    parts = hip2.grads()
+    for n in want:
+        if n.endswith(".bias"):
+            assert worst_ratio(parts[n], want[n] * np.float32(0.5)) <= 1.0, n
+    before = hip.params()
+    assert tr.train_chunk(rows, targets, masks).optimizer_step
+    after = hip.params()
+    assert all(not np.array_equal(before[n], after[n]) for n in want if n.endswith(".bias"))
+
+
 def test_targets_masking_is_bit_exact_against_oracle(ctx):
     """Skipped rows (mask 0 or target >= vocab) contribute exactly nothing:
     the loss equals the oracle's and flipping masked targets changes no bit."""
