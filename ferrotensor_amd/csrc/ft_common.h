@@ -88,4 +88,16 @@ int ft_internal_noalloc_init(int device);
 // Reports a launch-configuration error of the kernel just enqueued.
 #define FT_LAUNCH_CHECK() FT_HIP(hipGetLastError())
 
+// A wave-uniform kernel argument fetched once and kept in a register: the empty asm makes the value opaque,
+// so the compiler can neither fetch it again from the argument block in front of every use (a scalar load
+// and a full wait each time, inside unrolled loops) nor move the fetch into the branches that use it.
+// Pointers lose their address space on the way: cast them to ft_global_f (device memory) afterwards so
+// that their accesses stay `global_*` instructions.
+typedef __attribute__((address_space(1))) float ft_global_f;
+template <typename T>
+__device__ __forceinline__ T ft_pinned(T v) {
+    asm("" : "+s"(v));
+    return v;
+}
+
 static inline unsigned ft_div_up(size_t a, size_t b) { return (unsigned)((a + b - 1) / b); }

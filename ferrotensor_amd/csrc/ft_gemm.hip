@@ -640,7 +640,16 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(SplitReduceArgs a) {
 // Output elements leave with the non-temporal hint: nobody in this launch reads them again, and
 // lines that do not linger dirty in L2 shorten the write-back at the end of the kernel
 // (0.5-1 us per launch, measured).
-__device__ __forceinline__ void store_streaming(float* dst, float v) { __builtin_nontemporal_store(v, dst); }
+template <typename P>
+__device__ __forceinline__ void store_streaming(P* dst, float v) { __builtin_nontemporal_store(v, dst); }
+
+typedef ft_global_f GlobalF;
+typedef float CosSin __attribute__((ext_vector_type(2)));
+typedef __attribute__((address_space(1))) CosSin GlobalF2;
+template <typename T>
+__device__ __forceinline__ T pinned(T v) {
+    return ft_pinned(v);
+}
 
 // KW = 2: eight waves; a stage holds two consecutive K tiles and waves 4-7 multiply the second
 // one of every stage for the same 64x64 output tile (the two sums meet in LDS after the loop):
@@ -681,24 +690,125 @@ __global__ __launch_bounds__(256 * KW) void gemm_async_kernel(AsyncBatch g) {
     // panel row block after row block. Consecutive workgroup ids go to different XCDs, each with
     // its own L2: XCD x takes the x-th contiguous chunk of that order, so the workgroups resident
     // on one XCD cover a compact block of rows and columns and share their operand tiles in L2.
+    // The scalars of the argument block this workgroup needs are fetched in two batches (the header,
+    // then the product's entry) and pinned in registers. Left to itself the compiler fetches each of them
+    // again in front of every use (a scalar load and a full wait per element of the epilogue loops),
+    // which held every workgroup of a launch for microseconds before its first tile request.
+    // (All the reads first, then all the pins: a pin waits for its value, and a wait in front of a
+    // later read would make two round trips of one.)
+    const int r_xcds = g.xcds, r_tiles_m = g.tiles_m,
+              r_tiles_n = g.tiles_n, r_panel = g.panel, r_count = g.count, r_splits = g.splits,
+              r_begin1 = g.p[1].tile_begin, r_begin2 = g.p[2].tile_begin, r_M = g.M;
+    float* const r_partial = g.partial;
+    // (The pointers are device memory: saying so keeps their loads and stores `global_*` instructions
+    // once the pinning has hidden where they came from.)
+    struct SegRegs {
+        const char* a;
+        const char* b;
+        const float* a2;
+        int lda, ldb, nt;
+    };
+    struct ProbRegs {
+        const AsyncSeg* seg;
+        GlobalF* out;
+        const GlobalF* add;
+        const void* b_alt;
+        GlobalF* out2;
+        GlobalF* out3;
+        const GlobalF* e1;
+        const GlobalF* e2;
+        int N, ldc, tile_begin, nseg;
+        long partial_off;
+        const GlobalF2* rope;
+        int rope_seq;
+        SegRegs sr[NSEG];
+    };
+    struct RawProb {
+        float* out;
+        const float* add;
+        const void* b_alt;
+        float* out2;
+        float* out3;
+        const float* e1;
+        const float* e2;
+        int N, ldc, tile_begin, nseg;
+        long partial_off;
+        const float2* rope;
+        int rope_seq;
+        const void* sa[NSEG];
+        const void* sb[NSEG];
+        const float* sa2[NSEG];
+        int slda[NSEG], sldb[NSEG], snt[NSEG];
+    };
+    auto read_prob = [&](const AsyncProb& pk) {
+        RawProb q{pk.out, pk.add, pk.b_alt, pk.out2, pk.out3, pk.e1, pk.e2, pk.N, pk.ldc, pk.tile_begin, pk.nseg,
+                  pk.partial_off, pk.rope, pk.rope_seq, {}, {}, {}, {}, {}, {}};
+#pragma unroll
+        for (int s = 0; s < NSEG; s++) {  // every slot is read (unused ones are zero), so the offsets are constants
+            const AsyncSeg& sg = pk.seg[s];
+            q.sa[s] = sg.a;
+            q.sb[s] = sg.b;
+            q.sa2[s] = sg.a2;
+            q.slda[s] = sg.lda;
+            q.sldb[s] = sg.ldb;
+            q.snt[s] = sg.nt;
+        }
+        return q;
+    };
+    auto pin_prob = [&](const AsyncProb& pk, const RawProb& r) {
+        ProbRegs q{pk.seg,
+                   (GlobalF*)pinned(r.out),
+                   (const GlobalF*)pinned(r.add),
+                   EPI == kEpiGateUp ? pinned(r.b_alt) : nullptr,
+                   EPI != kEpiPlain ? (GlobalF*)pinned(r.out2) : nullptr,
+                   EPI == kEpiGateUp ? (GlobalF*)pinned(r.out3) : nullptr,
+                   EPI == kEpiSiluBwd ? (const GlobalF*)pinned(r.e1) : nullptr,
+                   EPI == kEpiSiluBwd ? (const GlobalF*)pinned(r.e2) : nullptr,
+                   pinned(r.N),
+                   pinned(r.ldc),
+                   pinned(r.tile_begin),
+                   pinned(r.nseg),
+                   pinned(r.partial_off),
+                   (const GlobalF2*)pinned(r.rope),
+                   pinned(r.rope_seq),
+                   {}};
+#pragma unroll
+        for (int s = 0; s < NSEG; s++)
+            q.sr[s] = SegRegs{reinterpret_cast<const char*>(pinned(r.sa[s])), reinterpret_cast<const char*>(pinned(r.sb[s])),
+                              pinned(r.sa2[s]), pinned(r.slda[s]), pinned(r.sldb[s]), pinned(r.snt[s])};
+        return q;
+    };
+    // The first product's entry sits at a constant offset: it is fetched with the header, and only a
+    // workgroup of a later product of the batch pays a second round trip to the argument block.
+    const RawProb raw0 = read_prob(g.p[0]);
+    const int g_xcds = pinned(r_xcds);
+    const int g_tiles_m = pinned(r_tiles_m), g_tiles_n = pinned(r_tiles_n), g_panel = pinned(r_panel);
+    const int g_count = pinned(r_count), g_splits = pinned(r_splits);
+    const int begin1 = pinned(r_begin1), begin2 = pinned(r_begin2);
+    const int M = pinned(r_M);
+    GlobalF* const g_partial = (GlobalF*)pinned(r_partial);
+    ProbRegs p = pin_prob(g.p[0], raw0);
     int bid = (int)blockIdx.x;
-    if (g.xcds > 1) {
-        const int total = (int)gridDim.x, x = bid % g.xcds, q = total / g.xcds, r = total % g.xcds;
-        bid = x * q + (x < r ? x : r) + bid / g.xcds;
+    if (g_xcds == 8) {  // (8 or 1: shifts instead of divisions on the way to the first tile request)
+        const int total = g_tiles_m * g_tiles_n;
+        const int x = bid & 7, q = total >> 3, r = total & 7;
+        bid = x * q + (x < r ? x : r) + (bid >> 3);
     }
-    const int per_panel = g.tiles_m * g.panel;
-    const int last = (g.tiles_n - 1) / g.panel;
-    int pnl = bid / per_panel;
-    pnl = pnl < last ? pnl : last;
-    const int rem = bid - pnl * per_panel;
-    const int width = pnl == last ? g.tiles_n - last * g.panel : g.panel;
-    const int tm = rem / width;
-    const int tn = pnl * g.panel + rem % width;
+    int tm, tn;
+    {
+        const int per_panel = g_tiles_m * g_panel;
+        const int last = (g_tiles_n - 1) / g_panel;
+        int pnl = bid / per_panel;
+        pnl = pnl < last ? pnl : last;
+        const int rem = bid - pnl * per_panel;
+        const int width = pnl == last ? g_tiles_n - last * g_panel : g_panel;
+        tm = rem / width;
+        tn = pnl * g_panel + rem % width;
+    }
     int pi = 0;
-    if (g.count > 1 && tn >= g.p[1].tile_begin) pi = 1;
-    if (g.count > 2 && tn >= g.p[2].tile_begin) pi = 2;
-    const AsyncProb& p = g.p[pi];
-    const int M = g.M;
+    if (g_count > 1 && tn >= begin1) pi = 1;
+    if (g_count > 2 && tn >= begin2) pi = 2;
+    if (pi != 0) p = pin_prob(g.p[pi], read_prob(g.p[pi]));
     const int m0 = tm * BM;
     const int n0 = (tn - p.tile_begin) * BN;
     const int lane = threadIdx.x % 64, wave = (threadIdx.x / 64) % 4;
@@ -714,40 +824,6 @@ __global__ __launch_bounds__(256 * KW) void gemm_async_kernel(AsyncBatch g) {
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
 
-    // Epilogue operands (the residual of `out = a@b + add`, gate and up of the SiLU-gate
-    // backward) are fetched before the K loop: their latency would otherwise be paid after the
-    // last MFMA, when the workgroups of a CU all finish together. Older than every tile load, so
-    // the loop's vmcnt waits cover them.
-    constexpr bool PRE = BM == 64 && BN == 64 && NSEG == 1 && (EPI == kEpiPlain || EPI == kEpiSiluBwd);
-    float pre1[PRE ? 16 : 1], pre2[PRE ? 16 : 1];  // plain: residual | (cos, sin); SiLU backward: gate, up
-    bool pre_add = false;
-    if constexpr (PRE) {
-        const float* s1 = EPI == kEpiSiluBwd ? p.e1 : p.add;
-        pre_add = grp == 0 && (EPI == kEpiSiluBwd || (p.add != nullptr && g.splits == 1 && p.rope == nullptr));
-        if (pre_add) {
-            const int col = n0 + wn0 + l32;
-#pragma unroll
-            for (int r = 0; r < 16; r++) {
-                const int row = m0 + wm0 + (r / 4) * 8 + half * 4 + (r % 4);
-                const bool ok = row < M && col < p.N;
-                const long o = (long)row * p.ldc + col;
-                pre1[r] = ok ? s1[o] : 0.0f;
-                if constexpr (EPI == kEpiSiluBwd) pre2[r] = ok ? p.e2[o] : 0.0f;
-            }
-        }
-        if constexpr (EPI == kEpiPlain) {
-            if (p.rope) {  // the rotation's (cos, sin) of this lane's 16 rows
-#pragma unroll
-                for (int r = 0; r < 16; r++) {
-                    const int row = m0 + wm0 + (r / 4) * 8 + half * 4 + (r % 4);
-                    const float2 cs = p.rope[(long)(row % p.rope_seq) * 32 + l32];
-                    pre1[r] = cs.x;
-                    pre2[r] = cs.y;
-                }
-            }
-        }
-    }
-
     // Uniform description of the segments (a missing one repeats the last: never reached).
     const char* abase[NSEG];
     const char* bbase[NSEG];
@@ -755,9 +831,9 @@ __global__ __launch_bounds__(256 * KW) void gemm_async_kernel(AsyncBatch g) {
     bool has_ext[NSEG];
 #pragma unroll
     for (int s = 0; s < NSEG; s++) {
-        const AsyncSeg& sg = p.seg[s < p.nseg ? s : 0];
-        abase[s] = reinterpret_cast<const char*>(sg.a);
-        bbase[s] = reinterpret_cast<const char*>(sg.b);
+        const SegRegs& sg = p.sr[s < p.nseg ? s : 0];
+        abase[s] = sg.a;
+        bbase[s] = sg.b;
         lda_b[s] = sg.lda * 4;
         ldb_b[s] = sg.ldb * 2;
         tend[s] = (s > 0 ? tend[s - 1] : 0) + (s < p.nseg ? sg.nt : 0);
@@ -768,25 +844,13 @@ __global__ __launch_bounds__(256 * KW) void gemm_async_kernel(AsyncBatch g) {
     // (KW = 2: counted in pairs of tiles; the host only chooses it when every segment has an even number.)
     const int nt_all = tend[NSEG - 1] / KW;
     const int split = (int)blockIdx.y;
-    const int t0 = (int)(((long)nt_all * split) / g.splits);
-    const int nt = (int)(((long)nt_all * (split + 1)) / g.splits);
+    const int nsplit = g_splits;
+    // (32-bit: at most 2^15 K tiles and 8 shares; most launches have one share)
+    const int t0 = nsplit == 1 ? 0 : (int)((unsigned)(nt_all * split) / (unsigned)nsplit);
+    const int nt = nsplit == 1 ? nt_all : (int)((unsigned)(nt_all * (split + 1)) / (unsigned)nsplit);
     if (split > 0) {
 #pragma unroll
         for (int s = 0; s < NSEG; s++) has_ext[s] = false;  // the rank-r term is added once, by share 0
-    }
-
-    // The rank-r products' operands: ordinary loads, issued first, consumed last.
-    ExA xa[NSEG];
-    ExB xb[NSEG];
-#pragma unroll
-    for (int s = 0; s < NSEG; s++) {
-        if (has_ext[s]) {
-            const AsyncSeg& sg = p.seg[s];
-            xa[s].set_offsets(sg.lda2, m0, M, 4);
-            xb[s].set_offsets(sg.ldb2, n0, p.N, 4);
-            xa[s].template load<float, true>(reinterpret_cast<const char*>(sg.a2), 0, sg.K2);
-            xb[s].template load<float, true>(reinterpret_cast<const char*>(sg.b2), 0, sg.K2);
-        }
     }
 
     // Per-lane source coordinates: byte offset = row * (leading dimension in
@@ -926,6 +990,55 @@ __global__ __launch_bounds__(256 * KW) void gemm_async_kernel(AsyncBatch g) {
     // Prologue: tiles t0 .. t0+2 requested, the first one landed, its first fragments read.
     issue(t0, St0);
     issue(t0 + 1, St1);
+    // Epilogue operands (the residual of `out = a@b + add`, gate and up of the SiLU-gate backward,
+    // the rotation's cos and sin) are requested here, behind the first two tiles and in front of the
+    // K loop: after the last MFMA their latency would be paid when the workgroups of a CU all finish
+    // together. The loop's vmcnt waits cover them (they are older than every later tile request).
+    // Out-of-range elements read element 0 instead of branching around the load.
+    constexpr bool PRE = BM == 64 && BN == 64 && NSEG == 1 && (EPI == kEpiPlain || EPI == kEpiSiluBwd);
+    float2 pre[PRE ? 16 : 1];  // plain: .x = residual, or (cos, sin); SiLU backward: (gate, up)
+    bool pre_add = false;
+    if constexpr (PRE) {
+        const GlobalF* s1 = EPI == kEpiSiluBwd ? p.e1 : p.add;
+        pre_add = grp == 0 && (EPI == kEpiSiluBwd || (p.add != nullptr && g_splits == 1 && p.rope == nullptr));
+        bool rotated = false;
+        if constexpr (EPI == kEpiPlain) rotated = p.rope != nullptr;
+        if (rotated) {  // the rotation's (cos, sin) of this lane's 16 rows (never together with a residual)
+            const int pos0 = (m0 + wm0 + half * 4) % p.rope_seq;  // one division; the rows follow by steps < 64
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                int pos = pos0 + (r / 4) * 8 + (r % 4);
+                if (pos >= p.rope_seq) pos -= p.rope_seq;
+                if (pos >= p.rope_seq) pos %= p.rope_seq;  // sequences shorter than a tile
+                const CosSin cs = p.rope[(long)pos * 32 + l32];
+                pre[r] = make_float2(cs.x, cs.y);
+            }
+        } else if (pre_add) {
+            const int col = n0 + wn0 + l32;
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int row = m0 + wm0 + (r / 4) * 8 + half * 4 + (r % 4);
+                const long o = row < M && col < p.N ? (long)row * p.ldc + col : 0;
+                pre[r].x = s1[o];
+                if constexpr (EPI == kEpiSiluBwd) pre[r].y = p.e2[o];
+            }
+        }
+    }
+
+    // The rank-r products' operands: ordinary loads, consumed last.
+    ExA xa[NSEG];
+    ExB xb[NSEG];
+#pragma unroll
+    for (int s = 0; s < NSEG; s++) {
+        if (has_ext[s]) {
+            const AsyncSeg& sg = p.seg[s];
+            xa[s].set_offsets(sg.lda2, m0, M, 4);
+            xb[s].set_offsets(sg.ldb2, n0, p.N, 4);
+            xa[s].template load<float, true>(reinterpret_cast<const char*>(sg.a2), 0, sg.K2);
+            xb[s].template load<float, true>(reinterpret_cast<const char*>(sg.b2), 0, sg.K2);
+        }
+    }
+
     __builtin_amdgcn_s_waitcnt(0x0F70 | (WAIT & 15) | ((WAIT >> 4) << 14));
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_sched_barrier(0);
@@ -999,8 +1112,12 @@ __global__ __launch_bounds__(256 * KW) void gemm_async_kernel(AsyncBatch g) {
                 const int row = m0 + wm0 + (r / 4) * 8 + half * 4 + (r % 4);
                 if (row < M && col < p.N) {
                     float2 cs;
-                    if constexpr (PRE) cs = make_float2(pre1[r], pre2[r]);
-                    else cs = p.rope[(long)(row % p.rope_seq) * 32 + l32];
+                    if constexpr (PRE) {
+                        cs = pre[r];
+                    } else {
+                        const CosSin t = p.rope[(long)(row % p.rope_seq) * 32 + l32];
+                        cs = make_float2(t.x, t.y);
+                    }
                     const float self = acc[0][0][r], peer = other[r * 64 + lane];
                     // lower: x1*c - x2*s ; upper: x1*s + x2*c  (x1 = lower half, x2 = upper half)
                     p.out[(long)row * p.ldc + col] = upper ? peer * cs.y + self * cs.x : self * cs.x - peer * cs.y;
@@ -1010,39 +1127,54 @@ __global__ __launch_bounds__(256 * KW) void gemm_async_kernel(AsyncBatch g) {
         }
     }
 
+    // What becomes of a finished element is the same for the whole workgroup: chosen once, outside the loops.
+    auto emit_all = [&](auto&& emit) {
 #pragma unroll
-    for (int i = 0; i < FM; i++)
+        for (int i = 0; i < FM; i++)
 #pragma unroll
-        for (int j = 0; j < FN; j++) {
-            const int col = n0 + wn0 + j * 32 + l32;
-            if (col >= p.N) continue;
+            for (int j = 0; j < FN; j++) {
+                const int col = n0 + wn0 + j * 32 + l32;
+                if (col >= p.N) continue;
 #pragma unroll
-            for (int r = 0; r < 16; r++) {
-                const int row = m0 + wm0 + i * 32 + (r / 4) * 8 + half * 4 + (r % 4);
-                if (row < M) {
-                    const long o = (long)row * p.ldc + col;
-                    if (EPI == kEpiPlain && g.splits > 1) {
-                        g.partial[p.partial_off + ((long)split * M + row) * p.N + col] = acc[i][j][r];
-                    } else if constexpr (EPI == kEpiGateUp) {
-                        const float up = acc[i][j][r], x = acc[i][FN + j][r];
-                        store_streaming(&p.out[o], up);
-                        store_streaming(&p.out2[o], x);
-                        store_streaming(&p.out3[o], x * (1.0f / (1.0f + __expf(-x))) * up);
-                    } else if constexpr (EPI == kEpiSiluBwd) {
-                        const float d = acc[i][j][r], x = pre1[r], y = pre2[r];
-                        const float sg = 1.0f / (1.0f + __expf(-x));
-                        store_streaming(&p.out2[o], d * (x * sg));
-                        store_streaming(&p.out[o], d * y * (sg * (1.0f + x * (1.0f - sg))));
-                    } else {
-                        if constexpr (PRE) {
-                            store_streaming(&p.out[o], pre_add ? acc[i][j][r] + pre1[r] : (p.add ? acc[i][j][r] + p.add[o] : acc[i][j][r]));
-                        } else {
-                            store_streaming(&p.out[o], p.add ? acc[i][j][r] + p.add[o] : acc[i][j][r]);
-                        }
-                    }
+                for (int r = 0; r < 16; r++) {
+                    const int row = m0 + wm0 + i * 32 + (r / 4) * 8 + half * 4 + (r % 4);
+                    if (row < M) emit(i, j, r, row, col);
                 }
             }
-        }
+    };
+    if constexpr (EPI == kEpiGateUp) {
+        emit_all([&](int i, int j, int r, int row, int col) {
+            const long o = (long)row * p.ldc + col;
+            const float up = acc[i][j][r], x = acc[i][FN + j][r];
+            store_streaming(&p.out[o], up);
+            store_streaming(&p.out2[o], x);
+            store_streaming(&p.out3[o], x * (1.0f / (1.0f + __expf(-x))) * up);
+        });
+    } else if constexpr (EPI == kEpiSiluBwd) {
+        emit_all([&](int i, int j, int r, int row, int col) {
+            const long o = (long)row * p.ldc + col;
+            const float d = acc[i][j][r], x = pre[r].x, y = pre[r].y;
+            const float sg = 1.0f / (1.0f + __expf(-x));
+            store_streaming(&p.out2[o], d * (x * sg));
+            store_streaming(&p.out[o], d * y * (sg * (1.0f + x * (1.0f - sg))));
+        });
+    } else if (g_splits > 1) {
+        GlobalF* dst = g_partial + p.partial_off + (long)split * M * p.N;
+        emit_all([&](int i, int j, int r, int row, int col) { dst[(long)row * p.N + col] = acc[i][j][r]; });
+    } else if (PRE && pre_add) {
+        emit_all([&](int i, int j, int r, int row, int col) {
+            store_streaming(&p.out[(long)row * p.ldc + col], acc[i][j][r] + pre[PRE ? r : 0].x);
+        });
+    } else if (p.add) {
+        emit_all([&](int i, int j, int r, int row, int col) {
+            const long o = (long)row * p.ldc + col;
+            store_streaming(&p.out[o], acc[i][j][r] + p.add[o]);
+        });
+    } else {
+        emit_all([&](int i, int j, int r, int row, int col) {
+            store_streaming(&p.out[(long)row * p.ldc + col], acc[i][j][r]);
+        });
+    }
 }
 
 // ---------------------------------------------------------------------------
@@ -1342,6 +1474,8 @@ __global__ __launch_bounds__(256) void mfma_probe_kernel(float* __restrict__ out
 
 constexpr size_t kSplitScratchFloats = (size_t)16 << 20;  // 64 MiB of split-K partial tiles
 
+bool aligned16p(const void* q) { return (((uintptr_t)q) & 15) == 0; }
+
 // XCDs of the device (MI355X: 8 of 32 CUs, each with its own L2).
 static int ft_gemm_xcds(ft_context* ctx) { return ctx->num_cus % 8 == 0 && ctx->num_cus >= 64 ? 8 : 1; }
 
@@ -1412,6 +1546,10 @@ int launch_async(ft_context* ctx, AsyncBatch g, int layout, int epi = kEpiPlain)
     bool pairs = false;
     if (epi == kEpiPlain && mn4 && !any_rope && tiles > 0 && (few_tiles || long_k)) {
         int want = (int)((2 * (size_t)ctx->num_cus + tiles - 1) / tiles);
+        // A few tiles more than CUs (288 on 256: the 576-column products): with w shares a CU holds
+        // ceil(288 w / 256) of them, 2, 3, 4 for w = 1, 2, 3, i.e. 2, 1.5, 1.33 tiles' worth; measured,
+        // three shares beat two (and four) in the 135M-shaped step.
+        if (BM == 64 && tiles > ctx->num_cus) want = 3;
         // 128x128 tiles hold two workgroups on a CU: the shares must fit one round of them
         if (BM == 128) want = (int)(2 * (size_t)ctx->num_cus / tiles);
         if (want > 8) want = 8;
@@ -1555,8 +1693,6 @@ int launch_async_auto(ft_context* ctx, const AsyncBatch& g, int layout) {
         return launch_async<128, 128, 64, 64>(ctx, g, layout);
     return launch_async<64, 64, 32, 32>(ctx, g, layout);
 }
-
-bool aligned16p(const void* q) { return (((uintptr_t)q) & 15) == 0; }
 
 // Can out[M,N] (+)= a[M,K] @ b (f16, `layout`) + a2[M,K2] @ b2 run on the asynchronous path?
 bool async_eligible(int layout, const float* a, const void* b, const float* out, const float* add, size_t M, size_t K,

@@ -32,18 +32,50 @@ struct ThinBatch {
 // so MFMA e of an iteration contracts k = 16*it + 4*q + e.
 typedef float thin_f4 __attribute__((ext_vector_type(4)));
 
+// 16 bytes from device memory (16-byte aligned).
+__device__ __forceinline__ float4 load_f4(const ft_global_f* q) {
+    const thin_f4 v = *reinterpret_cast<const __attribute__((address_space(1))) thin_f4*>(q);
+    return make_float4(v.x, v.y, v.z, v.w);
+}
+
 constexpr int kRowWaves = 8;
 
 template <int C, bool YT>
 __global__ __launch_bounds__(kRowWaves * 64) void thin_rowwise_kernel(ThinBatch b) {
-    const ft_thin_problem& p = b.p[blockIdx.y];
+    // The problem's entry of the argument block, read once (all reads, then all pins: one round trip).
+    const ft_thin_problem& pk = b.p[blockIdx.y];
+    struct {
+        const ft_global_f* x;
+        const ft_global_f* y;
+        ft_global_f* out;
+        int M, K;
+        long ldx, ldy, ldo;
+        float scale;
+    } p;
+    {
+        const float* rx = pk.x;
+        const float* ry = pk.y;
+        float* ro = pk.out;
+        const int rM = pk.M, rK = pk.K;
+        const long rldx = pk.ldx, rldy = pk.ldy, rldo = pk.ldo;
+        const float rs = pk.scale;
+        p.x = (const ft_global_f*)ft_pinned(rx);
+        p.y = (const ft_global_f*)ft_pinned(ry);
+        p.out = (ft_global_f*)ft_pinned(ro);
+        p.M = ft_pinned(rM);
+        p.K = ft_pinned(rK);
+        p.ldx = ft_pinned(rldx);
+        p.ldy = ft_pinned(rldy);
+        p.ldo = ft_pinned(rldo);
+        p.scale = ft_pinned(rs);
+    }
     const int row0 = blockIdx.x * 16;
     if (row0 >= p.M) return;
     __shared__ float red[kRowWaves][16][17];
     const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
     const int li = lane % 16, q = lane / 16;
     const int row = row0 + li < p.M ? row0 + li : p.M - 1;  // clamped rows are computed and dropped
-    const float* xr = p.x + (long)row * p.ldx + 4 * q;
+    const ft_global_f* xr = p.x + (long)row * p.ldx + 4 * q;
     const bool col_live = li < C;
     // K is a multiple of 4; the parts are multiples of 16, so a 4-run of k is all in or all out.
     const int part = ((p.K + 16 * kRowWaves - 1) / (16 * kRowWaves)) * 16;
@@ -58,10 +90,9 @@ __global__ __launch_bounds__(kRowWaves * 64) void thin_rowwise_kernel(ThinBatch 
         for (int u = 0; u < U; u++) {
             const int k = k0 + 16 * u + 4 * q;
             const bool in = k < k_end;
-            xa[u] = in ? *reinterpret_cast<const float4*>(xr + k0 + 16 * u) : make_float4(0.f, 0.f, 0.f, 0.f);
+            xa[u] = in ? load_f4(xr + k0 + 16 * u) : make_float4(0.f, 0.f, 0.f, 0.f);
             if constexpr (YT) {
-                const float4 t = (in && col_live) ? *reinterpret_cast<const float4*>(p.y + (long)li * p.ldy + k)
-                                                  : make_float4(0.f, 0.f, 0.f, 0.f);
+                const float4 t = (in && col_live) ? load_f4(p.y + (long)li * p.ldy + k) : make_float4(0.f, 0.f, 0.f, 0.f);
                 yb[u][0] = t.x, yb[u][1] = t.y, yb[u][2] = t.z, yb[u][3] = t.w;
             } else {
 #pragma unroll
