@@ -16,6 +16,16 @@
 // The device-buffer pool: exact-size free lists, like the reference's
 // BufferPool (ferrotensor-backend/src/pool.rs), without its 512 MiB cap:
 // 288 GB of HBM leaves room to keep every step buffer resident.
+// The K shares of a split GEMM left unadded for the kernel that consumes the product (a norm kernel
+// that reads the row anyway): out = (add +) partial[0] + partial[1] + ... in that order, share s of
+// element i at partial[s * stride + i]. splits == 1: nothing was deferred, `out` is complete.
+struct ft_deferred_sum {
+    const float* partial = nullptr;
+    const float* add = nullptr;
+    long stride = 0;
+    int splits = 1;
+};
+
 struct ft_context {
     int device = 0;
     hipStream_t stream = nullptr;
@@ -29,6 +39,10 @@ struct ft_context {
     float* thin_scratch = nullptr;
     // Partial tiles of split-K GEMMs (few output tiles, long K); allocated on first use.
     float* gemm_scratch = nullptr;
+    // Set by the step driver right before one GEMM call whose output's only reader can add the K
+    // shares itself; the launch fills it in (and leaves out splitk_reduce_kernel) when it splits K,
+    // and clears the pointer either way.
+    ft_deferred_sum* defer = nullptr;
     // Per-query-head partial dK/dV of the attention backward at small batch; allocated on first use.
     float* attn_scratch = nullptr;
 

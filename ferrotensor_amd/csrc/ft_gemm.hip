@@ -1575,8 +1575,19 @@ int launch_async(ft_context* ctx, AsyncBatch g, int layout, int epi = kEpiPlain)
         }
     }
     const dim3 grid((unsigned)tiles, (unsigned)g.splits);
+    // A deferred sum is honoured for one plain product whose shares are the plain [splits][M][N] arrays.
+    ft_deferred_sum* const defer = ctx->defer;
+    ctx->defer = nullptr;
+    if (defer) *defer = ft_deferred_sum{};
     auto reduce_shares = [&]() -> int {
         if (g.splits == 1) return FT_OK;
+        if (defer && g.count == 1 && epi == kEpiPlain && g.p[0].ldc == g.p[0].N) {
+            defer->partial = g.partial + g.p[0].partial_off;
+            defer->add = g.p[0].add;
+            defer->stride = (long)g.M * g.p[0].N;
+            defer->splits = g.splits;
+            return FT_OK;
+        }
         SplitReduceArgs ra{};
         long n4max = 0;
         for (int i = 0; i < g.count; i++) {

@@ -316,9 +316,49 @@ __global__ __launch_bounds__(256) void column_sum_kernel(const float* __restrict
 // between the reduction and the output, so every array is touched once and no
 // workgroup barrier is needed. 4 rows per 256-thread workgroup.
 // ---------------------------------------------------------------------------
+// A lane's NV float4 of one row of a deferred split-K sum: (add +) share 0 + share 1 + ... in that
+// order (the order of splitk_reduce_kernel). The loads of up to U shares are issued together, so a row
+// costs splits / U memory round trips instead of one per share.
 template <int NV>
+__device__ __forceinline__ void sum_shares_row(const ft_deferred_sum& d, size_t row_off, int lane, int n4,
+                                               float4 (&v)[NV]) {
+    constexpr int U = NV <= 4 ? 4 : 2;
+#pragma unroll
+    for (int j = 0; j < NV; j++) {
+        const int i = lane + j * kWave;
+        v[j] = (d.add && i < n4) ? reinterpret_cast<const float4*>(d.add + row_off)[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+    for (int s0 = 0; s0 < d.splits; s0 += U) {
+        float4 t[U][NV];
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const int sc = s0 + u < d.splits ? s0 + u : d.splits - 1;  // a share past the end re-reads the last one
+            const float4* src = reinterpret_cast<const float4*>(d.partial + (size_t)sc * d.stride + row_off);
+#pragma unroll
+            for (int j = 0; j < NV; j++) {
+                const int i = lane + j * kWave;
+                t[u][j] = src[i < n4 ? i : 0];
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            if (s0 + u < d.splits) {  // uniform
+#pragma unroll
+                for (int j = 0; j < NV; j++) {
+                    v[j].x += t[u][j].x;
+                    v[j].y += t[u][j].y;
+                    v[j].z += t[u][j].z;
+                    v[j].w += t[u][j].w;
+                }
+            }
+        }
+    }
+}
+
+template <int NV, bool SUM = false>
 __global__ __launch_bounds__(256) void rms_norm_wave_kernel(const float* __restrict__ x, const float* __restrict__ w,
-                                                            float* __restrict__ out, int rows, int size, float eps) {
+                                                            float* __restrict__ out, int rows, int size, float eps,
+                                                            ft_deferred_sum sum, float* __restrict__ x_out) {
     const int row = blockIdx.x * 4 + threadIdx.x / kWave;
     if (row >= rows) return;
     const int lane = threadIdx.x % kWave;
@@ -326,10 +366,20 @@ __global__ __launch_bounds__(256) void rms_norm_wave_kernel(const float* __restr
     const float4* x4 = reinterpret_cast<const float4*>(x + (size_t)row * size);
     float4 v[NV];
     float ss = 0.0f;
+    if constexpr (SUM) {
+        // x is still the K shares of the GEMM that produced it: added here (residual first, then share
+        // after share) and written out once.
+        sum_shares_row<NV>(sum, (size_t)row * size, lane, n4, v);
+    }
 #pragma unroll
     for (int j = 0; j < NV; j++) {
         const int i = lane + j * kWave;
-        v[j] = i < n4 ? x4[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+        if constexpr (SUM) {
+            if (i < n4) reinterpret_cast<float4*>(x_out + (size_t)row * size)[i] = v[j];
+            else v[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+        } else {
+            v[j] = i < n4 ? x4[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
         ss += v[j].x * v[j].x + v[j].y * v[j].y + v[j].z * v[j].z + v[j].w * v[j].w;
     }
     ss = wave_sum(ss);
@@ -348,10 +398,10 @@ __global__ __launch_bounds__(256) void rms_norm_wave_kernel(const float* __restr
 
 // gx = g*w*inv - x*coef (+ add): the input gradient of RMSNorm, optionally
 // summed with the gradient arriving over the residual connection.
-template <int NV>
+template <int NV, bool SUM = false>
 __global__ __launch_bounds__(256) void rms_norm_backward_wave_kernel(
     const float* __restrict__ x, const float* __restrict__ w, const float* __restrict__ g, const float* add,
-    float* gx, int rows, int size, float eps) {
+    float* gx, int rows, int size, float eps, ft_deferred_sum sum) {
     const int row = blockIdx.x * 4 + threadIdx.x / kWave;
     if (row >= rows) return;
     const int lane = threadIdx.x % kWave;
@@ -361,12 +411,16 @@ __global__ __launch_bounds__(256) void rms_norm_backward_wave_kernel(
     const float4* w4 = reinterpret_cast<const float4*>(w);
     float4 xv[NV], gv[NV];
     float ss = 0.0f, gwx = 0.0f;
+    if constexpr (SUM) sum_shares_row<NV>(sum, (size_t)row * size, lane, n4, gv);  // g arrives as K shares
 #pragma unroll
     for (int j = 0; j < NV; j++) {
         const int i = lane + j * kWave;
         if (i < n4) {
             xv[j] = x4[i];
-            const float4 gg = g4[i], ww = w4[i];
+            float4 gg;
+            if constexpr (SUM) gg = gv[j];
+            else gg = g4[i];
+            const float4 ww = w4[i];
             gv[j] = make_float4(gg.x * ww.x, gg.y * ww.y, gg.z * ww.z, gg.w * ww.w);  // g*w
         } else {
             xv[j] = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -888,10 +942,55 @@ int ft_internal_rms_norm_backward_add(ft_context* ctx, const float* x, const flo
     const dim3 grid(ft_div_up(rows, 4));
     if (size <= 1024)
         hipLaunchKernelGGL((rms_norm_backward_wave_kernel<4>), grid, dim3(256), 0, ctx->stream, x, w, g, add, gx,
-                           (int)rows, (int)size, eps);
+                           (int)rows, (int)size, eps, ft_deferred_sum{});
     else
         hipLaunchKernelGGL((rms_norm_backward_wave_kernel<8>), grid, dim3(256), 0, ctx->stream, x, w, g, add, gx,
-                           (int)rows, (int)size, eps);
+                           (int)rows, (int)size, eps, ft_deferred_sum{});
+    FT_LAUNCH_CHECK();
+    return FT_OK;
+}
+
+// Can a norm kernel add the K shares of a [rows, size] product itself?
+bool ft_internal_norm_can_sum(size_t rows, size_t size) { return size % 4 == 0 && size <= 2048 && rows < (1u << 30); }
+
+// x_out = the deferred sum `d` ([rows, size]); out = rms_norm(x_out) * w. One pass: the shares are read
+// where the plain kernel reads x.
+int ft_internal_rms_norm_sum(ft_context* ctx, const ft_deferred_sum* d, float* x_out, const float* w, float* out,
+                             size_t rows, size_t size, float eps) {
+    FT_CHECK_ARG(ctx && d && d->partial && d->splits > 1 && x_out && w && out, "rms_norm_sum: bad argument");
+    FT_CHECK_ARG(ft_internal_norm_can_sum(rows, size) && aligned16(d->partial) && aligned16(d->add) && d->stride % 4 == 0 &&
+                     aligned16(x_out) && aligned16(w) && aligned16(out),
+                 "rms_norm_sum: shape or alignment outside the fused kernel's");
+    if (rows == 0) return FT_OK;
+    ft_prof_scope prof(ctx, "rms_norm_kernel", 0.0, (12.0 + 4.0 * d->splits + (d->add ? 4.0 : 0.0)) * (double)rows * size);
+    const dim3 grid(ft_div_up(rows, 4));
+    if (size <= 1024)
+        hipLaunchKernelGGL((rms_norm_wave_kernel<4, true>), grid, dim3(256), 0, ctx->stream, x_out, w, out, (int)rows,
+                           (int)size, eps, *d, x_out);
+    else
+        hipLaunchKernelGGL((rms_norm_wave_kernel<8, true>), grid, dim3(256), 0, ctx->stream, x_out, w, out, (int)rows,
+                           (int)size, eps, *d, x_out);
+    FT_LAUNCH_CHECK();
+    return FT_OK;
+}
+
+// gx = rms_norm_backward(x, w, g) (+ add) with g = the deferred sum `d`. No weight gradient.
+int ft_internal_rms_norm_backward_sum(ft_context* ctx, const float* x, const float* w, const ft_deferred_sum* d,
+                                      const float* add, float* gx, size_t rows, size_t size, float eps) {
+    FT_CHECK_ARG(ctx && x && w && d && d->partial && d->splits > 1 && gx, "rms_norm_backward_sum: bad argument");
+    FT_CHECK_ARG(ft_internal_norm_can_sum(rows, size) && aligned16(d->partial) && aligned16(d->add) && d->stride % 4 == 0 &&
+                     aligned16(x) && aligned16(w) && aligned16(gx) && aligned16(add),
+                 "rms_norm_backward_sum: shape or alignment outside the fused kernel's");
+    if (rows == 0) return FT_OK;
+    ft_prof_scope prof(ctx, "rms_norm_backward_kernel", 0.0,
+                       (8.0 + 4.0 * d->splits + (d->add ? 4.0 : 0.0) + (add ? 4.0 : 0.0)) * (double)rows * size);
+    const dim3 grid(ft_div_up(rows, 4));
+    if (size <= 1024)
+        hipLaunchKernelGGL((rms_norm_backward_wave_kernel<4, true>), grid, dim3(256), 0, ctx->stream, x, w,
+                           (const float*)nullptr, add, gx, (int)rows, (int)size, eps, *d);
+    else
+        hipLaunchKernelGGL((rms_norm_backward_wave_kernel<8, true>), grid, dim3(256), 0, ctx->stream, x, w,
+                           (const float*)nullptr, add, gx, (int)rows, (int)size, eps, *d);
     FT_LAUNCH_CHECK();
     return FT_OK;
 }
@@ -1091,10 +1190,10 @@ int ft_rms_norm_eps(ft_context* ctx, const float* x, const float* w, float* out,
         const dim3 grid(ft_div_up(rows, 4));
         if (size <= 1024)
             hipLaunchKernelGGL((rms_norm_wave_kernel<4>), grid, dim3(256), 0, ctx->stream, x, w, out, (int)rows,
-                               (int)size, eps);
+                               (int)size, eps, ft_deferred_sum{}, (float*)nullptr);
         else
             hipLaunchKernelGGL((rms_norm_wave_kernel<8>), grid, dim3(256), 0, ctx->stream, x, w, out, (int)rows,
-                               (int)size, eps);
+                               (int)size, eps, ft_deferred_sum{}, (float*)nullptr);
         FT_LAUNCH_CHECK();
         return FT_OK;
     }

@@ -43,6 +43,11 @@ int ft_internal_rope_table(ft_context* ctx, float* table, size_t seq, size_t hea
 int ft_internal_rope_pair(ft_context* ctx, const float* a_src, float* a_dst, size_t heads_a, const float* b_src,
                           float* b_dst, size_t heads_b, const float* table, size_t batch, size_t seq,
                           size_t head_dim, int inverse);
+bool ft_internal_norm_can_sum(size_t rows, size_t size);
+int ft_internal_rms_norm_sum(ft_context* ctx, const ft_deferred_sum* d, float* x_out, const float* w, float* out,
+                             size_t rows, size_t size, float eps);
+int ft_internal_rms_norm_backward_sum(ft_context* ctx, const float* x, const float* w, const ft_deferred_sum* d,
+                                      const float* add, float* gx, size_t rows, size_t size, float eps);
 int ft_internal_row_bias_add(ft_context* ctx, float* y, const float* bias, size_t rows, size_t cols);
 int ft_internal_col_sum(ft_context* ctx, const float* g, float* out, size_t rows, size_t cols, int accumulate);
 bool ft_internal_attention_rope_fusable(const float* q, const float* k, const float* v, const float* out,
@@ -148,6 +153,8 @@ struct ft_model {
     float* dt_pool[kDtPool] = {};
     int dt_used = 0;
     std::vector<ft_thin_problem> pending_cols;
+    // The down projection of the block before, when its K shares were left for this block's first norm to add.
+    ft_deferred_sum pending_x;
 
     size_t head_dim() const { return cfg.hidden_size / cfg.num_attention_heads; }
 };
@@ -382,13 +389,30 @@ int linear_bias(ft_context* ctx, const LinearW& l, float* y, size_t T) {
     return ft_internal_row_bias_add(ctx, y, l.bias, T, l.out);
 }
 
+// Offers the next GEMM launch on `ctx` the chance to leave its K shares unadded (the caller's next
+// kernel is a norm that adds them while it reads the row). `d->splits > 1` afterwards: it did.
+struct DeferScope {
+    ft_context* ctx;
+    DeferScope(ft_context* c, ft_deferred_sum* d, bool enable) : ctx(c) {
+        *d = ft_deferred_sum{};
+        c->defer = enable ? d : nullptr;
+    }
+    ~DeferScope() { ctx->defer = nullptr; }
+};
+
 // y = x @ W (+ (scale * x @ A) @ B) (+ bias) (+ residual), keeping t = scale * x @ A for backward.
+// `defer` (optional): the product may leave its K shares unadded for the caller's next kernel.
 int linear_forward(ft_context* ctx, LinearW& l, const float* x, float* t, float* y, size_t T,
-                   const float* residual = nullptr) {
+                   const float* residual = nullptr, ft_deferred_sum* defer = nullptr) {
     LinearW* ls[1] = {&l};
     float* ts[1] = {t};
     FT_TRY(lora_down_group(ctx, ls, ts, 1, x, T));
-    if (!l.bias) return linear_gemm(ctx, l, x, t, y, T, residual);
+    ft_deferred_sum unused;
+    if (!l.bias) {
+        DeferScope scope(ctx, defer ? defer : &unused, defer != nullptr);
+        return linear_gemm(ctx, l, x, t, y, T, residual);
+    }
+    if (defer) *defer = ft_deferred_sum{};
     // the bias belongs to the linear's output, the residual is added to that sum afterwards
     FT_TRY(linear_gemm(ctx, l, x, t, y, T));
     FT_TRY(linear_bias(ctx, l, y, T));
@@ -474,9 +498,13 @@ int linear_backward(ft_model* m, LinearW& l, const float* x, const float* t, con
 // gradients are summed into dx (NULL: not wanted) by one GEMM whose K loop runs
 // over all the output gradients. Falls back to one linear at a time when the
 // adapters cannot be batched.
+// `defer` (optional): the summed input gradient may be left as K shares for the norm backward that reads it next.
 int linear_backward_group(ft_model* m, LinearW* const* ls, const float* const* ts, const float* const* dys,
-                          float* dx, int n, const float* x, size_t T, bool accumulate, bool flush) {
+                          float* dx, int n, const float* x, size_t T, bool accumulate, bool flush,
+                          ft_deferred_sum* defer = nullptr) {
     ft_context* ctx = m->ctx;
+    ft_deferred_sum unused;
+    if (defer) *defer = ft_deferred_sum{};
     bool batch = n <= 3;
     bool any_gw = false;
     for (int i = 0; i < n; i++) {
@@ -516,6 +544,7 @@ int linear_backward_group(ft_model* m, LinearW* const* ls, const float* const* t
         if (!dx) return FT_OK;
         ft_lora_dx_desc d[3];
         for (int i = 0; i < n; i++) d[i] = ft_lora_dx_desc{dys[i], ls[i]->w, ls[i]->dtype, nullptr, nullptr, ls[i]->out, 0};
+        DeferScope scope(ctx, defer ? defer : &unused, defer != nullptr);
         return ft_lora_linear_dx_group(ctx, d, (size_t)n, nullptr, dx, T, ls[0]->in);
     }
     FT_TRY(ft_thin_rowwise(ctx, rows, n));
@@ -525,13 +554,16 @@ int linear_backward_group(ft_model* m, LinearW* const* ls, const float* const* t
         ft_lora_dx_desc d[3];
         for (int i = 0; i < n; i++)
             d[i] = ft_lora_dx_desc{dys[i], ls[i]->w, ls[i]->dtype, dts[i], ls[i]->a, ls[i]->out, ls[i]->r};
+        DeferScope scope(ctx, defer ? defer : &unused, defer != nullptr);
         FT_TRY(ft_lora_linear_dx_group(ctx, d, (size_t)n, nullptr, dx, T, ls[0]->in));
     }
     return FT_OK;
 }
 
 // One transformer block: acts[l].x -> acts[l + 1].x (or x_final), filling acts[l].
-int layer_forward(ft_model* m, size_t l, size_t B, size_t S) {
+// `defer_tail`: the next kernel after this block is the next block's first norm (the plain forward pass, not a
+// recomputation), so the down projection may leave its K shares to it (m->pending_x).
+int layer_forward(ft_model* m, size_t l, size_t B, size_t S, bool defer_tail = false) {
     ft_context* ctx = m->ctx;
     const ft_model_config& c = m->cfg;
     const size_t T = B * S, H = c.hidden_size, F = c.intermediate_size;
@@ -542,7 +574,12 @@ int layer_forward(ft_model* m, size_t l, size_t B, size_t S) {
         Layer& L = m->layers[l];
         LayerActs& a = m->acts[l];
         float* x_next = l + 1 < m->layers.size() ? m->acts[l + 1].x : m->x_final;
-        FT_TRY(ft_rms_norm_eps(ctx, a.x, L.norm1, a.h1, T, H, c.rms_norm_eps));
+        if (m->pending_x.splits > 1) {
+            FT_TRY(ft_internal_rms_norm_sum(ctx, &m->pending_x, a.x, L.norm1, a.h1, T, H, c.rms_norm_eps));
+            m->pending_x = ft_deferred_sum{};
+        } else {
+            FT_TRY(ft_rms_norm_eps(ctx, a.x, L.norm1, a.h1, T, H, c.rms_norm_eps));
+        }
         {
             LinearW* ls[3] = {&L.q, &L.k, &L.v};
             float* ts[3] = {a.tq, a.tk, a.tv};
@@ -568,9 +605,17 @@ int layer_forward(ft_model* m, size_t l, size_t B, size_t S) {
             FT_TRY(ft_rope_theta(ctx, a.k, B, S, nkv * D, D, 0, c.rope_theta));
         }
         FT_TRY(ft_flash_attention_v2_with_stats(ctx, a.q, a.k, a.v, a.attn, a.stats, B, S, S, nh, nkv, D, &opts));
-        // h = x + o_proj(attn): the residual is added in the GEMM epilogue
-        FT_TRY(linear_forward(ctx, L.o, a.attn, a.to, a.h, T, a.x));
-        FT_TRY(ft_rms_norm_eps(ctx, a.h, L.norm2, a.h2, T, H, c.rms_norm_eps));
+        // h = x + o_proj(attn): the residual is added in the GEMM epilogue, or, when the product's K is shared
+        // out over workgroups, by the norm kernel that reads h next
+        const bool can_sum = ft_internal_norm_can_sum(T, H);
+        {
+            ft_deferred_sum d;
+            FT_TRY(linear_forward(ctx, L.o, a.attn, a.to, a.h, T, a.x, can_sum ? &d : nullptr));
+            if (d.splits > 1)
+                FT_TRY(ft_internal_rms_norm_sum(ctx, &d, a.h, L.norm2, a.h2, T, H, c.rms_norm_eps));
+            else
+                FT_TRY(ft_rms_norm_eps(ctx, a.h, L.norm2, a.h2, T, H, c.rms_norm_eps));
+        }
         {
             LinearW* ls[2] = {&L.up, &L.gate};
             float* ts[2] = {a.tup, a.tgate};
@@ -586,7 +631,9 @@ int layer_forward(ft_model* m, size_t l, size_t B, size_t S) {
             for (int i = 0; i < 2; i++) FT_TRY(linear_bias(ctx, *ls[i], ys[i], T));
             FT_TRY(ft_silu_gate_fused(ctx, a.gate, a.up, a.act, T * F));
         }
-        FT_TRY(linear_forward(ctx, L.down, a.act, a.tdown, x_next, T, a.h));
+        m->pending_x = ft_deferred_sum{};
+        FT_TRY(linear_forward(ctx, L.down, a.act, a.tdown, x_next, T, a.h,
+                              defer_tail && can_sum && l + 1 < m->layers.size() ? &m->pending_x : nullptr));
     }
     return FT_OK;
 }
@@ -653,7 +700,8 @@ int model_forward(ft_model* m, size_t B, size_t S) {
     const ft_model_config& c = m->cfg;
     const size_t T = B * S, H = c.hidden_size;
     FT_TRY(ft_embedding(ctx, m->embed, c.vocab_size, H, m->ids_dev, T, m->acts.empty() ? m->x_final : m->acts[0].x));
-    for (size_t l = 0; l < m->layers.size(); l++) FT_TRY(layer_forward(m, l, B, S));
+    m->pending_x = ft_deferred_sum{};
+    for (size_t l = 0; l < m->layers.size(); l++) FT_TRY(layer_forward(m, l, B, S, true));
     const float* xf = m->x_final;
     if (m->head_compact) {
         // gather: row k of xc = row head[k] of x_final
@@ -678,11 +726,16 @@ int fetch_step_out(ft_model* m) {
 // computed too (RMSNormNode::backward, autograd/src/lib.rs:575-595), added to the earlier
 // micro-batches' when `accumulate`; `tmp` [rows, H] is scratch for that unfused form and must not
 // alias x, g or add.
+// `g_sum` (optional, only without `gw`): g arrives as the K shares of the GEMM that produced it.
 int norm_backward(ft_model* m, const float* x, const float* w, float* gw, const float* g, const float* add,
-                  float* gx, float* tmp, size_t rows, bool accumulate) {
+                  float* gx, float* tmp, size_t rows, bool accumulate, const ft_deferred_sum* g_sum = nullptr) {
     ft_context* ctx = m->ctx;
     const size_t H = m->cfg.hidden_size;
     const float eps = m->cfg.rms_norm_eps;
+    if (g_sum && g_sum->splits > 1) {
+        FT_CHECK_ARG(!gw, "norm_backward: a deferred gradient with a trainable norm scale");
+        return ft_internal_rms_norm_backward_sum(ctx, x, w, g_sum, add, gx, rows, H, eps);
+    }
     if (!gw) {
         if (add) return ft_internal_rms_norm_backward_add(ctx, x, w, g, add, gx, rows, H, eps);
         return ft_rms_norm_backward(ctx, x, w, g, gx, nullptr, rows, H, eps);
@@ -714,9 +767,11 @@ int model_backward(ft_model* m, size_t B, size_t S, bool accumulate) {
     } else {
         FT_TRY(norm_backward(m, m->x_final, m->norm_f, m->gnorm_f, m->d_h2, nullptr, g, nullptr, T, accumulate));
     }
+    const bool can_sum = ft_internal_norm_can_sum(T, H);
     for (size_t li = m->layers.size(); li-- > 0;) {
         Layer& L = m->layers[li];
         LayerActs& a = m->acts[li];
+        ft_deferred_sum dsum;  // an input gradient left as K shares for the norm backward that follows it
         // The factor gradients of a block read its activations, output gradients and dT buffers; they
         // are launched (flush_cols) at the block's end, before g, the buffers of the next block's
         // gradients and, with checkpointing, the shared block buffers are rewritten.
@@ -737,10 +792,12 @@ int model_backward(ft_model* m, size_t B, size_t S, bool accumulate) {
             LinearW* ls[2] = {&L.up, &L.gate};
             const float* ts[2] = {a.tup, a.tgate};
             const float* dys[2] = {m->d_up, m->d_gate};
-            FT_TRY(linear_backward_group(m, ls, ts, dys, m->d_h2, 2, a.h2, T, accumulate, false));
+            dsum = ft_deferred_sum{};
+            FT_TRY(linear_backward_group(m, ls, ts, dys, m->d_h2, 2, a.h2, T, accumulate, false,
+                                         can_sum && !L.gnorm2 ? &dsum : nullptr));
         }
         // g_h = g + norm2_backward(d_h2) (into g_other)
-        FT_TRY(norm_backward(m, a.h, L.norm2, L.gnorm2, m->d_h2, g, g_other, m->d_h1, T, accumulate));
+        FT_TRY(norm_backward(m, a.h, L.norm2, L.gnorm2, m->d_h2, g, g_other, m->d_h1, T, accumulate, &dsum));
         // h = x + o_proj(attn)
         FT_TRY(linear_backward(m, L.o, a.attn, a.to, g_other, m->d_attn, T, accumulate));
         if (m->rope_table &&
@@ -769,11 +826,13 @@ int model_backward(ft_model* m, size_t B, size_t S, bool accumulate) {
             const float* dys[3] = {m->dq, m->dk, m->dv};
             // d_h1 = dx_q + dx_k + dx_v
             // the block's last adapters: everything that waited is launched now
-            FT_TRY(linear_backward_group(m, ls, ts, dys, need_dx ? m->d_h1 : nullptr, 3, a.h1, T, accumulate, true));
+            dsum = ft_deferred_sum{};
+            FT_TRY(linear_backward_group(m, ls, ts, dys, need_dx ? m->d_h1 : nullptr, 3, a.h1, T, accumulate, true,
+                                         can_sum && !L.gnorm1 ? &dsum : nullptr));
         }
         if (!need_dx) break;
         // g = g_h + norm1_backward(d_h1)
-        FT_TRY(norm_backward(m, a.x, L.norm1, L.gnorm1, m->d_h1, g_other, g, m->d_h2, T, accumulate));
+        FT_TRY(norm_backward(m, a.x, L.norm1, L.gnorm1, m->d_h1, g_other, g, m->d_h2, T, accumulate, &dsum));
     }
     return flush_cols(m);
 }
