@@ -528,8 +528,9 @@ def main():
         "step_mfma_frac": step_flops(w, int(st.tokens)) / (elapsed / args.steps) / 1e12 / FP32_MFMA_PEAK_TFLOPS,
         "roofline": {"bound": "mfma", "kernel": dom["name"], "achieved": achieved, "peak": FP32_MFMA_PEAK_TFLOPS,
                      "unit": "TFLOP/s", "frac": achieved / FP32_MFMA_PEAK_TFLOPS,
-                     "traffic": measured_traffic(dom["name"], args.workload),
-                     "traffic_source": traffic_source() if args.workload == "360m" else None,
+                     # the record is of the default batch: other micro-batch sizes have other launches
+                     "traffic": measured_traffic(dom["name"], args.workload) if not args.micro_batch else None,
+                     "traffic_source": traffic_source() if args.workload == "360m" and not args.micro_batch else None,
                      "launches_per_step": dom["launches"] // args.steps,
                      "avg_launch_us": dom["ms"] * 1e3 / dom["launches"],
                      "all_gemm_kernels_tflops": all_gemm_tf,
