@@ -602,7 +602,26 @@ struct AsyncBatch {
     int tiles_m, tiles_n;  // row blocks; n tiles of all products together
     int xcds;              // chunks of the tile order (one per XCD), 1 = workgroup id order
     int panel;             // n tiles per panel of the tile order
+    // Tail split: a tile count a little above a multiple of the CU count (800 on 256) leaves 32 CUs with a
+    // fourth workgroup, and the launch lasts as long as they do (56 us for 768 tiles, 71 us for 800). The last
+    // tiles of the tile order (positions >= tail_first) are instead each shared out along K over
+    // 1 << tail_shift workgroups, whose partial tiles ([tile][share][BM x BN] in `partial`)
+    // splitk_tail_reduce_kernel adds. tail_first == tiles_m * tiles_n: none. Never with splits > 1.
+    int tail_first, tail_shift;
 };
+
+// Position in the tile order -> (row block, n tile over all products): panels of `panel` n tiles,
+// inside a panel row block after row block.
+__host__ __device__ __forceinline__ void tile_in_order(const AsyncBatch& g, int idx, int* tm, int* tn) {
+    const int per_panel = g.tiles_m * g.panel;
+    const int last = (g.tiles_n - 1) / g.panel;
+    int pnl = idx / per_panel;
+    pnl = pnl < last ? pnl : last;
+    const int rem = idx - pnl * per_panel;
+    const int width = pnl == last ? g.tiles_n - last * g.panel : g.panel;
+    *tm = rem / width;
+    *tn = pnl * g.panel + rem % width;
+}
 
 template <int NSEG, typename T>
 __device__ __forceinline__ T seg_pick(const T (&v)[NSEG], int s) {
@@ -635,6 +654,37 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(SplitReduceArgs a) {
         v.w += t.w;
     }
     reinterpret_cast<float4*>(a.out[pi])[i] = v;
+}
+
+// The shares of one tail tile (64 x 64), added in share order (after the residual): one workgroup of 1024
+// threads per tile, a thread per four consecutive columns with the loads of all shares in flight at once.
+__global__ __launch_bounds__(1024) void splitk_tail_reduce_kernel(AsyncBatch g) {
+    int tm, tn;
+    tile_in_order(g, g.tail_first + (int)blockIdx.x, &tm, &tn);
+    int pi = 0;
+    if (g.count > 1 && tn >= g.p[1].tile_begin) pi = 1;
+    if (g.count > 2 && tn >= g.p[2].tile_begin) pi = 2;
+    const AsyncProb& p = g.p[pi];
+    const int m0 = tm * 64, n0 = (tn - p.tile_begin) * 64;
+    const int shares = 1 << g.tail_shift;
+    const int row = threadIdx.x / 16, col = (threadIdx.x % 16) * 4;
+    if (m0 + row >= g.M || n0 + col >= p.N) return;  // N is a multiple of 4 on this path
+    const float* src = g.partial + ((long)blockIdx.x << g.tail_shift) * 4096 + row * 64 + col;
+    float4 t[8];
+#pragma unroll
+    for (int sh = 0; sh < 8; sh++) t[sh] = *reinterpret_cast<const float4*>(src + (sh < shares ? sh : shares - 1) * 4096);
+    const long o = (long)(m0 + row) * p.ldc + n0 + col;
+    float4 v = p.add ? *reinterpret_cast<const float4*>(p.add + o) : make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+    for (int sh = 0; sh < 8; sh++) {
+        if (sh < shares) {
+            v.x += t[sh].x;
+            v.y += t[sh].y;
+            v.z += t[sh].z;
+            v.w += t[sh].w;
+        }
+    }
+    *reinterpret_cast<float4*>(p.out + o) = v;
 }
 
 // Output elements leave with the non-temporal hint: nobody in this launch reads them again, and
@@ -696,7 +746,7 @@ __global__ __launch_bounds__(256 * KW) void gemm_async_kernel(AsyncBatch g) {
     // which held every workgroup of a launch for microseconds before its first tile request.
     // (All the reads first, then all the pins: a pin waits for its value, and a wait in front of a
     // later read would make two round trips of one.)
-    const int r_xcds = g.xcds, r_tiles_m = g.tiles_m,
+    const int r_xcds = g.xcds, r_tail_first = g.tail_first, r_tail_shift = g.tail_shift, r_tiles_m = g.tiles_m,
               r_tiles_n = g.tiles_n, r_panel = g.panel, r_count = g.count, r_splits = g.splits,
               r_begin1 = g.p[1].tile_begin, r_begin2 = g.p[2].tile_begin, r_M = g.M;
     float* const r_partial = g.partial;
@@ -781,7 +831,7 @@ __global__ __launch_bounds__(256 * KW) void gemm_async_kernel(AsyncBatch g) {
     // The first product's entry sits at a constant offset: it is fetched with the header, and only a
     // workgroup of a later product of the batch pays a second round trip to the argument block.
     const RawProb raw0 = read_prob(g.p[0]);
-    const int g_xcds = pinned(r_xcds);
+    const int g_xcds = pinned(r_xcds), g_tail_first = pinned(r_tail_first), g_tail_shift = pinned(r_tail_shift);
     const int g_tiles_m = pinned(r_tiles_m), g_tiles_n = pinned(r_tiles_n), g_panel = pinned(r_panel);
     const int g_count = pinned(r_count), g_splits = pinned(r_splits);
     const int begin1 = pinned(r_begin1), begin2 = pinned(r_begin2);
@@ -789,8 +839,15 @@ __global__ __launch_bounds__(256 * KW) void gemm_async_kernel(AsyncBatch g) {
     GlobalF* const g_partial = (GlobalF*)pinned(r_partial);
     ProbRegs p = pin_prob(g.p[0], raw0);
     int bid = (int)blockIdx.x;
-    if (g_xcds == 8) {  // (8 or 1: shifts instead of divisions on the way to the first tile request)
-        const int total = g_tiles_m * g_tiles_n;
+    // A workgroup past the whole tiles takes one K share of a tail tile (uniform per workgroup).
+    const bool tail = bid >= g_tail_first;
+    int tail_share = 0;
+    if (tail) {
+        const int u = bid - g_tail_first;
+        tail_share = u & ((1 << g_tail_shift) - 1);
+        bid = g_tail_first + (u >> g_tail_shift);
+    } else if (g_xcds == 8) {  // (8 or 1: shifts instead of divisions on the way to the first tile request)
+        const int total = g_tail_first;  // the whole tiles: all of them when there is no tail
         const int x = bid & 7, q = total >> 3, r = total & 7;
         bid = x * q + (x < r ? x : r) + (bid >> 3);
     }
@@ -843,8 +900,8 @@ __global__ __launch_bounds__(256 * KW) void gemm_async_kernel(AsyncBatch g) {
     // This workgroup's share of the K tiles: [t0, nt).
     // (KW = 2: counted in pairs of tiles; the host only chooses it when every segment has an even number.)
     const int nt_all = tend[NSEG - 1] / KW;
-    const int split = (int)blockIdx.y;
-    const int nsplit = g_splits;
+    const int split = tail ? tail_share : (int)blockIdx.y;
+    const int nsplit = tail ? 1 << g_tail_shift : g_splits;
     // (32-bit: at most 2^15 K tiles and 8 shares; most launches have one share)
     const int t0 = nsplit == 1 ? 0 : (int)((unsigned)(nt_all * split) / (unsigned)nsplit);
     const int nt = nsplit == 1 ? nt_all : (int)((unsigned)(nt_all * (split + 1)) / (unsigned)nsplit);
@@ -1000,7 +1057,7 @@ __global__ __launch_bounds__(256 * KW) void gemm_async_kernel(AsyncBatch g) {
     bool pre_add = false;
     if constexpr (PRE) {
         const GlobalF* s1 = EPI == kEpiSiluBwd ? p.e1 : p.add;
-        pre_add = grp == 0 && (EPI == kEpiSiluBwd || (p.add != nullptr && g_splits == 1 && p.rope == nullptr));
+        pre_add = grp == 0 && (EPI == kEpiSiluBwd || (p.add != nullptr && g_splits == 1 && !tail && p.rope == nullptr));
         bool rotated = false;
         if constexpr (EPI == kEpiPlain) rotated = p.rope != nullptr;
         if (rotated) {  // the rotation's (cos, sin) of this lane's 16 rows (never together with a residual)
@@ -1158,6 +1215,9 @@ __global__ __launch_bounds__(256 * KW) void gemm_async_kernel(AsyncBatch g) {
             store_streaming(&p.out2[o], d * (x * sg));
             store_streaming(&p.out[o], d * y * (sg * (1.0f + x * (1.0f - sg))));
         });
+    } else if (tail) {
+        GlobalF* dst = g_partial + ((((long)(bid - g_tail_first)) << g_tail_shift) + split) * (BM * BN);
+        emit_all([&](int i, int j, int r, int row, int col) { dst[(row - m0) * BN + (col - n0)] = acc[i][j][r]; });
     } else if (g_splits > 1) {
         GlobalF* dst = g_partial + p.partial_off + (long)split * M * p.N;
         emit_all([&](int i, int j, int r, int row, int col) { dst[(long)row * p.N + col] = acc[i][j][r]; });
@@ -1544,7 +1604,54 @@ int launch_async(ft_context* ctx, AsyncBatch g, int layout, int epi = kEpiPlain)
     for (int i = 0; i < g.count && pairs_ok; i++)
         for (int s = 0; s < g.p[i].nseg; s++) pairs_ok = pairs_ok && g.p[i].seg[s].nt % 2 == 0;
     bool pairs = false;
-    if (epi == kEpiPlain && mn4 && !any_rope && tiles > 0 && (few_tiles || long_k)) {
+    g.tail_first = tiles;
+    g.tail_shift = 0;
+    if (BM == 64 && epi == kEpiPlain && (size_t)tiles * 4 > (size_t)ctx->num_cus * 5 && !long_k) {
+        // More tiles than the few-tile rule below shares out, and a remainder over the CUs of at most a quarter
+        // of them: its tiles (the last of the order) must be plain ones (no RoPE epilogue, whole float4 groups).
+        const int cus = ctx->num_cus, tail = tiles % cus;
+        // at most 8 shares of at least 3 K tiles each (4 and 8 shares measured alike: 66-68 us against 73)
+        int shift = 0;
+        while (shift < 3 && (tail << (shift + 1)) <= cus && (min_kt >> (shift + 1)) >= 3) shift++;
+        bool ok = tail > 0 && shift >= 2 && (size_t)(tail << shift) * BM * BN <= kSplitScratchFloats;
+        ok = ok && !(pairs_ok && (size_t)tiles <= 2 * (size_t)cus && min_kt >= 32);  // not with eight waves per tile
+        auto tail_is_plain = [&]() {
+            bool plain = true;
+            for (int u = 0; u < tail && plain; u++) {
+                int tm, tn;
+                tile_in_order(g, tiles - tail + u, &tm, &tn);
+                int pi = 0;
+                if (g.count > 1 && tn >= g.p[1].tile_begin) pi = 1;
+                if (g.count > 2 && tn >= g.p[2].tile_begin) pi = 2;
+                const AsyncProb& p = g.p[pi];
+                plain = p.rope == nullptr && p.N % 4 == 0 && p.ldc % 4 == 0 && aligned16p(p.out) && aligned16p(p.add);
+            }
+            return plain;
+        };
+        if (ok && !tail_is_plain()) {
+            // q and k are rotated, v is not: with panels as wide as the last product the order ends in its tiles
+            // alone (narrower panels re-read more of a; the launch is matrix-bound).
+            const AsyncProb& last = g.p[g.count - 1];
+            const int lw = (last.N + BN - 1) / BN;
+            const int keep = g.panel;
+            ok = g.count > 1 && last.rope == nullptr && lw > 0 && last.tile_begin % lw == 0 && tail <= tiles_m * lw;
+            if (ok) {
+                g.panel = lw;
+                ok = tail_is_plain();
+                if (!ok) g.panel = keep;
+            }
+        }
+        if (ok) {
+            if (!ctx->gemm_scratch) {
+                FT_HIP(hipSetDevice(ctx->device));
+                FT_HIP(hipMalloc((void**)&ctx->gemm_scratch, kSplitScratchFloats * sizeof(float)));
+            }
+            g.tail_first = tiles - tail;
+            g.tail_shift = shift;
+            g.partial = ctx->gemm_scratch;
+        }
+    }
+    if (g.tail_shift == 0 && epi == kEpiPlain && mn4 && !any_rope && tiles > 0 && (few_tiles || long_k)) {
         int want = (int)((2 * (size_t)ctx->num_cus + tiles - 1) / tiles);
         // A few tiles more than CUs (288 on 256: the 576-column products): with w shares a CU holds
         // ceil(288 w / 256) of them, 2, 3, 4 for w = 1, 2, 3, i.e. 2, 1.5, 1.33 tiles' worth; measured,
@@ -1574,12 +1681,18 @@ int launch_async(ft_context* ctx, AsyncBatch g, int layout, int epi = kEpiPlain)
             }
         }
     }
-    const dim3 grid((unsigned)tiles, (unsigned)g.splits);
+    const dim3 grid((unsigned)(g.tail_first + ((tiles - g.tail_first) << g.tail_shift)), (unsigned)g.splits);
     // A deferred sum is honoured for one plain product whose shares are the plain [splits][M][N] arrays.
     ft_deferred_sum* const defer = ctx->defer;
     ctx->defer = nullptr;
     if (defer) *defer = ft_deferred_sum{};
     auto reduce_shares = [&]() -> int {
+        if (g.tail_shift > 0) {
+            hipLaunchKernelGGL(splitk_tail_reduce_kernel, dim3((unsigned)(tiles - g.tail_first)), dim3(1024), 0,
+                               ctx->stream, g);
+            FT_LAUNCH_CHECK();
+            return FT_OK;
+        }
         if (g.splits == 1) return FT_OK;
         if (defer && g.count == 1 && epi == kEpiPlain && g.p[0].ldc == g.p[0].N) {
             defer->partial = g.partial + g.p[0].partial_off;

@@ -169,6 +169,31 @@ def test_f32_products_with_short_k_and_smallest_split_shares(g, M, N, K):
     assert_close(f"matmul_at {M}x{K}x{N}", out.to_numpy(), want, atol=1e-3, rtol=1e-4)
 
 
+@pytest.mark.parametrize("M,K,N", [(2048, 960, 1600), (2000, 512, 1600), (2048, 960, 1664)])
+def test_tile_counts_just_above_a_multiple_of_the_cu_count(g, M, K, N):
+    """800 (or 832) tiles of 64x64 on 256 CUs: the last 32 (64) tiles of the order are shared out along K over
+    8 or 4 workgroups each and added by a second kernel. Plain product, product with residual and rank-8 term,
+    and the input-gradient layout; 2000 rows: a ragged last row block among the shared tiles."""
+    from ferrotensor_amd import UnifiedTensor
+    ctx, eng = g
+    a, w = rnd(K + N, M, K), rnd(K * 2 + N, K, N, scale=0.05)
+    w16 = UnifiedTensor.from_f32_as_f16(ctx, w, [K, N])
+    wr = cpu.round_f16(w)
+    out = empty(ctx, M, N)
+    eng.matmul_f16b(ctx, up(ctx, a), w16, out)
+    want = f64_mm(a, wr)
+    assert_close("matmul_f16b", out.to_numpy(), want, atol=1e-3, rtol=1e-4)
+    t, b2, res = rnd(3, M, 8), rnd(4, 8, N), rnd(5, M, N)
+    out = empty(ctx, M, N)
+    eng.lora_linear(ctx, up(ctx, a), w16, up(ctx, t), up(ctx, b2), out, up(ctx, res))
+    assert_close("lora_linear + residual", out.to_numpy(), want + f64_mm(t, b2) + res, atol=1e-3, rtol=1e-4)
+    w2 = rnd(K * 3 + N, N, K, scale=0.05)
+    w2_16 = UnifiedTensor.from_f32_as_f16(ctx, w2, [N, K])
+    dx = empty(ctx, M, N)
+    eng.matmul_bt_f16b(ctx, up(ctx, a), w2_16, dx)
+    assert_close("matmul_bt_f16b", dx.to_numpy(), f64_mm(a, cpu.round_f16(w2).T), atol=1e-3, rtol=1e-4)
+
+
 @pytest.mark.parametrize("M,K,N", [(1536, 2560, 960), (2048, 1024, 960), (1472, 2048, 896)])
 def test_long_k_products_on_eight_waves(g, M, K, N):
     """320 to 512 output tiles of 64x64 and K >= 1024: the workgroup's eight waves share the K loop
