@@ -1606,15 +1606,18 @@ int launch_async(ft_context* ctx, AsyncBatch g, int layout, int epi = kEpiPlain)
     bool pairs = false;
     g.tail_first = tiles;
     g.tail_shift = 0;
-    if (BM == 64 && epi == kEpiPlain && (size_t)tiles * 4 > (size_t)ctx->num_cus * 5 && !long_k) {
-        // More tiles than the few-tile rule below shares out, and a remainder over the CUs of at most a quarter
-        // of them: its tiles (the last of the order) must be plain ones (no RoPE epilogue, whole float4 groups).
+    if (BM == 64 && epi == kEpiPlain && tiles > ctx->num_cus && !long_k) {
+        // A remainder over the CUs of at most a quarter of them (288 tiles: the 576-column products of the 135M
+        // shape; 800: q/k/v at 360M): its tiles (the last of the order) must be plain ones (no RoPE epilogue,
+        // whole float4 groups).
         const int cus = ctx->num_cus, tail = tiles % cus;
         // at most 8 shares of at least 3 K tiles each (4 and 8 shares measured alike: 66-68 us against 73)
+        // (with eight waves per tile the K tiles are shared out in pairs)
+        const bool pairs_here = pairs_ok && (size_t)tiles <= 2 * (size_t)cus && min_kt >= 32;
+        const int kt_units = pairs_here ? min_kt / 2 : min_kt;
         int shift = 0;
-        while (shift < 3 && (tail << (shift + 1)) <= cus && (min_kt >> (shift + 1)) >= 3) shift++;
+        while (shift < 3 && (tail << (shift + 1)) <= cus && (kt_units >> (shift + 1)) >= 3) shift++;
         bool ok = tail > 0 && shift >= 2 && (size_t)(tail << shift) * BM * BN <= kSplitScratchFloats;
-        ok = ok && !(pairs_ok && (size_t)tiles <= 2 * (size_t)cus && min_kt >= 32);  // not with eight waves per tile
         auto tail_is_plain = [&]() {
             bool plain = true;
             for (int u = 0; u < tail && plain; u++) {
@@ -1655,7 +1658,8 @@ int launch_async(ft_context* ctx, AsyncBatch g, int layout, int epi = kEpiPlain)
         int want = (int)((2 * (size_t)ctx->num_cus + tiles - 1) / tiles);
         // A few tiles more than CUs (288 on 256: the 576-column products): with w shares a CU holds
         // ceil(288 w / 256) of them, 2, 3, 4 for w = 1, 2, 3, i.e. 2, 1.5, 1.33 tiles' worth; measured,
-        // three shares beat two (and four) in the 135M-shaped step.
+        // three shares beat two (and four) in the 135M-shaped step. (Only where the tail split above does not
+        // apply: it leaves a CU with one whole tile and an eighth, 15.3 -> 14.9 ms per 135M step.)
         if (BM == 64 && tiles > ctx->num_cus) want = 3;
         // 128x128 tiles hold two workgroups on a CU: the shares must fit one round of them
         if (BM == 128) want = (int)(2 * (size_t)ctx->num_cus / tiles);
