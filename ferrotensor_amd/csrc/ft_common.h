@@ -17,13 +17,22 @@
 // BufferPool (ferrotensor-backend/src/pool.rs), without its 512 MiB cap:
 // 288 GB of HBM leaves room to keep every step buffer resident.
 // The K shares of a split GEMM left unadded for the kernel that consumes the product (a norm kernel
-// that reads the row anyway): out = (add +) partial[0] + partial[1] + ... in that order, share s of
-// element i at partial[s * stride + i]. splits == 1: nothing was deferred, `out` is complete.
+// that reads the row anyway). Two forms:
+//  * every tile split (`splits > 1`): out = (add +) partial[0] + partial[1] + ... in that order, share s of
+//    element i at partial[s * stride + i]; `out` holds nothing yet.
+//  * tail split (`tail_shift > 0`): `out` is complete except for the 64 x 64 tiles at positions >= tail_first
+//    of the tile order (panels of `panel` n tiles, inside a panel row block after row block); tile
+//    tail_first + u is (add +) its 1 << tail_shift shares, share s at partial[((u << tail_shift) + s) * 4096],
+//    row-major inside the tile.
+// Neither: nothing was deferred, `out` is complete.
 struct ft_deferred_sum {
     const float* partial = nullptr;
     const float* add = nullptr;
     long stride = 0;
     int splits = 1;
+    const float* out = nullptr;
+    int tail_first = 0, tail_shift = 0, tiles_m = 0, tiles_n = 0, panel = 1;
+    bool pending() const { return splits > 1 || tail_shift > 0; }
 };
 
 struct ft_context {

@@ -645,13 +645,23 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(SplitReduceArgs a) {
     const long i = (long)blockIdx.x * 256 + threadIdx.x;
     if (i >= a.n4[pi]) return;
     const float4* src = reinterpret_cast<const float4*>(a.partial[pi]) + i;
+    const long n4 = a.n4[pi];
+    const int splits = a.splits;
     float4 v = a.add[pi] ? reinterpret_cast<const float4*>(a.add[pi])[i] : make_float4(0.f, 0.f, 0.f, 0.f);
-    for (int s = 0; s < a.splits; s++) {
-        const float4 t = src[(long)s * a.n4[pi]];
-        v.x += t.x;
-        v.y += t.y;
-        v.z += t.z;
-        v.w += t.w;
+    // four shares' loads in flight at a time (a share past the end re-reads the last one and is not added)
+    for (int s0 = 0; s0 < splits; s0 += 4) {
+        float4 t[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) t[u] = src[(long)(s0 + u < splits ? s0 + u : splits - 1) * n4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            if (s0 + u < splits) {
+                v.x += t[u].x;
+                v.y += t[u].y;
+                v.z += t[u].z;
+                v.w += t[u].w;
+            }
+        }
     }
     reinterpret_cast<float4*>(a.out[pi])[i] = v;
 }
@@ -1686,12 +1696,24 @@ int launch_async(ft_context* ctx, AsyncBatch g, int layout, int epi = kEpiPlain)
         }
     }
     const dim3 grid((unsigned)(g.tail_first + ((tiles - g.tail_first) << g.tail_shift)), (unsigned)g.splits);
-    // A deferred sum is honoured for one plain product whose shares are the plain [splits][M][N] arrays.
+    // A deferred sum is honoured for one plain product with a dense output: its shares are the plain
+    // [splits][M][N] arrays, or the partial tiles of a tail split.
     ft_deferred_sum* const defer = ctx->defer;
     ctx->defer = nullptr;
     if (defer) *defer = ft_deferred_sum{};
     auto reduce_shares = [&]() -> int {
         if (g.tail_shift > 0) {
+            if (defer && BM == 64 && g.count == 1 && epi == kEpiPlain && g.p[0].ldc == g.p[0].N) {
+                defer->partial = g.partial;
+                defer->add = g.p[0].add;
+                defer->out = g.p[0].out;
+                defer->tail_first = g.tail_first;
+                defer->tail_shift = g.tail_shift;
+                defer->tiles_m = g.tiles_m;
+                defer->tiles_n = g.tiles_n;
+                defer->panel = g.panel;
+                return FT_OK;
+            }
             hipLaunchKernelGGL(splitk_tail_reduce_kernel, dim3((unsigned)(tiles - g.tail_first)), dim3(1024), 0,
                                ctx->stream, g);
             FT_LAUNCH_CHECK();

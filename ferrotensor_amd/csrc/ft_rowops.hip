@@ -355,7 +355,71 @@ __device__ __forceinline__ void sum_shares_row(const ft_deferred_sum& d, size_t 
     }
 }
 
-template <int NV, bool SUM = false>
+// A lane's NV float4 of row `row` of a product whose last tiles are still K shares (tail split): elements
+// of whole tiles come from d.out; an element of tail tile u is (add +) share 0 + share 1 + ... in that
+// order (the order of the GEMM's own reduce kernel). is_tail[j] says which of the lane's float4 were
+// summed here. A wave whose row block holds no tail tile issues no extra load. No load sits under a
+// lane-dependent branch (the compiler waits for every earlier load in front of such a load: one round
+// trip per load instead of one per batch): lanes outside the tail tiles read share addresses of tile 0
+// and drop the values.
+template <int NV>
+__device__ __forceinline__ void sum_tail_row(const ft_deferred_sum& d, int row, int lane, int n4, float4 (&v)[NV],
+                                             bool (&is_tail)[NV]) {
+    constexpr int U = 4;
+    const size_t row_off = (size_t)row * 4 * n4;
+    const int tm = row >> 6;
+    const int shares = 1 << d.tail_shift;
+    const int last = (d.tiles_n - 1) / d.panel;
+    const float* src[NV];
+    bool any = false;
+#pragma unroll
+    for (int j = 0; j < NV; j++) {
+        const int i = lane + j * kWave;
+        const int ii = i < n4 ? i : 0;
+        const int tn = ii >> 4;  // 16 float4 per 64-column tile
+        const int pnl = tn / d.panel;
+        const int width = pnl == last ? d.tiles_n - last * d.panel : d.panel;
+        const int pos = pnl * d.tiles_m * d.panel + tm * width + (tn - pnl * d.panel);
+        is_tail[j] = i < n4 && pos >= d.tail_first;
+        any = any || is_tail[j];
+        src[j] = d.partial + ((size_t)(is_tail[j] ? pos - d.tail_first : 0) << d.tail_shift) * 4096 + (row & 63) * 64 +
+                 (ii & 15) * 4;
+        const float* base = (is_tail[j] && d.add) ? d.add : d.out;
+        const float4 t = reinterpret_cast<const float4*>(base + row_off)[ii];
+        const bool zero = i >= n4 || (is_tail[j] && !d.add);
+        v[j] = make_float4(zero ? 0.f : t.x, zero ? 0.f : t.y, zero ? 0.f : t.z, zero ? 0.f : t.w);
+    }
+    if (__ballot(any) == 0) return;  // wave-uniform
+    // Four shares' loads at a time, in straight-line code (a share past the end re-reads the last one and
+    // is not added); a tail tile has at most eight shares.
+    auto batch = [&](int s0) {
+        float4 t[U][NV];
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const int sc = s0 + u < shares ? s0 + u : shares - 1;
+#pragma unroll
+            for (int j = 0; j < NV; j++) t[u][j] = *reinterpret_cast<const float4*>(src[j] + (size_t)sc * 4096);
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+#pragma unroll
+            for (int j = 0; j < NV; j++) {
+                const bool take = is_tail[j] && s0 + u < shares;
+                v[j].x = take ? v[j].x + t[u][j].x : v[j].x;
+                v[j].y = take ? v[j].y + t[u][j].y : v[j].y;
+                v[j].z = take ? v[j].z + t[u][j].z : v[j].z;
+                v[j].w = take ? v[j].w + t[u][j].w : v[j].w;
+            }
+        }
+    };
+    batch(0);
+    if (shares > U) batch(U);
+}
+
+// SUM: 0 = x is complete; 1 = x is the K shares of the GEMM that produced it; 2 = x is complete except for
+// the tail tiles of that GEMM (ft_deferred_sum). In both deferred forms the summed elements are written to
+// x_out (which is the product's output buffer).
+template <int NV, int SUM = 0>
 __global__ __launch_bounds__(256) void rms_norm_wave_kernel(const float* __restrict__ x, const float* __restrict__ w,
                                                             float* __restrict__ out, int rows, int size, float eps,
                                                             ft_deferred_sum sum, float* __restrict__ x_out) {
@@ -364,33 +428,49 @@ __global__ __launch_bounds__(256) void rms_norm_wave_kernel(const float* __restr
     const int lane = threadIdx.x % kWave;
     const int n4 = size / 4;
     const float4* x4 = reinterpret_cast<const float4*>(x + (size_t)row * size);
-    float4 v[NV];
+    const float4* w4 = reinterpret_cast<const float4*>(w);
+    float4 v[NV], wv[NV];
     float ss = 0.0f;
-    if constexpr (SUM) {
+    bool is_tail[NV];
+    // Every load of the lane is issued before the first wait, none under a lane-dependent branch (a lane
+    // past the row's end re-reads element 0 and drops it): one memory round trip for the row.
+#pragma unroll
+    for (int j = 0; j < NV; j++) {
+        const int i = lane + j * kWave;
+        wv[j] = w4[i < n4 ? i : 0];
+    }
+    if constexpr (SUM == 1) {
         // x is still the K shares of the GEMM that produced it: added here (residual first, then share
         // after share) and written out once.
         sum_shares_row<NV>(sum, (size_t)row * size, lane, n4, v);
+    } else if constexpr (SUM == 2) {
+        sum_tail_row<NV>(sum, row, lane, n4, v, is_tail);
+    } else {
+#pragma unroll
+        for (int j = 0; j < NV; j++) {
+            const int i = lane + j * kWave;
+            v[j] = x4[i < n4 ? i : 0];
+        }
     }
 #pragma unroll
     for (int j = 0; j < NV; j++) {
         const int i = lane + j * kWave;
-        if constexpr (SUM) {
+        if constexpr (SUM == 1) {
             if (i < n4) reinterpret_cast<float4*>(x_out + (size_t)row * size)[i] = v[j];
-            else v[j] = make_float4(0.f, 0.f, 0.f, 0.f);
-        } else {
-            v[j] = i < n4 ? x4[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+        } else if constexpr (SUM == 2) {
+            if (is_tail[j]) reinterpret_cast<float4*>(x_out + (size_t)row * size)[i] = v[j];
         }
+        if (i >= n4) v[j] = make_float4(0.f, 0.f, 0.f, 0.f);
         ss += v[j].x * v[j].x + v[j].y * v[j].y + v[j].z * v[j].z + v[j].w * v[j].w;
     }
     ss = wave_sum(ss);
     const float inv = 1.0f / sqrtf(ss / (float)size + eps);
-    const float4* w4 = reinterpret_cast<const float4*>(w);
     float4* o4 = reinterpret_cast<float4*>(out + (size_t)row * size);
 #pragma unroll
     for (int j = 0; j < NV; j++) {
         const int i = lane + j * kWave;
         if (i < n4) {
-            const float4 g = w4[i];
+            const float4 g = wv[j];
             o4[i] = make_float4(v[j].x * inv * g.x, v[j].y * inv * g.y, v[j].z * inv * g.z, v[j].w * inv * g.w);
         }
     }
@@ -398,7 +478,8 @@ __global__ __launch_bounds__(256) void rms_norm_wave_kernel(const float* __restr
 
 // gx = g*w*inv - x*coef (+ add): the input gradient of RMSNorm, optionally
 // summed with the gradient arriving over the residual connection.
-template <int NV, bool SUM = false>
+// SUM as in rms_norm_wave_kernel, for g (nothing is written back: this kernel is g's only reader).
+template <int NV, int SUM = 0>
 __global__ __launch_bounds__(256) void rms_norm_backward_wave_kernel(
     const float* __restrict__ x, const float* __restrict__ w, const float* __restrict__ g, const float* add,
     float* gx, int rows, int size, float eps, ft_deferred_sum sum) {
@@ -409,19 +490,32 @@ __global__ __launch_bounds__(256) void rms_norm_backward_wave_kernel(
     const float4* x4 = reinterpret_cast<const float4*>(x + (size_t)row * size);
     const float4* g4 = reinterpret_cast<const float4*>(g + (size_t)row * size);
     const float4* w4 = reinterpret_cast<const float4*>(w);
-    float4 xv[NV], gv[NV];
+    // (without a residual gradient the slot re-reads x and the value is dropped)
+    const float4* a4 = add ? reinterpret_cast<const float4*>(add + (size_t)row * size) : x4;
+    float4 xv[NV], gv[NV], wv[NV], av[NV];
     float ss = 0.0f, gwx = 0.0f;
-    if constexpr (SUM) sum_shares_row<NV>(sum, (size_t)row * size, lane, n4, gv);  // g arrives as K shares
+    // Every load of the lane is issued before the first wait, none under a lane-dependent branch (a lane
+    // past the row's end re-reads element 0 and drops it): one memory round trip for x, w, g and the
+    // residual gradient together.
+#pragma unroll
+    for (int j = 0; j < NV; j++) {
+        const int i = lane + j * kWave;
+        const int ii = i < n4 ? i : 0;
+        xv[j] = x4[ii];
+        wv[j] = w4[ii];
+        av[j] = a4[ii];
+        if constexpr (SUM == 0) gv[j] = g4[ii];
+    }
+    if constexpr (SUM == 1) sum_shares_row<NV>(sum, (size_t)row * size, lane, n4, gv);  // g arrives as K shares
+    if constexpr (SUM == 2) {
+        bool is_tail[NV];
+        sum_tail_row<NV>(sum, row, lane, n4, gv, is_tail);
+    }
 #pragma unroll
     for (int j = 0; j < NV; j++) {
         const int i = lane + j * kWave;
         if (i < n4) {
-            xv[j] = x4[i];
-            float4 gg;
-            if constexpr (SUM) gg = gv[j];
-            else gg = g4[i];
-            const float4 ww = w4[i];
-            gv[j] = make_float4(gg.x * ww.x, gg.y * ww.y, gg.z * ww.z, gg.w * ww.w);  // g*w
+            gv[j] = make_float4(gv[j].x * wv[j].x, gv[j].y * wv[j].y, gv[j].z * wv[j].z, gv[j].w * wv[j].w);  // g*w
         } else {
             xv[j] = make_float4(0.f, 0.f, 0.f, 0.f);
             gv[j] = xv[j];
@@ -433,7 +527,6 @@ __global__ __launch_bounds__(256) void rms_norm_backward_wave_kernel(
     gwx = wave_sum(gwx);
     const float inv = 1.0f / sqrtf(ss / (float)size + eps);
     const float coef = gwx * inv * inv * inv / (float)size;
-    const float4* a4 = reinterpret_cast<const float4*>(add ? add + (size_t)row * size : nullptr);
     float4* o4 = reinterpret_cast<float4*>(gx + (size_t)row * size);
 #pragma unroll
     for (int j = 0; j < NV; j++) {
@@ -441,10 +534,7 @@ __global__ __launch_bounds__(256) void rms_norm_backward_wave_kernel(
         if (i < n4) {
             float4 r = make_float4(gv[j].x * inv - xv[j].x * coef, gv[j].y * inv - xv[j].y * coef,
                                    gv[j].z * inv - xv[j].z * coef, gv[j].w * inv - xv[j].w * coef);
-            if (add) {
-                const float4 a = a4[i];
-                r = make_float4(a.x + r.x, a.y + r.y, a.z + r.z, a.w + r.w);
-            }
+            if (add) r = make_float4(av[j].x + r.x, av[j].y + r.y, av[j].z + r.z, av[j].w + r.w);
             o4[i] = r;
         }
     }
@@ -953,22 +1043,37 @@ int ft_internal_rms_norm_backward_add(ft_context* ctx, const float* x, const flo
 // Can a norm kernel add the K shares of a [rows, size] product itself?
 bool ft_internal_norm_can_sum(size_t rows, size_t size) { return size % 4 == 0 && size <= 2048 && rows < (1u << 30); }
 
+// Do the tail tiles `d` describes belong to a dense [rows, size] product in 64 x 64 tiles?
+static bool tail_sum_fits(const ft_deferred_sum* d, size_t rows, size_t size) {
+    return d->out && aligned16(d->out) && d->panel >= 1 && d->tail_shift <= 3 &&
+           (size_t)d->tiles_m == ft_div_up(rows, 64) && (size_t)d->tiles_n == ft_div_up(size, 64) &&
+           d->tail_first >= 0 && d->tail_first < d->tiles_m * d->tiles_n;
+}
+
 // x_out = the deferred sum `d` ([rows, size]); out = rms_norm(x_out) * w. One pass: the shares are read
 // where the plain kernel reads x.
 int ft_internal_rms_norm_sum(ft_context* ctx, const ft_deferred_sum* d, float* x_out, const float* w, float* out,
                              size_t rows, size_t size, float eps) {
-    FT_CHECK_ARG(ctx && d && d->partial && d->splits > 1 && x_out && w && out, "rms_norm_sum: bad argument");
+    FT_CHECK_ARG(ctx && d && d->partial && d->pending() && x_out && w && out, "rms_norm_sum: bad argument");
     FT_CHECK_ARG(ft_internal_norm_can_sum(rows, size) && aligned16(d->partial) && aligned16(d->add) && d->stride % 4 == 0 &&
                      aligned16(x_out) && aligned16(w) && aligned16(out),
                  "rms_norm_sum: shape or alignment outside the fused kernel's");
+    const bool tail = d->tail_shift > 0;
+    if (tail) FT_CHECK_ARG(tail_sum_fits(d, rows, size) && d->out == x_out, "rms_norm_sum: tail tiles of another product");
     if (rows == 0) return FT_OK;
     ft_prof_scope prof(ctx, "rms_norm_kernel", 0.0, (12.0 + 4.0 * d->splits + (d->add ? 4.0 : 0.0)) * (double)rows * size);
     const dim3 grid(ft_div_up(rows, 4));
-    if (size <= 1024)
-        hipLaunchKernelGGL((rms_norm_wave_kernel<4, true>), grid, dim3(256), 0, ctx->stream, x_out, w, out, (int)rows,
+    if (tail && size <= 1024)
+        hipLaunchKernelGGL((rms_norm_wave_kernel<4, 2>), grid, dim3(256), 0, ctx->stream, x_out, w, out, (int)rows,
+                           (int)size, eps, *d, x_out);
+    else if (tail)
+        hipLaunchKernelGGL((rms_norm_wave_kernel<8, 2>), grid, dim3(256), 0, ctx->stream, x_out, w, out, (int)rows,
+                           (int)size, eps, *d, x_out);
+    else if (size <= 1024)
+        hipLaunchKernelGGL((rms_norm_wave_kernel<4, 1>), grid, dim3(256), 0, ctx->stream, x_out, w, out, (int)rows,
                            (int)size, eps, *d, x_out);
     else
-        hipLaunchKernelGGL((rms_norm_wave_kernel<8, true>), grid, dim3(256), 0, ctx->stream, x_out, w, out, (int)rows,
+        hipLaunchKernelGGL((rms_norm_wave_kernel<8, 1>), grid, dim3(256), 0, ctx->stream, x_out, w, out, (int)rows,
                            (int)size, eps, *d, x_out);
     FT_LAUNCH_CHECK();
     return FT_OK;
@@ -977,19 +1082,27 @@ int ft_internal_rms_norm_sum(ft_context* ctx, const ft_deferred_sum* d, float* x
 // gx = rms_norm_backward(x, w, g) (+ add) with g = the deferred sum `d`. No weight gradient.
 int ft_internal_rms_norm_backward_sum(ft_context* ctx, const float* x, const float* w, const ft_deferred_sum* d,
                                       const float* add, float* gx, size_t rows, size_t size, float eps) {
-    FT_CHECK_ARG(ctx && x && w && d && d->partial && d->splits > 1 && gx, "rms_norm_backward_sum: bad argument");
+    FT_CHECK_ARG(ctx && x && w && d && d->partial && d->pending() && gx, "rms_norm_backward_sum: bad argument");
     FT_CHECK_ARG(ft_internal_norm_can_sum(rows, size) && aligned16(d->partial) && aligned16(d->add) && d->stride % 4 == 0 &&
                      aligned16(x) && aligned16(w) && aligned16(gx) && aligned16(add),
                  "rms_norm_backward_sum: shape or alignment outside the fused kernel's");
+    const bool tail = d->tail_shift > 0;
+    if (tail) FT_CHECK_ARG(tail_sum_fits(d, rows, size), "rms_norm_backward_sum: tail tiles of another product");
     if (rows == 0) return FT_OK;
     ft_prof_scope prof(ctx, "rms_norm_backward_kernel", 0.0,
                        (8.0 + 4.0 * d->splits + (d->add ? 4.0 : 0.0) + (add ? 4.0 : 0.0)) * (double)rows * size);
     const dim3 grid(ft_div_up(rows, 4));
-    if (size <= 1024)
-        hipLaunchKernelGGL((rms_norm_backward_wave_kernel<4, true>), grid, dim3(256), 0, ctx->stream, x, w,
+    if (tail && size <= 1024)
+        hipLaunchKernelGGL((rms_norm_backward_wave_kernel<4, 2>), grid, dim3(256), 0, ctx->stream, x, w,
+                           (const float*)nullptr, add, gx, (int)rows, (int)size, eps, *d);
+    else if (tail)
+        hipLaunchKernelGGL((rms_norm_backward_wave_kernel<8, 2>), grid, dim3(256), 0, ctx->stream, x, w,
+                           (const float*)nullptr, add, gx, (int)rows, (int)size, eps, *d);
+    else if (size <= 1024)
+        hipLaunchKernelGGL((rms_norm_backward_wave_kernel<4, 1>), grid, dim3(256), 0, ctx->stream, x, w,
                            (const float*)nullptr, add, gx, (int)rows, (int)size, eps, *d);
     else
-        hipLaunchKernelGGL((rms_norm_backward_wave_kernel<8, true>), grid, dim3(256), 0, ctx->stream, x, w,
+        hipLaunchKernelGGL((rms_norm_backward_wave_kernel<8, 1>), grid, dim3(256), 0, ctx->stream, x, w,
                            (const float*)nullptr, add, gx, (int)rows, (int)size, eps, *d);
     FT_LAUNCH_CHECK();
     return FT_OK;

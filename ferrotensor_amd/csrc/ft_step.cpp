@@ -390,7 +390,7 @@ int linear_bias(ft_context* ctx, const LinearW& l, float* y, size_t T) {
 }
 
 // Offers the next GEMM launch on `ctx` the chance to leave its K shares unadded (the caller's next
-// kernel is a norm that adds them while it reads the row). `d->splits > 1` afterwards: it did.
+// kernel is a norm that adds them while it reads the row). `d->pending()` afterwards: it did.
 struct DeferScope {
     ft_context* ctx;
     DeferScope(ft_context* c, ft_deferred_sum* d, bool enable) : ctx(c) {
@@ -574,7 +574,7 @@ int layer_forward(ft_model* m, size_t l, size_t B, size_t S, bool defer_tail = f
         Layer& L = m->layers[l];
         LayerActs& a = m->acts[l];
         float* x_next = l + 1 < m->layers.size() ? m->acts[l + 1].x : m->x_final;
-        if (m->pending_x.splits > 1) {
+        if (m->pending_x.pending()) {
             FT_TRY(ft_internal_rms_norm_sum(ctx, &m->pending_x, a.x, L.norm1, a.h1, T, H, c.rms_norm_eps));
             m->pending_x = ft_deferred_sum{};
         } else {
@@ -611,7 +611,7 @@ int layer_forward(ft_model* m, size_t l, size_t B, size_t S, bool defer_tail = f
         {
             ft_deferred_sum d;
             FT_TRY(linear_forward(ctx, L.o, a.attn, a.to, a.h, T, a.x, can_sum ? &d : nullptr));
-            if (d.splits > 1)
+            if (d.pending())
                 FT_TRY(ft_internal_rms_norm_sum(ctx, &d, a.h, L.norm2, a.h2, T, H, c.rms_norm_eps));
             else
                 FT_TRY(ft_rms_norm_eps(ctx, a.h, L.norm2, a.h2, T, H, c.rms_norm_eps));
@@ -732,7 +732,7 @@ int norm_backward(ft_model* m, const float* x, const float* w, float* gw, const 
     ft_context* ctx = m->ctx;
     const size_t H = m->cfg.hidden_size;
     const float eps = m->cfg.rms_norm_eps;
-    if (g_sum && g_sum->splits > 1) {
+    if (g_sum && g_sum->pending()) {
         FT_CHECK_ARG(!gw, "norm_backward: a deferred gradient with a trainable norm scale");
         return ft_internal_rms_norm_backward_sum(ctx, x, w, g_sum, add, gx, rows, H, eps);
     }
