@@ -995,15 +995,17 @@ def test_head_dim_64_step_matches_oracle(ctx, checkpoint):
             assert_close(f"step {step} weight {n}", params[n], w, atol=1e-6, rtol=1e-4)
 
 
-def test_135m_width_step_matches_oracle(ctx):
+@pytest.mark.parametrize("checkpoint", [False, True])
+def test_135m_width_step_matches_oracle(ctx, checkpoint):
     """Hidden 576 at 8 x 256 tokens: every 576-column product has 288 output tiles, a few more than the GPU has
     CUs, so its last tiles are shared out along K and their shares are added by the norm kernel that reads the
     product next (forward: o and down projections; backward: both grouped input gradients) or by the reduce
-    kernel (o projection's input gradient). Logits, gradients and one optimizer step against the oracle."""
+    kernel (o projection's input gradient). Logits, gradients and one optimizer step against the oracle, also
+    with the blocks' forward recomputed in the backward pass."""
     from ferrotensor_amd.trainer import ModelConfig, Trainer
     cfg = ModelConfig(vocab_size=256, hidden_size=576, intermediate_size=1536, num_hidden_layers=2,
                       num_attention_heads=9, num_key_value_heads=3, rms_norm_eps=1e-5, rope_theta=100000.0,
-                      tie_word_embeddings=True, f16_linears=True)
+                      tie_word_embeddings=True, f16_linears=True, checkpoint_blocks=checkpoint)
     hip, orc = build_pair(ctx, cfg, ["q_proj", "k_proj", "v_proj", "o_proj"], rank=8, alpha=16.0, seed=77)
     rng = np.random.default_rng(8)
     B, S = 8, 256
